@@ -1,0 +1,315 @@
+"""ctypes binding of libdmoe.so (include/dmoe.h) for Python callers.
+
+PyTorch is used only as the owner of device memory and streams: every call passes
+raw device pointers (tensor.data_ptr()) and the current HIP stream to the C ABI.
+There is no fallback: if the library is missing or a call fails, an exception is raised.
+"""
+import ctypes as C
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libdmoe.so")
+
+QUANT_AFFINE, QUANT_MXFP4, QUANT_FP8_ROW = 0, 1, 2
+WEIGHTS_COPY_FROM_HOST, WEIGHTS_COPY_FROM_DEVICE, WEIGHTS_BORROW_DEVICE = 0, 1, 2
+
+
+class DmoeError(RuntimeError):
+    pass
+
+
+class _Handle(C.Structure):
+    _fields_ = [("ctx", C.c_void_p)]
+
+
+class QWeightC(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("scales", C.c_void_p), ("biases", C.c_void_p),
+                ("n_mats", C.c_int), ("rows", C.c_int), ("cols", C.c_int),
+                ("mode", C.c_int), ("bits", C.c_int), ("group_size", C.c_int)]
+
+
+class LayerDescC(C.Structure):
+    _fields_ = [("hidden", C.c_int), ("ffn", C.c_int), ("top_k", C.c_int),
+                ("gate", QWeightC), ("up", QWeightC), ("down", QWeightC),
+                ("swiglu_limit", C.c_float), ("score_before_down", C.c_int),
+                ("has_shared", C.c_int),
+                ("shared_gate", QWeightC), ("shared_up", QWeightC), ("shared_down", QWeightC),
+                ("shared_swiglu_limit", C.c_float),
+                ("remap", C.c_void_p), ("n_experts_total", C.c_int),
+                ("weight_source", C.c_int)]
+
+
+# every symbol include/dmoe.h declares
+EXPORTS = [
+    "dmoe_quant_mode_from_string", "dmoe_version", "dmoe_last_error", "dmoe_init",
+    "dmoe_stream_create", "dmoe_stream_destroy", "dmoe_stream_synchronize",
+    "dmoe_malloc", "dmoe_free", "dmoe_copy_to_device", "dmoe_copy_to_host",
+    "dmoe_workspace_create", "dmoe_workspace_destroy", "dmoe_workspace_reserved",
+    "dmoe_workspace_set_stage_timing", "dmoe_workspace_read_stage_times",
+    "dmoe_topk_route", "dmoe_gate_route", "dmoe_remap_indices", "dmoe_expand_tokens",
+    "dmoe_reduce_experts", "dmoe_smelt_build_mask", "dmoe_build_remap", "dmoe_preload_remap",
+    "dmoe_pack", "dmoe_dequantize", "dmoe_gather_qmm",
+    "dmoe_layer_create", "dmoe_layer_destroy", "dmoe_moe_forward",
+    "dmoe_switch_glu_forward_no_scores", "dmoe_moe_layer_forward", "dmoe_debug_last_activations",
+]
+
+_lib = None
+
+
+def lib():
+    """Load libdmoe.so (built by dmlx_amd/csrc/Makefile). Raises if it is not there."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise DmoeError(f"{LIB_PATH} not found: build it with `make -C dmlx_amd/csrc` "
+                            "(or __graft_entry__.build()); there is no fallback path")
+        _lib = C.CDLL(LIB_PATH)
+        _lib.dmoe_last_error.restype = C.c_char_p
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise DmoeError(f"dmoe error {rc}: {lib().dmoe_last_error().decode()}")
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    assert t.is_contiguous(), "dmoe takes dense row-major tensors"
+    return C.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return _Handle(C.c_void_p(torch.cuda.current_stream().cuda_stream))
+
+
+def init(device=0):
+    check(lib().dmoe_init(device))
+
+
+class Workspace:
+    def __init__(self, initial_bytes=0):
+        self.h = _Handle()
+        check(lib().dmoe_workspace_create(C.byref(self.h), C.c_size_t(initial_bytes)))
+
+    def reserved(self):
+        n = C.c_size_t()
+        check(lib().dmoe_workspace_reserved(C.byref(n), self.h))
+        return n.value
+
+    STAGES = ("route", "pack", "gate_up", "down", "shared", "combine")
+
+    def set_stage_timing(self, enabled):
+        check(lib().dmoe_workspace_set_stage_timing(self.h, int(enabled)))
+
+    def stage_times(self):
+        """{stage: (total_ms, samples)} of the forward calls made since timing was enabled"""
+        ms = (C.c_float * len(self.STAGES))()
+        n = (C.c_int * len(self.STAGES))()
+        check(lib().dmoe_workspace_read_stage_times(ms, n, self.h))
+        return {s: (ms[i], n[i]) for i, s in enumerate(self.STAGES)}
+
+    def close(self):
+        if self.h.ctx:
+            check(lib().dmoe_workspace_destroy(self.h))
+            self.h = _Handle()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class QWeight:
+    """A stack [n, rows, cols] of quantized matrices held as torch tensors (any device)."""
+
+    def __init__(self, w, scales, biases, rows, cols, mode, bits, group_size):
+        self.w, self.scales, self.biases = w.contiguous(), scales.contiguous(), biases
+        if self.biases is not None:
+            self.biases = self.biases.contiguous()
+        self.rows, self.cols, self.mode, self.bits, self.group_size = rows, cols, mode, bits, group_size
+        self.n_mats = w.shape[0] if w.dim() == 3 else 1
+
+    def to(self, device):
+        return QWeight(self.w.to(device), self.scales.to(device),
+                       None if self.biases is None else self.biases.to(device),
+                       self.rows, self.cols, self.mode, self.bits, self.group_size)
+
+    def c(self):
+        return QWeightC(_ptr(self.w), _ptr(self.scales), _ptr(self.biases), self.n_mats, self.rows,
+                        self.cols, self.mode, self.bits, self.group_size)
+
+    def nbytes(self):
+        n = self.w.numel() * self.w.element_size() + self.scales.numel() * self.scales.element_size()
+        if self.biases is not None:
+            n += self.biases.numel() * self.biases.element_size()
+        return n
+
+
+def topk_route(scores, K, normalize=True):
+    T, E = scores.shape
+    idx = torch.empty((T, K), dtype=torch.int32, device=scores.device)
+    w = torch.empty((T, K), dtype=torch.float32, device=scores.device)
+    check(lib().dmoe_topk_route(_ptr(idx), _ptr(w), _ptr(scores), T, E, K, int(normalize), _stream()))
+    return idx, w
+
+
+def gate_route(scores, bias, resident_mask, K, renorm, route_scale):
+    T, E = scores.shape
+    idx = torch.empty((T, K), dtype=torch.int32, device=scores.device)
+    w = torch.empty((T, K), dtype=torch.float32, device=scores.device)
+    check(lib().dmoe_gate_route(_ptr(idx), _ptr(w), _ptr(scores), _ptr(bias), _ptr(resident_mask),
+                                T, E, K, int(renorm), C.c_float(route_scale), _stream()))
+    return idx, w
+
+
+def remap_indices(remap, idx):
+    out = torch.empty_like(idx)
+    check(lib().dmoe_remap_indices(_ptr(out), _ptr(remap), _ptr(idx), C.c_size_t(idx.numel()),
+                                   remap.numel(), _stream()))
+    return out
+
+
+def expand_tokens(x, K):
+    T, D = x.shape
+    out = torch.empty((T * K, D), dtype=x.dtype, device=x.device)
+    check(lib().dmoe_expand_tokens(_ptr(out), _ptr(x), T, D, K, x.element_size(), _stream()))
+    return out
+
+
+def reduce_experts(expert_outs, weights):
+    T, K = weights.shape
+    D = expert_outs.shape[1]
+    out = torch.empty((T, D), dtype=torch.float32, device=weights.device)
+    check(lib().dmoe_reduce_experts(_ptr(out), _ptr(expert_outs), int(expert_outs.dtype == torch.bfloat16),
+                                    _ptr(weights), T, K, D, _stream()))
+    return out
+
+
+def smelt_build_mask(n_experts, load_fraction, strategy=0, enabled=True):
+    mask = (C.c_uint8 * n_experts)()
+    n = C.c_int()
+    check(lib().dmoe_smelt_build_mask(mask, C.byref(n), n_experts, C.c_float(load_fraction), strategy,
+                                      int(enabled)))
+    return list(mask), n.value
+
+
+def build_remap(mask):
+    n = len(mask)
+    m = (C.c_uint8 * n)(*mask)
+    out = (C.c_int32 * n)()
+    check(lib().dmoe_build_remap(out, m, n))
+    return list(out)
+
+
+def preload_remap(expert_ids, n_total):
+    ids = (C.c_uint32 * max(len(expert_ids), 1))(*expert_ids)
+    out = (C.c_int32 * n_total)()
+    cb = (C.c_float * n_total)()
+    check(lib().dmoe_preload_remap(out, cb, ids, len(expert_ids), n_total))
+    return list(out), list(cb)
+
+
+def pack(idx, E, ws):
+    T, K = idx.shape
+    n = T * K
+    dev = idx.device
+    i32 = dict(dtype=torch.int32, device=dev)
+    out = dict(order=torch.empty(n, **i32), inv=torch.empty(n, **i32), token=torch.empty(n, **i32),
+               sorted_e=torch.empty(n, **i32), counts=torch.empty(E, **i32),
+               offsets=torch.empty(E + 1, **i32), live=torch.full((E,), -1, **i32),
+               n_live=torch.empty(1, **i32))
+    check(lib().dmoe_pack(_ptr(out["order"]), _ptr(out["inv"]), _ptr(out["token"]), _ptr(out["sorted_e"]),
+                          _ptr(out["counts"]), _ptr(out["offsets"]), _ptr(out["live"]), _ptr(out["n_live"]),
+                          _ptr(idx), T, K, E, ws.h, _stream()))
+    return out
+
+
+def dequantize(qw, mat_index=0):
+    out = torch.empty((qw.rows, qw.cols), dtype=torch.bfloat16, device=qw.w.device)
+    c = qw.c()
+    check(lib().dmoe_dequantize(_ptr(out), C.byref(c), mat_index, _stream()))
+    return out
+
+
+def gather_qmm(x, qw, rhs_indices, ws, lhs_indices=None, sorted_indices=False):
+    R = rhs_indices.numel()
+    out = torch.empty((R, qw.rows), dtype=torch.bfloat16, device=x.device)
+    c = qw.c()
+    check(lib().dmoe_gather_qmm(_ptr(out), _ptr(x), C.byref(c), _ptr(lhs_indices), _ptr(rhs_indices), R,
+                                int(sorted_indices), ws.h, _stream()))
+    return out
+
+
+class Layer:
+    """Resident MoE layer (dmoe_layer). Weights are copied to (or borrowed from) device memory."""
+
+    def __init__(self, hidden, ffn, top_k, gate, up, down, swiglu_limit=0.0, score_before_down=False,
+                 shared=None, shared_swiglu_limit=0.0, remap=None, borrow=False):
+        d = LayerDescC()
+        d.hidden, d.ffn, d.top_k = hidden, ffn, top_k
+        d.gate, d.up, d.down = gate.c(), up.c(), down.c()
+        d.swiglu_limit = swiglu_limit
+        d.score_before_down = int(score_before_down)
+        d.has_shared = int(shared is not None)
+        if shared is not None:
+            d.shared_gate, d.shared_up, d.shared_down = shared[0].c(), shared[1].c(), shared[2].c()
+        d.shared_swiglu_limit = shared_swiglu_limit
+        self._remap_host = None
+        if remap is not None:
+            self._remap_host = (C.c_int32 * len(remap))(*[int(v) for v in remap])
+            d.remap = C.cast(self._remap_host, C.c_void_p)
+            d.n_experts_total = len(remap)
+        on_device = gate.w.is_cuda
+        d.weight_source = (WEIGHTS_BORROW_DEVICE if borrow else WEIGHTS_COPY_FROM_DEVICE) if on_device \
+            else WEIGHTS_COPY_FROM_HOST
+        self._keep = (gate, up, down, shared) if borrow else None
+        self.hidden, self.ffn, self.top_k = hidden, ffn, top_k
+        self.h = _Handle()
+        check(lib().dmoe_layer_create(C.byref(self.h), C.byref(d), _stream()))
+
+    def forward(self, x, indices, scores, ws):
+        T = x.shape[0]
+        out = torch.empty((T, self.hidden), dtype=torch.bfloat16, device=x.device)
+        check(lib().dmoe_moe_forward(_ptr(out), self.h, _ptr(x), _ptr(indices), _ptr(scores), T, ws.h,
+                                     _stream()))
+        return out
+
+    def forward_no_scores(self, x, slot_indices, ws):
+        T = x.shape[0]
+        out = torch.empty((T, self.top_k, self.hidden), dtype=torch.bfloat16, device=x.device)
+        check(lib().dmoe_switch_glu_forward_no_scores(_ptr(out), self.h, _ptr(x), _ptr(slot_indices), T,
+                                                      ws.h, _stream()))
+        return out
+
+    def layer_forward(self, x, scores, bias, resident_mask, renorm, route_scale, ws, want_routing=False):
+        T, E_total = scores.shape
+        out = torch.empty((T, self.hidden), dtype=torch.bfloat16, device=x.device)
+        idx = w = None
+        if want_routing:
+            idx = torch.empty((T, self.top_k), dtype=torch.int32, device=x.device)
+            w = torch.empty((T, self.top_k), dtype=torch.float32, device=x.device)
+        check(lib().dmoe_moe_layer_forward(_ptr(out), _ptr(idx), _ptr(w), self.h, _ptr(x), _ptr(scores),
+                                           _ptr(bias), _ptr(resident_mask), T, E_total, int(renorm),
+                                           C.c_float(route_scale), ws.h, _stream()))
+        return (out, idx, w) if want_routing else out
+
+    def last_activations(self, T, ws):
+        out = torch.empty((T * self.top_k, self.ffn), dtype=torch.bfloat16, device="cuda")
+        check(lib().dmoe_debug_last_activations(_ptr(out), self.h, T, ws.h, _stream()))
+        return out
+
+    def close(self):
+        if self.h.ctx:
+            check(lib().dmoe_layer_destroy(self.h))
+            self.h = _Handle()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -1,0 +1,191 @@
+// Shared host/device helpers of libdmoe (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "dmoe.h"
+
+namespace dmoe {
+
+// ---- errors (thread-local message, mlx-c style rc) ---------------------------------------------
+void set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+int hip_fail(hipError_t e, const char *what);
+
+#define DMOE_HIP(call)                                                   \
+    do {                                                                 \
+        hipError_t e__ = (call);                                         \
+        if (e__ != hipSuccess) return ::dmoe::hip_fail(e__, #call);      \
+    } while (0)
+
+#define DMOE_REQUIRE(cond, ...)                                          \
+    do {                                                                 \
+        if (!(cond)) {                                                   \
+            ::dmoe::set_error(__VA_ARGS__);                              \
+            return DMOE_ERR_INVALID;                                     \
+        }                                                                \
+    } while (0)
+
+#define DMOE_TRY(expr)                                                   \
+    do {                                                                 \
+        int rc__ = (expr);                                               \
+        if (rc__ != DMOE_OK) return rc__;                                \
+    } while (0)
+
+// checks the launch itself (bad configuration shows up here, not later)
+#define DMOE_LAUNCH_CHECK() DMOE_HIP(hipGetLastError())
+
+inline hipStream_t to_hip(dmoe_stream s) { return (hipStream_t)s.ctx; }
+
+// ---- workspace: one grow-only device allocation, carved with a bump allocator ---------------------
+struct StageTimer {
+    bool enabled = false;
+    hipEvent_t start[DMOE_STAGE_COUNT] = {}, stop[DMOE_STAGE_COUNT] = {};
+    bool pending[DMOE_STAGE_COUNT] = {};
+    float total_ms[DMOE_STAGE_COUNT] = {};
+    int samples[DMOE_STAGE_COUNT] = {};
+};
+
+struct Workspace {
+    void *base = nullptr;
+    size_t bytes = 0;
+    int device = 0;
+    StageTimer timer;
+};
+
+// stage timing helpers (no-ops unless enabled on the workspace)
+int stage_begin(Workspace *w, int stage, hipStream_t st);
+int stage_end(Workspace *w, int stage, hipStream_t st);
+int stage_flush(Workspace *w);
+
+// makes sure at least `bytes` are reserved (may synchronize the device and reallocate)
+int workspace_reserve(dmoe_workspace ws, size_t bytes, Workspace **out);
+
+struct Bump {
+    size_t off = 0;
+    size_t take(size_t bytes) {
+        size_t o = off;
+        off += (bytes + 255) & ~(size_t)255;
+        return o;
+    }
+};
+
+template <typename T>
+inline T *at(Workspace *w, size_t off) {
+    return (T *)((char *)w->base + off);
+}
+
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// ---- tile list produced by the pack kernels ----------------------------------------------------------
+// one entry per (expert segment, row tile): rows [row0, row0 + nrows) of the sorted row order
+struct Tile {
+    uint32_t expert;
+    uint32_t row0;
+    uint32_t nrows;
+    uint32_t pad;
+};
+
+struct PackOut {
+    uint32_t *order = nullptr, *inv = nullptr, *token = nullptr, *sorted_e = nullptr;
+    uint32_t *counts = nullptr, *offsets = nullptr, *live = nullptr, *n_live = nullptr;
+    Tile *tiles = nullptr;       // capacity pack_max_tiles(n, E, tile_m)
+    uint32_t *n_tiles = nullptr; // device scalar
+};
+
+inline int pack_max_tiles(size_t n, int E, int tile_m) {
+    size_t full = n / (size_t)tile_m;
+    size_t part = n < (size_t)E ? n : (size_t)E;
+    return (int)(full + part);
+}
+size_t pack_scratch_bytes(size_t n, int E);
+// stable counting sort of n = T*K expert ids (< E) + tile list with `tile_m` rows per tile (0 = none)
+int launch_pack(const PackOut &o, const uint32_t *d_idx, size_t n, int K, int E, int tile_m,
+                void *d_scratch, hipStream_t st);
+
+// ---- grouped quantized GEMM ----------------------------------------------------------------------------
+struct QView { // device view of one dmoe_qweight stack
+    const uint8_t *w = nullptr, *scales = nullptr, *biases = nullptr;
+    size_t w_mat = 0, s_mat = 0;   // bytes between consecutive matrices
+    size_t w_row = 0, s_row = 0;   // bytes between consecutive rows
+    int rows = 0, cols = 0, n_mats = 0;
+    int mode = 0, bits = 4, group = 64;
+};
+int make_qview(QView *out, const dmoe_qweight *q, const char *name);
+size_t qweight_w_bytes(const dmoe_qweight *q);
+size_t qweight_s_bytes(const dmoe_qweight *q);
+size_t qweight_b_bytes(const dmoe_qweight *q);
+
+struct GemmArgs {
+    QView b0, b1;                 // b1 = up projection when gate_up
+    bool gate_up = false;         // out[p, f] = swiglu(x.b0[f], x.b1[f]) instead of x.b0[n]
+    const uint16_t *a = nullptr;  // bf16 [*, cols]
+    const uint32_t *a_rows = nullptr;   // nullable: source row of sorted row p
+    uint16_t *out = nullptr;      // bf16 [*, ldo]
+    int ldo = 0;
+    const uint32_t *out_rows = nullptr; // nullable: destination row of sorted row p
+    const float *row_scale = nullptr;   // nullable: multiplier of sorted row p's output
+    const uint32_t *row_scale_idx = nullptr; // nullable: row_scale index of sorted row p (else p)
+    const Tile *tiles = nullptr;  // nullable: dense mode (one segment, expert 0, `dense_rows` rows)
+    const uint32_t *n_tiles = nullptr;
+    int max_tiles = 0;
+    int dense_rows = 0;
+    float swiglu_limit = 0.0f;
+};
+// tile_m the kernels were built for
+constexpr int kSmallTileM = 4;
+constexpr int kMfmaTileM = 128;
+int launch_qgemm_small(const GemmArgs &g, hipStream_t st);
+int launch_qgemm_mfma(const GemmArgs &g, hipStream_t st);
+bool qgemm_small_supports(const QView &b);
+bool qgemm_mfma_supports(const QView &b);
+
+} // namespace dmoe
+
+// ---- device helpers ------------------------------------------------------------------------------------
+#if defined(__HIPCC__)
+namespace dmoe {
+
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+// round to nearest even, one v_cvt_pk_bf16_f32 per pair
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    bf16x2_t v;
+    v.x = (__bf16)lo;
+    v.y = (__bf16)hi;
+    return __builtin_bit_cast(uint32_t, v);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    return (uint16_t)(pack_bf16x2(f, 0.0f) & 0xffffu);
+}
+__device__ __forceinline__ float round_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
+
+__device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & 63u); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+// limited SwiGLU on the bf16-rounded projections (deepseek_v4.zig:947-966); limit <= 0: plain SwiGLU
+__device__ __forceinline__ float limited_swiglu(float g, float u, float limit) {
+    g = round_bf16(g);
+    u = round_bf16(u);
+    if (limit > 0.0f) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+    }
+    float silu = g / (1.0f + __expf(-g));
+    return silu * u;
+}
+
+} // namespace dmoe
+#endif

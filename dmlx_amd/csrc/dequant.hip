@@ -1,0 +1,118 @@
+// dmoe_dequantize and the host-side description of quantized stacks.
+#include "common.h"
+#include "qformat.h"
+
+namespace dmoe {
+
+static size_t w_row_bytes(const dmoe_qweight *q) {
+    return q->mode == DMOE_QUANT_FP8_ROW ? (size_t)q->cols : (size_t)q->cols * (size_t)q->bits / 8;
+}
+static size_t s_row_bytes(const dmoe_qweight *q) {
+    if (q->mode == DMOE_QUANT_FP8_ROW) return 4;
+    if (q->mode == DMOE_QUANT_MXFP4) return (size_t)q->cols / 32;
+    return (size_t)(q->cols / q->group_size) * 2;
+}
+size_t qweight_w_bytes(const dmoe_qweight *q) { return w_row_bytes(q) * (size_t)q->rows * (size_t)q->n_mats; }
+size_t qweight_s_bytes(const dmoe_qweight *q) { return s_row_bytes(q) * (size_t)q->rows * (size_t)q->n_mats; }
+size_t qweight_b_bytes(const dmoe_qweight *q) {
+    return (q->mode == DMOE_QUANT_AFFINE && q->biases) ? qweight_s_bytes(q) : 0;
+}
+
+int make_qview(QView *v, const dmoe_qweight *q, const char *name) {
+    DMOE_REQUIRE(q != nullptr, "%s: descriptor is null", name);
+    DMOE_REQUIRE(q->w && q->scales, "%s: weight / scales pointer is null", name);
+    DMOE_REQUIRE(q->n_mats >= 1 && q->rows >= 1 && q->cols >= 1, "%s: bad shape [%d,%d,%d]", name, q->n_mats,
+                 q->rows, q->cols);
+    switch (q->mode) {
+    case DMOE_QUANT_AFFINE:
+        DMOE_REQUIRE(q->bits == 4 || q->bits == 8, "%s: affine bits must be 4 or 8 (got %d)", name, q->bits);
+        DMOE_REQUIRE(q->group_size == 32 || q->group_size == 64 || q->group_size == 128,
+                     "%s: affine group_size must be 32, 64 or 128 (got %d)", name, q->group_size);
+        DMOE_REQUIRE(q->cols % q->group_size == 0, "%s: cols %d not a multiple of group_size %d", name, q->cols,
+                     q->group_size);
+        break;
+    case DMOE_QUANT_MXFP4:
+        DMOE_REQUIRE(q->bits == 4 && q->group_size == 32, "%s: mxfp4 needs bits=4, group_size=32", name);
+        DMOE_REQUIRE(q->biases == nullptr, "%s: mxfp4 takes no biases", name);
+        DMOE_REQUIRE(q->cols % 32 == 0, "%s: cols %d not a multiple of 32", name, q->cols);
+        break;
+    case DMOE_QUANT_FP8_ROW:
+        DMOE_REQUIRE(q->bits == 8, "%s: fp8 needs bits=8", name);
+        DMOE_REQUIRE(q->biases == nullptr, "%s: fp8 takes no biases", name);
+        DMOE_REQUIRE(q->cols % 16 == 0, "%s: cols %d not a multiple of 16", name, q->cols);
+        break;
+    default:
+        set_error("%s: unknown quantization mode %d", name, q->mode);
+        return DMOE_ERR_INVALID;
+    }
+    DMOE_REQUIRE(((uintptr_t)q->w % 16) == 0 && (w_row_bytes(q) % 16) == 0,
+                 "%s: packed rows must be 16-byte aligned (row = %zu bytes)", name, w_row_bytes(q));
+    v->w = (const uint8_t *)q->w;
+    v->scales = (const uint8_t *)q->scales;
+    v->biases = (const uint8_t *)q->biases;
+    v->w_row = w_row_bytes(q);
+    v->s_row = s_row_bytes(q);
+    v->w_mat = v->w_row * (size_t)q->rows;
+    v->s_mat = v->s_row * (size_t)q->rows;
+    v->rows = q->rows;
+    v->cols = q->cols;
+    v->n_mats = q->n_mats;
+    v->mode = q->mode;
+    v->bits = q->bits;
+    v->group = q->mode == DMOE_QUANT_AFFINE ? q->group_size : 32;
+    return DMOE_OK;
+}
+
+// one thread per 16-byte chunk of a row
+template <typename Fmt>
+__global__ void dequant_kernel(uint16_t *__restrict__ out, QView q, int mat) {
+    const int chunks_per_row = q.cols / Fmt::kVals;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)q.rows * chunks_per_row) return;
+    int row = (int)(i / chunks_per_row), c = (int)(i - (size_t)row * chunks_per_row);
+    int k0 = c * Fmt::kVals;
+    const uint8_t *wrow = q.w + (size_t)mat * q.w_mat + (size_t)row * q.w_row;
+    const uint8_t *srow = q.scales + (size_t)mat * q.s_mat + (size_t)row * q.s_row;
+    const uint8_t *brow = q.biases ? q.biases + (size_t)mat * q.s_mat + (size_t)row * q.s_row : nullptr;
+    uint4 raw = *(const uint4 *)(wrow + (size_t)c * 16);
+    Meta m = Fmt::load_meta(q, srow, brow, k0);
+    uint32_t pairs[Fmt::kVals / 2];
+    Fmt::decode(raw, m, pairs);
+    if (Fmt::kRowScale) {
+        float rs = *(const float *)srow;
+#pragma unroll
+        for (int p = 0; p < Fmt::kVals / 2; ++p)
+            pairs[p] = pack_bf16x2(bf16_bits_to_f32(pairs[p] & 0xffffu) * rs, bf16_bits_to_f32(pairs[p] >> 16) * rs);
+    }
+    uint32_t *o = (uint32_t *)(out + (size_t)row * q.cols + k0);
+#pragma unroll
+    for (int p = 0; p < Fmt::kVals / 2; ++p) o[p] = pairs[p];
+}
+
+struct DequantLaunch {
+    uint16_t *out;
+    QView q;
+    int mat;
+    hipStream_t st;
+    template <typename Fmt>
+    int operator()() {
+        size_t total = (size_t)q.rows * (q.cols / Fmt::kVals);
+        hipLaunchKernelGGL(dequant_kernel<Fmt>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, out, q, mat);
+        DMOE_LAUNCH_CHECK();
+        return DMOE_OK;
+    }
+};
+
+} // namespace dmoe
+
+using namespace dmoe;
+
+extern "C" int dmoe_dequantize(uint16_t *d_out, const dmoe_qweight *qw, int mat_index, dmoe_stream s) {
+    QView q;
+    DMOE_TRY(make_qview(&q, qw, "dequantize"));
+    DMOE_REQUIRE(d_out != nullptr, "dequantize: out is null");
+    DMOE_REQUIRE(mat_index >= 0 && mat_index < q.n_mats, "dequantize: mat_index %d out of [0,%d)", mat_index,
+                 q.n_mats);
+    DMOE_REQUIRE(q.cols % 32 == 0, "dequantize: cols %d not a multiple of 32", q.cols);
+    return dispatch_format(q, DequantLaunch{d_out, q, mat_index, to_hip(s)});
+}

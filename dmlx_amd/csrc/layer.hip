@@ -1,0 +1,472 @@
+// Resident MoE layer: weights held in HBM, and the forward pass
+//   remap -> pack -> grouped gate/up + limited SwiGLU -> grouped down -> weighted sum over k (+ shared).
+// Also dmoe_gather_qmm, the leaf operator, built from the same pack + grouped-GEMM kernels.
+#include <string.h>
+
+#include <new>
+
+#include "common.h"
+
+namespace dmoe {
+
+struct QOwned {
+    dmoe_qweight q;        // device pointers
+    void *own[3] = {nullptr, nullptr, nullptr};
+    QView view;
+};
+
+struct Layer {
+    int D = 0, F = 0, K = 0, E = 0, Fs = 0;
+    QOwned gate, up, down, sgate, sup, sdown;
+    bool has_shared = false;
+    float swiglu_limit = 0.0f, shared_swiglu_limit = 0.0f;
+    bool score_before_down = false;
+    int32_t *remap = nullptr; // device
+    int n_total = 0;
+    int device = 0;
+};
+
+static void free_owned(QOwned &o) {
+    for (void *&p : o.own) {
+        if (p) (void)hipFree(p);
+        p = nullptr;
+    }
+}
+
+static void free_layer(Layer *L) {
+    free_owned(L->gate);
+    free_owned(L->up);
+    free_owned(L->down);
+    free_owned(L->sgate);
+    free_owned(L->sup);
+    free_owned(L->sdown);
+    if (L->remap) (void)hipFree(L->remap);
+    delete L;
+}
+
+static int adopt(QOwned *dst, const dmoe_qweight *src, int source, const char *name, hipStream_t st) {
+    dst->q = *src;
+    if (source != DMOE_WEIGHTS_BORROW_DEVICE) {
+        DMOE_REQUIRE(src->w && src->scales, "%s: weight / scales pointer is null", name);
+        // validate the shape before sizing any copy
+        QView probe;
+        dmoe_qweight tmp = *src;
+        // make_qview checks pointer alignment; host pointers need not be aligned, device copies will be
+        tmp.w = (const void *)(uintptr_t)16;
+        DMOE_TRY(make_qview(&probe, &tmp, name));
+        const void *in[3] = {src->w, src->scales, src->biases};
+        size_t bytes[3] = {qweight_w_bytes(src), qweight_s_bytes(src), qweight_b_bytes(src)};
+        hipMemcpyKind kind = source == DMOE_WEIGHTS_COPY_FROM_HOST ? hipMemcpyHostToDevice : hipMemcpyDeviceToDevice;
+        for (int i = 0; i < 3; ++i) {
+            if (!in[i] || !bytes[i]) continue;
+            DMOE_HIP(hipMalloc(&dst->own[i], bytes[i]));
+            DMOE_HIP(hipMemcpyAsync(dst->own[i], in[i], bytes[i], kind, st));
+        }
+        dst->q.w = dst->own[0];
+        dst->q.scales = dst->own[1];
+        dst->q.biases = dst->own[2];
+    }
+    return make_qview(&dst->view, &dst->q, name);
+}
+
+// ---- small kernels ----------------------------------------------------------------------------------
+
+__global__ void compose_rows_kernel(uint32_t *__restrict__ out, const uint32_t *__restrict__ lhs,
+                                    const uint32_t *__restrict__ order, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = lhs[order[i]];
+}
+
+// out[dst[p], :] = in[p, :], 16 bytes per thread
+__global__ void scatter_rows_kernel(uint4 *__restrict__ out, const uint4 *__restrict__ in,
+                                    const uint32_t *__restrict__ dst, size_t row_vecs, size_t total) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    size_t p = i / row_vecs, c = i - p * row_vecs;
+    out[(size_t)dst[p] * row_vecs + c] = in[i];
+}
+
+// out[t, :] = sum_k (w ? w[t,k] : 1) * y[t*K+k, :] + (shared ? shared[t, :] : 0); 8 columns per thread
+__global__ void combine_kernel(uint16_t *__restrict__ out, const uint16_t *__restrict__ y,
+                               const float *__restrict__ w, const uint16_t *__restrict__ shared, int T, int K,
+                               int D) {
+    const size_t vec_per_row = (size_t)D / 8;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)T * vec_per_row) return;
+    size_t t = i / vec_per_row, c = i - t * vec_per_row;
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
+    for (int k = 0; k < K; ++k) {
+        size_t r = t * (size_t)K + k;
+        float wk = w ? w[r] : 1.0f;
+        uint4 q = *(const uint4 *)(y + r * (size_t)D + c * 8);
+        uint32_t u[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            acc[2 * j] += bf16_bits_to_f32(u[j] & 0xffffu) * wk;
+            acc[2 * j + 1] += bf16_bits_to_f32(u[j] >> 16) * wk;
+        }
+    }
+    if (shared) {
+        uint4 q = *(const uint4 *)(shared + t * (size_t)D + c * 8);
+        uint32_t u[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            acc[2 * j] += bf16_bits_to_f32(u[j] & 0xffffu);
+            acc[2 * j + 1] += bf16_bits_to_f32(u[j] >> 16);
+        }
+    }
+    uint4 o = make_uint4(pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3]), pack_bf16x2(acc[4], acc[5]),
+                         pack_bf16x2(acc[6], acc[7]));
+    *(uint4 *)(out + t * (size_t)D + c * 8) = o;
+}
+
+// ---- forward -------------------------------------------------------------------------------------------
+
+// average rows per expert at or below this run on the small-M path
+constexpr int kSmallAvgRows = 4;
+
+static bool use_small_path(size_t rows, int n_experts, const QView &b) {
+    return qgemm_small_supports(b) && rows <= (size_t)kSmallAvgRows * (size_t)n_experts;
+}
+
+struct FwdLayout {
+    size_t slot_idx, order, inv, token, sorted_e, counts, offsets, live, n_live, tiles, n_tiles, scratch;
+    size_t h, y, sh_h, sh_y, total;
+    int max_tiles, tile_m;
+    bool small;
+};
+
+static FwdLayout forward_layout(const Layer *L, int T) {
+    FwdLayout f;
+    Bump b;
+    size_t n = (size_t)T * L->K;
+    f.small = use_small_path(n, L->E, L->gate.view) && qgemm_small_supports(L->down.view);
+    f.tile_m = f.small ? kSmallTileM : kMfmaTileM;
+    f.max_tiles = pack_max_tiles(n, L->E, f.tile_m);
+    f.slot_idx = b.take(n * 4);
+    f.order = b.take(n * 4);
+    f.inv = b.take(n * 4);
+    f.token = b.take(n * 4);
+    f.sorted_e = b.take(n * 4);
+    f.counts = b.take((size_t)L->E * 4);
+    f.offsets = b.take((size_t)(L->E + 1) * 4);
+    f.live = b.take((size_t)L->E * 4);
+    f.n_live = b.take(4);
+    f.tiles = b.take((size_t)(f.max_tiles > 0 ? f.max_tiles : 1) * sizeof(Tile));
+    f.n_tiles = b.take(4);
+    f.scratch = b.take(pack_scratch_bytes(n, L->E));
+    f.h = b.take(n * (size_t)L->F * 2);
+    f.y = b.take(n * (size_t)L->D * 2);
+    f.sh_h = b.take(L->has_shared ? (size_t)T * L->Fs * 2 : 0);
+    f.sh_y = b.take(L->has_shared ? (size_t)T * L->D * 2 : 0);
+    f.total = b.off;
+    return f;
+}
+
+static int run_gemm(const GemmArgs &g, bool small, hipStream_t st) {
+    return small ? launch_qgemm_small(g, st) : launch_qgemm_mfma(g, st);
+}
+
+// routed experts on slot ids: fills ws->y ([T*K, D] bf16 in flat (t,k) order) or `y_out` when given
+static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, const uint16_t *d_x,
+                          const uint32_t *d_slots, const float *d_scores, int T, uint16_t *y_out, hipStream_t st) {
+    size_t n = (size_t)T * L->K;
+    PackOut po;
+    po.order = at<uint32_t>(w, f.order);
+    po.inv = at<uint32_t>(w, f.inv);
+    po.token = at<uint32_t>(w, f.token);
+    po.sorted_e = at<uint32_t>(w, f.sorted_e);
+    po.counts = at<uint32_t>(w, f.counts);
+    po.offsets = at<uint32_t>(w, f.offsets);
+    po.live = at<uint32_t>(w, f.live);
+    po.n_live = at<uint32_t>(w, f.n_live);
+    po.tiles = at<Tile>(w, f.tiles);
+    po.n_tiles = at<uint32_t>(w, f.n_tiles);
+    DMOE_TRY(launch_pack(po, d_slots, n, L->K, L->E, f.tile_m, at<void>(w, f.scratch), st));
+    DMOE_TRY(stage_end(w, DMOE_STAGE_PACK, st));
+
+    GemmArgs gu;
+    gu.b0 = L->gate.view;
+    gu.b1 = L->up.view;
+    gu.gate_up = true;
+    gu.a = d_x;
+    gu.a_rows = po.token;
+    gu.out = at<uint16_t>(w, f.h);
+    gu.ldo = L->F;
+    gu.tiles = po.tiles;
+    gu.n_tiles = po.n_tiles;
+    gu.max_tiles = f.max_tiles;
+    gu.swiglu_limit = L->swiglu_limit;
+    if (L->score_before_down && d_scores) {
+        gu.row_scale = d_scores;
+        gu.row_scale_idx = po.order;
+    }
+    DMOE_TRY(stage_begin(w, DMOE_STAGE_GATE_UP, st));
+    DMOE_TRY(run_gemm(gu, f.small, st));
+    DMOE_TRY(stage_end(w, DMOE_STAGE_GATE_UP, st));
+
+    GemmArgs dn;
+    dn.b0 = L->down.view;
+    dn.a = at<uint16_t>(w, f.h);
+    dn.out = y_out ? y_out : at<uint16_t>(w, f.y);
+    dn.ldo = L->D;
+    dn.out_rows = po.order; // unsort while storing (deepseek_v4.zig:809)
+    dn.tiles = po.tiles;
+    dn.n_tiles = po.n_tiles;
+    dn.max_tiles = f.max_tiles;
+    DMOE_TRY(stage_begin(w, DMOE_STAGE_DOWN, st));
+    DMOE_TRY(run_gemm(dn, f.small, st));
+    DMOE_TRY(stage_end(w, DMOE_STAGE_DOWN, st));
+    return DMOE_OK;
+}
+
+static int shared_forward(const Layer *L, Workspace *w, const FwdLayout &f, const uint16_t *d_x, int T,
+                          hipStream_t st) {
+    const bool small = T <= kSmallTileM && qgemm_small_supports(L->sgate.view) && qgemm_small_supports(L->sdown.view);
+    const int tile_m = small ? kSmallTileM : kMfmaTileM;
+    GemmArgs gu;
+    gu.b0 = L->sgate.view;
+    gu.b1 = L->sup.view;
+    gu.gate_up = true;
+    gu.a = d_x;
+    gu.out = at<uint16_t>(w, f.sh_h);
+    gu.ldo = L->Fs;
+    gu.dense_rows = T;
+    gu.max_tiles = ceil_div(T, tile_m);
+    gu.swiglu_limit = L->shared_swiglu_limit;
+    DMOE_TRY(run_gemm(gu, small, st));
+    GemmArgs dn;
+    dn.b0 = L->sdown.view;
+    dn.a = at<uint16_t>(w, f.sh_h);
+    dn.out = at<uint16_t>(w, f.sh_y);
+    dn.ldo = L->D;
+    dn.dense_rows = T;
+    dn.max_tiles = ceil_div(T, tile_m);
+    DMOE_TRY(run_gemm(dn, small, st));
+    return DMOE_OK;
+}
+
+} // namespace dmoe
+
+using namespace dmoe;
+
+extern "C" {
+
+int dmoe_layer_create(dmoe_layer *out, const dmoe_layer_desc *d, dmoe_stream s) {
+    DMOE_REQUIRE(out && d, "layer_create: null argument");
+    out->ctx = nullptr;
+    DMOE_REQUIRE(d->hidden > 0 && d->ffn > 0 && d->top_k > 0, "layer_create: bad dims D=%d F=%d K=%d", d->hidden,
+                 d->ffn, d->top_k);
+    DMOE_REQUIRE(d->weight_source >= 0 && d->weight_source <= 2, "layer_create: bad weight_source %d",
+                 d->weight_source);
+    DMOE_REQUIRE(d->hidden % 8 == 0 && d->ffn % 8 == 0, "layer_create: D and F must be multiples of 8");
+    DMOE_REQUIRE(d->gate.rows == d->ffn && d->gate.cols == d->hidden && d->up.rows == d->ffn &&
+                     d->up.cols == d->hidden && d->down.rows == d->hidden && d->down.cols == d->ffn,
+                 "layer_create: projection shapes do not match D=%d F=%d", d->hidden, d->ffn);
+    DMOE_REQUIRE(d->gate.n_mats == d->up.n_mats && d->gate.n_mats == d->down.n_mats && d->gate.n_mats >= 1 &&
+                     d->gate.n_mats <= 1024,
+                 "layer_create: expert counts differ or are out of range");
+    Layer *L = new (std::nothrow) Layer();
+    DMOE_REQUIRE(L != nullptr, "layer_create: out of host memory");
+    hipStream_t st = to_hip(s);
+    int rc = DMOE_OK;
+    do {
+        if (hipGetDevice(&L->device) != hipSuccess) { rc = hip_fail(hipGetLastError(), "hipGetDevice"); break; }
+        L->D = d->hidden;
+        L->F = d->ffn;
+        L->K = d->top_k;
+        L->E = d->gate.n_mats;
+        L->swiglu_limit = d->swiglu_limit;
+        L->score_before_down = d->score_before_down != 0;
+        if ((rc = adopt(&L->gate, &d->gate, d->weight_source, "gate_proj", st))) break;
+        if ((rc = adopt(&L->up, &d->up, d->weight_source, "up_proj", st))) break;
+        if ((rc = adopt(&L->down, &d->down, d->weight_source, "down_proj", st))) break;
+        if (d->has_shared) {
+            L->has_shared = true;
+            L->Fs = d->shared_gate.rows;
+            L->shared_swiglu_limit = d->shared_swiglu_limit;
+            if (d->shared_gate.n_mats != 1 || d->shared_up.n_mats != 1 || d->shared_down.n_mats != 1 ||
+                d->shared_gate.cols != L->D || d->shared_up.cols != L->D || d->shared_up.rows != L->Fs ||
+                d->shared_down.rows != L->D || d->shared_down.cols != L->Fs || L->Fs % 8 != 0) {
+                set_error("layer_create: shared expert shapes do not match D=%d", L->D);
+                rc = DMOE_ERR_INVALID;
+                break;
+            }
+            if ((rc = adopt(&L->sgate, &d->shared_gate, d->weight_source, "shared gate_proj", st))) break;
+            if ((rc = adopt(&L->sup, &d->shared_up, d->weight_source, "shared up_proj", st))) break;
+            if ((rc = adopt(&L->sdown, &d->shared_down, d->weight_source, "shared down_proj", st))) break;
+        }
+        if (d->remap) {
+            if (d->n_experts_total < 1) { set_error("layer_create: n_experts_total must be >= 1 with a remap"); rc = DMOE_ERR_INVALID; break; }
+            for (int i = 0; i < d->n_experts_total; ++i)
+                if (d->remap[i] < 0 || d->remap[i] >= L->E) {
+                    set_error("layer_create: remap[%d] = %d is not a slot in [0,%d)", i, d->remap[i], L->E);
+                    rc = DMOE_ERR_INVALID;
+                    break;
+                }
+            if (rc) break;
+            L->n_total = d->n_experts_total;
+            hipError_t e = hipMalloc((void **)&L->remap, sizeof(int32_t) * (size_t)L->n_total);
+            if (e == hipSuccess)
+                e = hipMemcpyAsync(L->remap, d->remap, sizeof(int32_t) * (size_t)L->n_total, hipMemcpyHostToDevice, st);
+            if (e != hipSuccess) { rc = hip_fail(e, "remap upload"); break; }
+        }
+        // host sources may be pageable and may be released by the caller right after this call
+        hipError_t e = hipStreamSynchronize(st);
+        if (e != hipSuccess) { rc = hip_fail(e, "hipStreamSynchronize"); break; }
+    } while (0);
+    if (rc != DMOE_OK) {
+        free_layer(L);
+        return rc;
+    }
+    out->ctx = L;
+    return DMOE_OK;
+}
+
+int dmoe_layer_destroy(dmoe_layer layer) {
+    if (layer.ctx) free_layer((Layer *)layer.ctx);
+    return DMOE_OK;
+}
+
+static int forward_common(uint16_t *d_out, uint16_t *y_out, Layer *L, const uint16_t *d_x, const uint32_t *d_indices,
+                          const float *d_scores, int T, bool apply_remap, bool with_shared, dmoe_workspace ws,
+                          dmoe_stream s) {
+    DMOE_REQUIRE(T >= 0, "forward: T=%d", T);
+    if (T == 0) return DMOE_OK;
+    DMOE_REQUIRE(d_x && d_indices, "forward: null pointer");
+    DMOE_REQUIRE(((uintptr_t)d_x % 16) == 0, "forward: x must be 16-byte aligned");
+    DMOE_REQUIRE(y_out || (d_out && ((uintptr_t)d_out % 16) == 0), "forward: out must be 16-byte aligned and non-null");
+    hipStream_t st = to_hip(s);
+    FwdLayout f = forward_layout(L, T);
+    Workspace *w = nullptr;
+    DMOE_TRY(workspace_reserve(ws, f.total, &w));
+    const uint32_t *slots = d_indices;
+    size_t n = (size_t)T * L->K;
+    DMOE_TRY(stage_begin(w, DMOE_STAGE_PACK, st));
+    if (apply_remap && L->remap) {
+        uint32_t *sl = at<uint32_t>(w, f.slot_idx);
+        DMOE_TRY(dmoe_remap_indices(sl, L->remap, d_indices, n, L->n_total, s));
+        slots = sl;
+    }
+    DMOE_TRY(routed_forward(L, w, f, d_x, slots, d_scores, T, y_out, st));
+    if (y_out) return DMOE_OK;
+    const bool shared = with_shared && L->has_shared;
+    if (shared) {
+        DMOE_TRY(stage_begin(w, DMOE_STAGE_SHARED, st));
+        DMOE_TRY(shared_forward(L, w, f, d_x, T, st));
+        DMOE_TRY(stage_end(w, DMOE_STAGE_SHARED, st));
+    }
+    DMOE_TRY(stage_begin(w, DMOE_STAGE_COMBINE, st));
+    size_t total = (size_t)T * (L->D / 8);
+    hipLaunchKernelGGL(combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, d_out,
+                       at<uint16_t>(w, f.y), L->score_before_down ? nullptr : d_scores,
+                       shared ? at<uint16_t>(w, f.sh_y) : nullptr, T, L->K, L->D);
+    DMOE_LAUNCH_CHECK();
+    DMOE_TRY(stage_end(w, DMOE_STAGE_COMBINE, st));
+    return DMOE_OK;
+}
+
+int dmoe_moe_forward(uint16_t *d_out, dmoe_layer layer, const uint16_t *d_x, const uint32_t *d_indices,
+                     const float *d_scores, int T, dmoe_workspace ws, dmoe_stream s) {
+    DMOE_REQUIRE(layer.ctx, "moe_forward: layer handle is null");
+    DMOE_REQUIRE(d_scores || T == 0, "moe_forward: scores pointer is null");
+    return forward_common(d_out, nullptr, (Layer *)layer.ctx, d_x, d_indices, d_scores, T, true, true, ws, s);
+}
+
+int dmoe_switch_glu_forward_no_scores(uint16_t *d_out, dmoe_layer layer, const uint16_t *d_x,
+                                      const uint32_t *d_slot_indices, int T, dmoe_workspace ws, dmoe_stream s) {
+    DMOE_REQUIRE(layer.ctx, "switch_glu_forward_no_scores: layer handle is null");
+    DMOE_REQUIRE(d_out || T == 0, "switch_glu_forward_no_scores: out is null");
+    DMOE_REQUIRE(((uintptr_t)d_out % 8) == 0, "switch_glu_forward_no_scores: out must be 8-byte aligned");
+    return forward_common(nullptr, d_out, (Layer *)layer.ctx, d_x, d_slot_indices, nullptr, T, false, false, ws, s);
+}
+
+int dmoe_moe_layer_forward(uint16_t *d_out, uint32_t *d_out_indices, float *d_out_weights, dmoe_layer layer,
+                           const uint16_t *d_x, const float *d_scores, const float *d_bias,
+                           const uint8_t *d_resident_mask, int T, int E_total, int renorm, float route_scale,
+                           dmoe_workspace ws, dmoe_stream s) {
+    DMOE_REQUIRE(layer.ctx, "moe_layer_forward: layer handle is null");
+    Layer *L = (Layer *)layer.ctx;
+    DMOE_REQUIRE(T >= 0, "moe_layer_forward: T=%d", T);
+    if (T == 0) return DMOE_OK;
+    if (L->remap) DMOE_REQUIRE(E_total == L->n_total, "moe_layer_forward: E_total %d != remap length %d", E_total, L->n_total);
+    else DMOE_REQUIRE(E_total == L->E, "moe_layer_forward: E_total %d != resident experts %d", E_total, L->E);
+    // routing outputs live in caller memory when given, else in a private tail of the workspace
+    FwdLayout f = forward_layout(L, T);
+    size_t n = (size_t)T * L->K;
+    Bump b;
+    b.off = f.total;
+    size_t o_idx = b.take(n * 4), o_w = b.take(n * 4);
+    Workspace *w = nullptr;
+    DMOE_TRY(workspace_reserve(ws, b.off, &w));
+    uint32_t *idx = d_out_indices ? d_out_indices : at<uint32_t>(w, o_idx);
+    float *wts = d_out_weights ? d_out_weights : at<float>(w, o_w);
+    DMOE_TRY(stage_begin(w, DMOE_STAGE_ROUTE, to_hip(s)));
+    DMOE_TRY(dmoe_gate_route(idx, wts, d_scores, d_bias, d_resident_mask, T, E_total, L->K, renorm, route_scale, s));
+    DMOE_TRY(stage_end(w, DMOE_STAGE_ROUTE, to_hip(s)));
+    return forward_common(d_out, nullptr, L, d_x, idx, wts, T, true, true, ws, s);
+}
+
+int dmoe_debug_last_activations(uint16_t *d_out, dmoe_layer layer, int T, dmoe_workspace ws, dmoe_stream s) {
+    DMOE_REQUIRE(layer.ctx && ws.ctx && d_out, "debug_last_activations: null argument");
+    Layer *L = (Layer *)layer.ctx;
+    Workspace *w = (Workspace *)ws.ctx;
+    FwdLayout f = forward_layout(L, T);
+    DMOE_REQUIRE(w->bytes >= f.total, "debug_last_activations: no forward of this size has run on the workspace");
+    size_t n = (size_t)T * L->K, rv = (size_t)L->F / 8, total = n * rv;
+    if (total == 0) return DMOE_OK;
+    hipLaunchKernelGGL(scatter_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, to_hip(s),
+                       (uint4 *)d_out, (const uint4 *)at<uint16_t>(w, f.h), at<uint32_t>(w, f.order), rv, total);
+    DMOE_LAUNCH_CHECK();
+    return DMOE_OK;
+}
+
+int dmoe_gather_qmm(uint16_t *d_out, const uint16_t *d_x, const dmoe_qweight *qw, const uint32_t *d_lhs_indices,
+                    const uint32_t *d_rhs_indices, int R, int sorted, dmoe_workspace ws, dmoe_stream s) {
+    (void)sorted; // the counting sort below is a no-op on already grouped rows
+    QView v;
+    DMOE_TRY(make_qview(&v, qw, "gather_qmm"));
+    DMOE_REQUIRE(R >= 0, "gather_qmm: R=%d", R);
+    if (R == 0) return DMOE_OK;
+    DMOE_REQUIRE(d_out && d_x && d_rhs_indices, "gather_qmm: null pointer");
+    DMOE_REQUIRE(v.n_mats <= 1024, "gather_qmm: more than 1024 matrices in the stack");
+    hipStream_t st = to_hip(s);
+    const bool small = use_small_path((size_t)R, v.n_mats, v);
+    DMOE_REQUIRE(small || qgemm_mfma_supports(v), "gather_qmm: unsupported weight shape rows=%d cols=%d", v.rows, v.cols);
+    const int tile_m = small ? kSmallTileM : kMfmaTileM;
+    const int max_tiles = pack_max_tiles((size_t)R, v.n_mats, tile_m);
+    Bump b;
+    size_t o_order = b.take((size_t)R * 4), o_arows = b.take((size_t)R * 4);
+    size_t o_tiles = b.take((size_t)max_tiles * sizeof(Tile)), o_nt = b.take(4);
+    size_t o_scr = b.take(pack_scratch_bytes((size_t)R, v.n_mats));
+    Workspace *w = nullptr;
+    DMOE_TRY(workspace_reserve(ws, b.off, &w));
+    PackOut po;
+    po.order = at<uint32_t>(w, o_order);
+    po.tiles = at<Tile>(w, o_tiles);
+    po.n_tiles = at<uint32_t>(w, o_nt);
+    DMOE_TRY(launch_pack(po, d_rhs_indices, (size_t)R, 1, v.n_mats, tile_m, at<void>(w, o_scr), st));
+    const uint32_t *a_rows = po.order;
+    if (d_lhs_indices) {
+        uint32_t *ar = at<uint32_t>(w, o_arows);
+        hipLaunchKernelGGL(compose_rows_kernel, dim3((unsigned)((R + 255) / 256)), dim3(256), 0, st, ar,
+                           d_lhs_indices, po.order, (size_t)R);
+        DMOE_LAUNCH_CHECK();
+        a_rows = ar;
+    }
+    GemmArgs g;
+    g.b0 = v;
+    g.a = d_x;
+    g.a_rows = a_rows;
+    g.out = d_out;
+    g.ldo = v.rows;
+    g.out_rows = po.order;
+    g.tiles = po.tiles;
+    g.n_tiles = po.n_tiles;
+    g.max_tiles = max_tiles;
+    return run_gemm(g, small, st);
+}
+
+} // extern "C"

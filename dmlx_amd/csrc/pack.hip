@@ -1,0 +1,266 @@
+// Token -> expert packing: a stable counting sort of the T*K routed expert ids.
+//
+// Each wavefront owns a contiguous sub-chunk of the flat (t*K+k) index space. Phase 1 builds one LDS
+// histogram per sub-chunk; phase 2 turns the [sub-chunk][expert] counts into starting offsets (exclusive
+// scan over sub-chunks inside each expert, then over experts) and emits counts / segment offsets / the
+// tile list / the list of live experts; phase 3 re-reads the ids and places every row at
+// base[sub-chunk][expert] + (number of earlier lanes with the same expert), found with ballots, so rows
+// of one expert keep ascending flat index. No global atomics; the result is deterministic.
+//
+// Up to 1024 rows everything runs in ONE launch (16 wavefronts x 64 rows); above that in three.
+#include "common.h"
+
+namespace dmoe {
+
+constexpr int kPackThreads = 1024;              // scan / fused kernels: one expert per thread
+constexpr int kPackWaves = kPackThreads / 64;   // 16
+constexpr int kSubGroups = 4;                   // multi-launch path: groups of 64 rows per wavefront
+constexpr int kSubRows = 64 * kSubGroups;       // 256 rows per sub-chunk
+constexpr int kScatterWaves = 4;                // wavefronts per block in the multi-launch path
+
+// exclusive scan of one value per thread across a 1024-thread block; *total gets the block sum
+__device__ uint32_t block_excl_scan(uint32_t v, uint32_t *total, uint32_t *sm /*[kPackWaves + 1]*/) {
+    const int lane = lane_id(), wave = (int)(threadIdx.x >> 6);
+    uint32_t incl = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        uint32_t o = (uint32_t)__shfl_up((int)incl, off, 64);
+        if (lane >= off) incl += o;
+    }
+    __syncthreads(); // sm may still be read from a previous call
+    if (lane == 63) sm[wave] = incl;
+    __syncthreads();
+    if (wave == 0) {
+        uint32_t t = lane < kPackWaves ? sm[lane] : 0u, ti = t;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            uint32_t o = (uint32_t)__shfl_up((int)ti, off, 64);
+            if (lane >= off) ti += o;
+        }
+        if (lane < kPackWaves) sm[lane] = ti - t;
+        if (lane == 63) sm[kPackWaves] = ti;
+    }
+    __syncthreads();
+    *total = sm[kPackWaves];
+    return sm[wave] + incl - v;
+}
+
+// lanes of this wavefront that hold the same expert id (only among `active` lanes)
+__device__ __forceinline__ uint64_t match_expert(uint32_t e, bool active, int nbits) {
+    uint64_t peers = __ballot(active);
+    for (int b = 0; b < nbits; ++b) {
+        bool bit = (e >> b) & 1u;
+        uint64_t bal = __ballot(active && bit);
+        peers &= bit ? bal : ~bal;
+    }
+    return peers;
+}
+
+__device__ __forceinline__ int log2_ceil(int E) {
+    int b = 0;
+    while ((1 << b) < E) ++b;
+    return b;
+}
+
+// phase 2 body shared by the fused and the stand-alone scan kernel. `count` is this thread's expert total.
+__device__ uint32_t emit_segments(uint32_t count, int e, int E, size_t n, int tile_m, const PackOut &o,
+                                  uint32_t *sm) {
+    uint32_t total;
+    uint32_t off = block_excl_scan(count, &total, sm);
+    if (e < E) {
+        if (o.counts) o.counts[e] = count;
+        if (o.offsets) o.offsets[e] = off;
+    }
+    if (e == 0 && o.offsets) o.offsets[E] = (uint32_t)n;
+    if (o.live || o.n_live) {
+        uint32_t lt;
+        uint32_t lb = block_excl_scan(count > 0 ? 1u : 0u, &lt, sm);
+        if (count > 0 && o.live) o.live[lb] = (uint32_t)e;
+        if (e == 0 && o.n_live) *o.n_live = lt;
+    }
+    if (tile_m > 0 && o.tiles) {
+        uint32_t nt = (count + (uint32_t)tile_m - 1) / (uint32_t)tile_m, tt;
+        uint32_t tb = block_excl_scan(nt, &tt, sm);
+        for (uint32_t j = 0; j < nt; ++j) {
+            Tile t;
+            t.expert = (uint32_t)e;
+            t.row0 = off + j * (uint32_t)tile_m;
+            uint32_t left = count - j * (uint32_t)tile_m;
+            t.nrows = left < (uint32_t)tile_m ? left : (uint32_t)tile_m;
+            t.pad = 0;
+            o.tiles[tb + j] = t;
+        }
+        if (e == 0 && o.n_tiles) *o.n_tiles = tt;
+    }
+    return off;
+}
+
+__device__ __forceinline__ void place_row(const PackOut &o, uint32_t pos, uint32_t i, uint32_t e, int K) {
+    o.order[pos] = i;
+    if (o.inv) o.inv[i] = pos;
+    if (o.token) o.token[pos] = i / (uint32_t)K;
+    if (o.sorted_e) o.sorted_e[pos] = e;
+}
+
+// ---- one launch, n <= 1024 ---------------------------------------------------------------------------------
+__global__ __launch_bounds__(kPackThreads) void pack_fused_kernel(PackOut o, const uint32_t *__restrict__ idx,
+                                                                  uint32_t n, int K, int E, int tile_m) {
+    extern __shared__ uint32_t pack_sm[]; // hist[kPackWaves][E]
+    __shared__ uint32_t scan_sm[kPackWaves + 1];
+    const int tid = (int)threadIdx.x, lane = lane_id(), wave = tid >> 6;
+    for (int i = tid; i < kPackWaves * E; i += kPackThreads) pack_sm[i] = 0;
+    __syncthreads();
+    const uint32_t i = (uint32_t)tid;
+    const bool active = i < n;
+    uint32_t e = active ? idx[i] : 0u;
+    if (active && e >= (uint32_t)E) e = (uint32_t)E - 1; // ids are validated by the caller's contract; stay in bounds
+    if (active) atomicAdd(&pack_sm[wave * E + e], 1u);
+    __syncthreads();
+    uint32_t count = 0;
+    if (tid < E) {
+        for (int w = 0; w < kPackWaves; ++w) {
+            uint32_t c = pack_sm[w * E + tid];
+            pack_sm[w * E + tid] = count;
+            count += c;
+        }
+    }
+    uint32_t off = emit_segments(count, tid, E, n, tile_m, o, scan_sm);
+    if (tid < E)
+        for (int w = 0; w < kPackWaves; ++w) pack_sm[w * E + tid] += off;
+    __syncthreads();
+    uint64_t peers = match_expert(e, active, log2_ceil(E));
+    if (active) {
+        uint32_t rank = (uint32_t)__popcll(peers & ((1ull << lane) - 1ull));
+        place_row(o, pack_sm[wave * E + e] + rank, i, e, K);
+    }
+}
+
+// ---- three launches, any n --------------------------------------------------------------------------------
+__global__ __launch_bounds__(kScatterWaves * 64) void pack_hist_kernel(uint32_t *__restrict__ cnt,
+                                                                       const uint32_t *__restrict__ idx,
+                                                                       size_t n, int E, int n_sub) {
+    extern __shared__ uint32_t pack_sm[]; // hist[kScatterWaves][E]
+    const int tid = (int)threadIdx.x, lane = lane_id(), wave = tid >> 6;
+    for (int i = tid; i < kScatterWaves * E; i += kScatterWaves * 64) pack_sm[i] = 0;
+    __syncthreads();
+    const int sub = (int)blockIdx.x * kScatterWaves + wave;
+    if (sub < n_sub) {
+        for (int g = 0; g < kSubGroups; ++g) {
+            size_t i = (size_t)sub * kSubRows + (size_t)g * 64 + lane;
+            if (i < n) {
+                uint32_t e = idx[i];
+                if (e >= (uint32_t)E) e = (uint32_t)E - 1;
+                atomicAdd(&pack_sm[wave * E + e], 1u);
+            }
+        }
+    }
+    __syncthreads();
+    if (sub < n_sub)
+        for (int e = lane; e < E; e += 64) cnt[(size_t)sub * E + e] = pack_sm[wave * E + e];
+}
+
+__global__ __launch_bounds__(kPackThreads) void pack_scan_kernel(PackOut o, uint32_t *__restrict__ cnt,
+                                                                 size_t n, int E, int n_sub, int tile_m) {
+    __shared__ uint32_t scan_sm[kPackWaves + 1];
+    const int tid = (int)threadIdx.x;
+    uint32_t count = 0;
+    if (tid < E) {
+        for (int sidx = 0; sidx < n_sub; ++sidx) {
+            uint32_t c = cnt[(size_t)sidx * E + tid];
+            cnt[(size_t)sidx * E + tid] = count;
+            count += c;
+        }
+    }
+    uint32_t off = emit_segments(count, tid, E, n, tile_m, o, scan_sm);
+    // the scatter kernel needs the segment starts even if the caller did not ask for offsets
+    if (tid < E) cnt[(size_t)n_sub * E + tid] = off;
+}
+
+__global__ __launch_bounds__(kScatterWaves * 64) void pack_scatter_kernel(PackOut o,
+                                                                          const uint32_t *__restrict__ cnt,
+                                                                          const uint32_t *__restrict__ idx,
+                                                                          size_t n, int K, int E, int n_sub) {
+    extern __shared__ uint32_t pack_sm[]; // run[kScatterWaves][E]
+    const int tid = (int)threadIdx.x, lane = lane_id(), wave = tid >> 6;
+    const int sub = (int)blockIdx.x * kScatterWaves + wave;
+    const bool wave_on = sub < n_sub;
+    if (wave_on)
+        for (int e = lane; e < E; e += 64)
+            pack_sm[wave * E + e] = cnt[(size_t)sub * E + e] + cnt[(size_t)n_sub * E + e];
+    __syncthreads();
+    const int nbits = log2_ceil(E);
+    for (int g = 0; g < kSubGroups; ++g) {
+        size_t i = (size_t)sub * kSubRows + (size_t)g * 64 + lane;
+        const bool active = wave_on && i < n;
+        uint32_t e = active ? idx[i] : 0u;
+        if (active && e >= (uint32_t)E) e = (uint32_t)E - 1;
+        uint64_t peers = match_expert(e, active, nbits);
+        uint32_t base = 0, rank = 0;
+        if (active) {
+            base = pack_sm[wave * E + e];
+            rank = (uint32_t)__popcll(peers & ((1ull << lane) - 1ull));
+            place_row(o, base + rank, (uint32_t)i, e, K);
+        }
+        __syncthreads(); // every lane has read its base before any counter moves
+        if (active && (peers >> lane) <= 1ull) // highest lane of its peer group
+            pack_sm[wave * E + e] = base + rank + 1u;
+        __syncthreads();
+    }
+}
+
+size_t pack_scratch_bytes(size_t n, int E) {
+    size_t n_sub = (n + kSubRows - 1) / kSubRows;
+    return (n_sub + 1) * (size_t)E * sizeof(uint32_t);
+}
+
+int launch_pack(const PackOut &o, const uint32_t *d_idx, size_t n, int K, int E, int tile_m, void *d_scratch,
+                hipStream_t st) {
+    DMOE_REQUIRE(E >= 1 && E <= kPackThreads, "pack: E=%d out of range [1,%d]", E, kPackThreads);
+    DMOE_REQUIRE(K >= 1, "pack: K=%d", K);
+    DMOE_REQUIRE(n < (1ull << 31), "pack: too many rows");
+    DMOE_REQUIRE(o.order != nullptr && (d_idx != nullptr || n == 0), "pack: null pointer");
+    if (n <= (size_t)kPackThreads) {
+        // also covers n == 0: counts/offsets/n_tiles/n_live are still written (all zero)
+        size_t lds = sizeof(uint32_t) * (size_t)kPackWaves * E;
+        hipLaunchKernelGGL(pack_fused_kernel, dim3(1), dim3(kPackThreads), lds, st, o, d_idx, (uint32_t)n, K, E,
+                           tile_m);
+        DMOE_LAUNCH_CHECK();
+        return DMOE_OK;
+    }
+    DMOE_REQUIRE(d_scratch != nullptr, "pack: scratch is null");
+    uint32_t *cnt = (uint32_t *)d_scratch;
+    int n_sub = (int)((n + kSubRows - 1) / kSubRows);
+    dim3 grid((unsigned)ceil_div(n_sub, kScatterWaves)), block(kScatterWaves * 64);
+    size_t lds = sizeof(uint32_t) * (size_t)kScatterWaves * E;
+    hipLaunchKernelGGL(pack_hist_kernel, grid, block, lds, st, cnt, d_idx, n, E, n_sub);
+    DMOE_LAUNCH_CHECK();
+    hipLaunchKernelGGL(pack_scan_kernel, dim3(1), dim3(kPackThreads), 0, st, o, cnt, n, E, n_sub, tile_m);
+    DMOE_LAUNCH_CHECK();
+    hipLaunchKernelGGL(pack_scatter_kernel, grid, block, lds, st, o, cnt, d_idx, n, K, E, n_sub);
+    DMOE_LAUNCH_CHECK();
+    return DMOE_OK;
+}
+
+} // namespace dmoe
+
+using namespace dmoe;
+
+extern "C" int dmoe_pack(uint32_t *d_out_order, uint32_t *d_out_inv_order, uint32_t *d_out_token,
+                         uint32_t *d_out_sorted_expert, uint32_t *d_out_counts, uint32_t *d_out_offsets,
+                         uint32_t *d_out_live_experts, uint32_t *d_out_n_live, const uint32_t *d_indices, int T,
+                         int K, int E, dmoe_workspace ws, dmoe_stream s) {
+    DMOE_REQUIRE(T >= 0 && K >= 1, "pack: bad shape T=%d K=%d", T, K);
+    size_t n = (size_t)T * K;
+    Workspace *w = nullptr;
+    DMOE_TRY(workspace_reserve(ws, pack_scratch_bytes(n, E > 0 ? E : 1), &w));
+    PackOut o;
+    o.order = d_out_order;
+    o.inv = d_out_inv_order;
+    o.token = d_out_token;
+    o.sorted_e = d_out_sorted_expert;
+    o.counts = d_out_counts;
+    o.offsets = d_out_offsets;
+    o.live = d_out_live_experts;
+    o.n_live = d_out_n_live;
+    return launch_pack(o, d_indices, n, K, E, 0, w->base, to_hip(s));
+}

@@ -1,0 +1,152 @@
+// Device-side decoding of the quantized weight formats (MLX affine 4/8-bit, MXFP4, FP8-E4M3 per-row).
+//
+// Every format is read in 16-byte pieces ("chunks"): kVals values of one weight row that share one
+// scale (and bias). Value i of a chunk is element (k0 + i) of the row, so pairs (2p, 2p+1) are adjacent
+// along the reduction dimension.
+#pragma once
+
+#include "common.h"
+
+#if defined(__HIPCC__)
+namespace dmoe {
+
+// ---- scalar decoders (exact; used by dmoe_dequantize and as the definition of each format) -----------
+
+// E8M0 shared exponent -> 2^(s-127); 255 is NaN
+__device__ __forceinline__ float e8m0_to_f32(uint32_t s) {
+    if (s == 255u) return __uint_as_float(0x7fc00000u);
+    if (s == 0u) return __uint_as_float(0x00400000u); // 2^-127, an f32 subnormal
+    return __uint_as_float(s << 23);
+}
+
+// E2M1 code (sign in bit 3) -> f32: 0, .5, 1, 1.5, 2, 3, 4, 6
+__device__ __forceinline__ float e2m1_to_f32(uint32_t q) {
+    uint32_t m = q & 7u;
+    uint32_t bits = m >= 2u ? 0x3f800000u + ((m - 2u) << 22) : (m ? 0x3f000000u : 0u);
+    return __uint_as_float(bits | ((q & 8u) << 28));
+}
+
+// OCP E4M3FN byte -> f32
+__device__ __forceinline__ float e4m3_to_f32(uint32_t v) {
+    uint32_t e = (v >> 3) & 15u, m = v & 7u, sign = (v & 0x80u) << 24;
+    uint32_t bits;
+    if (e == 15u && m == 7u) bits = 0x7fc00000u;
+    else if (e == 0u) return __uint_as_float(__float_as_uint((float)m * 0.001953125f) | sign); // m * 2^-9
+    else bits = ((e + 120u) << 23) | (m << 20);
+    return __uint_as_float(bits | sign);
+}
+
+// ---- per-chunk decoders -------------------------------------------------------------------------------
+// Fmt::kVals                         values per 16-byte chunk
+// Fmt::load_meta(b, row_s, row_b, k0) scale/bias of the chunk starting at column k0 (f32 pair)
+// Fmt::decode(raw, meta, out)        kVals/2 packed bf16 pairs, natural order, fully dequantized
+// Fmt::kRowScale                     true: an f32 per-row scale is applied to the finished dot product
+
+struct Meta {
+    float s, b;
+};
+
+struct FmtAffine4 {
+    static constexpr int kVals = 32;
+    static constexpr bool kRowScale = false;
+    __device__ static __forceinline__ Meta load_meta(const QView &q, const uint8_t *row_s, const uint8_t *row_b,
+                                                     int k0) {
+        int g = k0 / q.group;
+        Meta m;
+        m.s = bf16_bits_to_f32(((const uint16_t *)row_s)[g]);
+        m.b = row_b ? bf16_bits_to_f32(((const uint16_t *)row_b)[g]) : 0.0f;
+        return m;
+    }
+    __device__ static __forceinline__ void decode_word(uint32_t w, Meta m, uint32_t *out /*[4]*/) {
+        uint32_t lo = w & 0x0f0f0f0fu, hi = (w >> 4) & 0x0f0f0f0fu; // nibbles 0,2,4,6 / 1,3,5,7 as bytes
+        out[0] = pack_bf16x2(fmaf((float)(lo & 0xffu), m.s, m.b), fmaf((float)(hi & 0xffu), m.s, m.b));
+        out[1] = pack_bf16x2(fmaf((float)((lo >> 8) & 0xffu), m.s, m.b), fmaf((float)((hi >> 8) & 0xffu), m.s, m.b));
+        out[2] = pack_bf16x2(fmaf((float)((lo >> 16) & 0xffu), m.s, m.b), fmaf((float)((hi >> 16) & 0xffu), m.s, m.b));
+        out[3] = pack_bf16x2(fmaf((float)(lo >> 24), m.s, m.b), fmaf((float)(hi >> 24), m.s, m.b));
+    }
+    __device__ static __forceinline__ void decode(const uint4 &raw, Meta m, uint32_t *out /*[16]*/) {
+        decode_word(raw.x, m, out);
+        decode_word(raw.y, m, out + 4);
+        decode_word(raw.z, m, out + 8);
+        decode_word(raw.w, m, out + 12);
+    }
+};
+
+struct FmtAffine8 {
+    static constexpr int kVals = 16;
+    static constexpr bool kRowScale = false;
+    __device__ static __forceinline__ Meta load_meta(const QView &q, const uint8_t *row_s, const uint8_t *row_b,
+                                                     int k0) {
+        return FmtAffine4::load_meta(q, row_s, row_b, k0);
+    }
+    __device__ static __forceinline__ void decode_word(uint32_t w, Meta m, uint32_t *out /*[2]*/) {
+        out[0] = pack_bf16x2(fmaf((float)(w & 0xffu), m.s, m.b), fmaf((float)((w >> 8) & 0xffu), m.s, m.b));
+        out[1] = pack_bf16x2(fmaf((float)((w >> 16) & 0xffu), m.s, m.b), fmaf((float)(w >> 24), m.s, m.b));
+    }
+    __device__ static __forceinline__ void decode(const uint4 &raw, Meta m, uint32_t *out /*[8]*/) {
+        decode_word(raw.x, m, out);
+        decode_word(raw.y, m, out + 2);
+        decode_word(raw.z, m, out + 4);
+        decode_word(raw.w, m, out + 6);
+    }
+};
+
+struct FmtMxfp4 {
+    static constexpr int kVals = 32;
+    static constexpr bool kRowScale = false;
+    __device__ static __forceinline__ Meta load_meta(const QView &, const uint8_t *row_s, const uint8_t *, int k0) {
+        Meta m;
+        m.s = e8m0_to_f32(row_s[k0 >> 5]);
+        m.b = 0.0f;
+        return m;
+    }
+    __device__ static __forceinline__ void decode_word(uint32_t w, Meta m, uint32_t *out /*[4]*/) {
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            float a = e2m1_to_f32((w >> (8 * p)) & 15u) * m.s;
+            float b = e2m1_to_f32((w >> (8 * p + 4)) & 15u) * m.s;
+            out[p] = pack_bf16x2(a, b); // exact: 2 significant bits times a power of two
+        }
+    }
+    __device__ static __forceinline__ void decode(const uint4 &raw, Meta m, uint32_t *out /*[16]*/) {
+        decode_word(raw.x, m, out);
+        decode_word(raw.y, m, out + 4);
+        decode_word(raw.z, m, out + 8);
+        decode_word(raw.w, m, out + 12);
+    }
+};
+
+struct FmtFp8Row {
+    static constexpr int kVals = 16;
+    static constexpr bool kRowScale = true; // scales: one f32 per row, applied after the reduction
+    __device__ static __forceinline__ Meta load_meta(const QView &, const uint8_t *, const uint8_t *, int) {
+        Meta m;
+        m.s = 1.0f;
+        m.b = 0.0f;
+        return m;
+    }
+    __device__ static __forceinline__ void decode_word(uint32_t w, Meta, uint32_t *out /*[2]*/) {
+        out[0] = pack_bf16x2(e4m3_to_f32(w & 0xffu), e4m3_to_f32((w >> 8) & 0xffu)); // exact in bf16
+        out[1] = pack_bf16x2(e4m3_to_f32((w >> 16) & 0xffu), e4m3_to_f32(w >> 24));
+    }
+    __device__ static __forceinline__ void decode(const uint4 &raw, Meta m, uint32_t *out /*[8]*/) {
+        decode_word(raw.x, m, out);
+        decode_word(raw.y, m, out + 2);
+        decode_word(raw.z, m, out + 4);
+        decode_word(raw.w, m, out + 6);
+    }
+};
+
+// dispatch a callable templated on the format: f.template operator()<Fmt>()
+template <typename F>
+inline int dispatch_format(const QView &q, F &&f) {
+    if (q.mode == DMOE_QUANT_AFFINE && q.bits == 4) return f.template operator()<FmtAffine4>();
+    if (q.mode == DMOE_QUANT_AFFINE && q.bits == 8) return f.template operator()<FmtAffine8>();
+    if (q.mode == DMOE_QUANT_MXFP4) return f.template operator()<FmtMxfp4>();
+    if (q.mode == DMOE_QUANT_FP8_ROW) return f.template operator()<FmtFp8Row>();
+    set_error("unsupported quantization mode %d / bits %d", q.mode, q.bits);
+    return DMOE_ERR_UNSUPPORTED;
+}
+
+} // namespace dmoe
+#endif

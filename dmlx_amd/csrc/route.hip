@@ -1,0 +1,248 @@
+// Router top-k (one wavefront per token, shuffle reductions), index remap, expand / reduce,
+// and the host-side Smelt mask / remap builders.
+#include <math.h>
+#include <string.h>
+
+#include "common.h"
+
+namespace dmoe {
+
+// Monotone u32 key of an f32 for "ascending stable argsort, NaN last, -0 == +0".
+// Never returns 0, so 0 can mark an entry that was already taken.
+__device__ __forceinline__ uint32_t f32_sort_key(float c) {
+    if (c != c) return 0xffffffffu;
+    if (c == 0.0f) return 0x80000000u;
+    uint32_t b = __float_as_uint(c);
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
+constexpr int kRouteWaves = 4;
+
+// One wavefront per token. The K winners are found by K rounds of a wave-wide arg-max over
+// (key, index) pairs: the pair order makes the HIGHER index win among equal scores, which is what
+// "take the last K columns of a stable ascending argsort" selects, and round r fills column K-1-r so
+// the columns come out in ascending score order.
+__global__ __launch_bounds__(kRouteWaves * 64) void route_kernel(
+    uint32_t *__restrict__ out_idx, float *__restrict__ out_w, const float *__restrict__ scores,
+    const float *__restrict__ bias, const uint8_t *__restrict__ resident, int T, int E, int K,
+    int normalize, int apply_scale, float route_scale) {
+    extern __shared__ uint32_t route_keys[]; // [kRouteWaves][E]
+    const int wave = (int)(threadIdx.x >> 6), lane = lane_id();
+    const int t = (int)blockIdx.x * kRouteWaves + wave;
+    if (t >= T) return; // no block-wide barrier below
+    uint32_t *key = route_keys + (size_t)wave * E;
+    const float *s = scores + (size_t)t * E;
+    // each lane only ever touches entries e == lane (mod 64): no cross-lane hazards on `key`
+    for (int e = lane; e < E; e += 64) {
+        float c = s[e];
+        if (bias) c = c + bias[e];
+        if (resident) c = c + (resident[e] ? 0.0f : -1e9f);
+        key[e] = f32_sort_key(c);
+    }
+    uint32_t my_idx = 0;
+    for (int it = 0; it < K; ++it) {
+        uint32_t bk = 0, bi = 0;
+        for (int e = lane; e < E; e += 64) {
+            uint32_t k = key[e];
+            if (k > bk || (k == bk && (uint32_t)e > bi)) { bk = k; bi = (uint32_t)e; }
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            uint32_t ok = (uint32_t)__shfl_xor((int)bk, off, 64);
+            uint32_t oi = (uint32_t)__shfl_xor((int)bi, off, 64);
+            if (ok > bk || (ok == bk && oi > bi)) { bk = ok; bi = oi; }
+        }
+        if ((int)(bi & 63u) == lane) key[bi] = 0; // taken
+        if (lane == K - 1 - it) my_idx = bi;
+    }
+    float my_w = (lane < K) ? s[my_idx] : 0.0f;
+    float sum = 0.0f;
+    for (int j = 0; j < K; ++j) sum += __shfl(my_w, j, 64); // left to right, like a row reduction
+    float w = my_w;
+    if (normalize) w = w / (sum + 1e-20f);
+    if (apply_scale) w = w * route_scale;
+    if (lane < K) {
+        out_idx[(size_t)t * K + lane] = my_idx;
+        out_w[(size_t)t * K + lane] = w;
+    }
+}
+
+static int launch_route(uint32_t *out_idx, float *out_w, const float *scores, const float *bias,
+                        const uint8_t *resident, int T, int E, int K, int normalize, int apply_scale,
+                        float route_scale, hipStream_t st) {
+    DMOE_REQUIRE(T >= 0 && E >= 1 && E <= 1024, "route: E=%d out of range [1,1024]", E);
+    DMOE_REQUIRE(K >= 1 && K <= E && K <= 64, "route: K=%d must satisfy 1 <= K <= min(E,64)", K);
+    if (T == 0) return DMOE_OK;
+    DMOE_REQUIRE(out_idx && out_w && scores, "route: null pointer");
+    dim3 grid((unsigned)ceil_div(T, kRouteWaves)), block(kRouteWaves * 64);
+    size_t lds = sizeof(uint32_t) * (size_t)kRouteWaves * E;
+    hipLaunchKernelGGL(route_kernel, grid, block, lds, st, out_idx, out_w, scores, bias, resident, T, E,
+                       K, normalize, apply_scale, route_scale);
+    DMOE_LAUNCH_CHECK();
+    return DMOE_OK;
+}
+
+__global__ void remap_kernel(uint32_t *__restrict__ out, const int32_t *__restrict__ remap,
+                             const uint32_t *__restrict__ idx, size_t n, uint32_t n_total) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    uint32_t e = idx[i];
+    // an id outside the table would read out of bounds; map it to slot 0 like an unloaded expert
+    out[i] = e < n_total ? (uint32_t)remap[e] : 0u;
+}
+
+// out[(t*K+k), :] = x[t, :], 16 bytes per thread
+__global__ void expand_kernel(uint4 *__restrict__ out, const uint4 *__restrict__ x, size_t row_vecs,
+                              int K, size_t total_vecs) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total_vecs) return;
+    size_t row = i / row_vecs, c = i - row * row_vecs;
+    out[i] = x[(row / (size_t)K) * row_vecs + c];
+}
+__global__ void expand_kernel_bytes(uint8_t *__restrict__ out, const uint8_t *__restrict__ x,
+                                    size_t row_bytes, int K, size_t total) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    size_t row = i / row_bytes, c = i - row * row_bytes;
+    out[i] = x[(row / (size_t)K) * row_bytes + c];
+}
+
+template <bool BF16>
+__global__ void reduce_kernel(float *__restrict__ out, const void *__restrict__ eo,
+                              const float *__restrict__ w, int T, int K, int D) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)T * D) return;
+    size_t t = i / (size_t)D, d = i - t * (size_t)D;
+    float acc = 0.0f;
+    for (int k = 0; k < K; ++k) {
+        size_t r = t * (size_t)K + k;
+        float v = BF16 ? bf16_bits_to_f32(((const uint16_t *)eo)[r * D + d]) : ((const float *)eo)[r * D + d];
+        acc += v * w[r]; // separate multiply and add, k ascending
+    }
+    out[i] = acc;
+}
+
+} // namespace dmoe
+
+using namespace dmoe;
+
+extern "C" {
+
+int dmoe_topk_route(uint32_t *d_out_indices, float *d_out_weights, const float *d_scores, int T, int E,
+                    int K, int normalize, dmoe_stream s) {
+    return launch_route(d_out_indices, d_out_weights, d_scores, nullptr, nullptr, T, E, K, normalize, 0,
+                        1.0f, to_hip(s));
+}
+
+int dmoe_gate_route(uint32_t *d_out_indices, float *d_out_weights, const float *d_scores,
+                    const float *d_bias, const uint8_t *d_resident_mask, int T, int E, int K, int renorm,
+                    float route_scale, dmoe_stream s) {
+    return launch_route(d_out_indices, d_out_weights, d_scores, d_bias, d_resident_mask, T, E, K, renorm,
+                        1, route_scale, to_hip(s));
+}
+
+int dmoe_remap_indices(uint32_t *d_out, const int32_t *d_remap, const uint32_t *d_indices, size_t n,
+                       int n_total, dmoe_stream s) {
+    if (n == 0) return DMOE_OK;
+    DMOE_REQUIRE(d_out && d_remap && d_indices && n_total > 0, "remap: bad argument");
+    hipLaunchKernelGGL(remap_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, to_hip(s), d_out,
+                       d_remap, d_indices, n, (uint32_t)n_total);
+    DMOE_LAUNCH_CHECK();
+    return DMOE_OK;
+}
+
+int dmoe_expand_tokens(void *d_out, const void *d_x, int T, int D, int K, int elem_size, dmoe_stream s) {
+    DMOE_REQUIRE(T >= 0 && D > 0 && K > 0 && (elem_size == 2 || elem_size == 4), "expand: bad shape");
+    if (T == 0) return DMOE_OK;
+    DMOE_REQUIRE(d_out && d_x, "expand: null pointer");
+    size_t row_bytes = (size_t)D * elem_size;
+    if (row_bytes % 16 == 0 && ((uintptr_t)d_out % 16 == 0) && ((uintptr_t)d_x % 16 == 0)) {
+        size_t rv = row_bytes / 16, total = rv * (size_t)T * K;
+        hipLaunchKernelGGL(expand_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, to_hip(s),
+                           (uint4 *)d_out, (const uint4 *)d_x, rv, K, total);
+    } else {
+        size_t total = row_bytes * (size_t)T * K;
+        hipLaunchKernelGGL(expand_kernel_bytes, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                           to_hip(s), (uint8_t *)d_out, (const uint8_t *)d_x, row_bytes, K, total);
+    }
+    DMOE_LAUNCH_CHECK();
+    return DMOE_OK;
+}
+
+int dmoe_reduce_experts(float *d_out, const void *d_expert_outs, int outs_are_bf16, const float *d_weights,
+                        int T, int K, int D, dmoe_stream s) {
+    DMOE_REQUIRE(T >= 0 && D > 0 && K > 0, "reduce: bad shape");
+    if (T == 0) return DMOE_OK;
+    DMOE_REQUIRE(d_out && d_expert_outs && d_weights, "reduce: null pointer");
+    size_t total = (size_t)T * D;
+    dim3 grid((unsigned)((total + 255) / 256)), block(256);
+    if (outs_are_bf16)
+        hipLaunchKernelGGL(reduce_kernel<true>, grid, block, 0, to_hip(s), d_out, d_expert_outs, d_weights,
+                           T, K, D);
+    else
+        hipLaunchKernelGGL(reduce_kernel<false>, grid, block, 0, to_hip(s), d_out, d_expert_outs,
+                           d_weights, T, K, D);
+    DMOE_LAUNCH_CHECK();
+    return DMOE_OK;
+}
+
+// ---- host-side builders (integers; no device work) -------------------------------------------------
+
+int dmoe_smelt_build_mask(uint8_t *h_out_mask, int *out_n_resident, int n_experts, float load_fraction,
+                          int strategy, int enabled) {
+    DMOE_REQUIRE(h_out_mask && n_experts > 0, "smelt mask: bad argument");
+    DMOE_REQUIRE(strategy == 0 || strategy == 1, "smelt mask: strategy must be 0 (uniform) or 1 (first)");
+    memset(h_out_mask, 0, (size_t)n_experts);
+    if (!enabled || load_fraction >= 1.0f) {
+        memset(h_out_mask, 1, (size_t)n_experts);
+    } else {
+        // f32 arithmetic and round-half-away, as the reference's @round on f32
+        long n_load = (long)roundf(load_fraction * (float)n_experts);
+        if (n_load < 1) n_load = 1;
+        if (n_load > n_experts) n_load = n_experts;
+        if (strategy == 1) {
+            for (long i = 0; i < n_load; ++i) h_out_mask[i] = 1;
+        } else if (n_load == 1) {
+            h_out_mask[0] = 1; // the reference divides by n_load-1 here; a single pick is expert 0
+        } else {
+            float step = (float)(n_experts - 1) / (float)(n_load - 1);
+            for (long i = 0; i < n_load; ++i) {
+                long idx = (long)roundf(step * (float)i);
+                if (idx > n_experts - 1) idx = n_experts - 1;
+                h_out_mask[idx] = 1;
+            }
+        }
+    }
+    if (out_n_resident) {
+        int c = 0;
+        for (int i = 0; i < n_experts; ++i) c += h_out_mask[i];
+        *out_n_resident = c;
+    }
+    return DMOE_OK;
+}
+
+int dmoe_build_remap(int32_t *h_out_remap, const uint8_t *h_mask, int n_experts) {
+    DMOE_REQUIRE(h_out_remap && h_mask && n_experts > 0, "build remap: bad argument");
+    int32_t slot = 0;
+    for (int e = 0; e < n_experts; ++e) h_out_remap[e] = h_mask[e] ? slot++ : 0;
+    return DMOE_OK;
+}
+
+int dmoe_preload_remap(int32_t *h_out_remap, float *h_out_cache_bias, const uint32_t *h_expert_ids,
+                       int n_ids, int n_total) {
+    DMOE_REQUIRE(h_out_remap && (h_expert_ids || n_ids == 0) && n_total > 0 && n_ids >= 0,
+                 "preload remap: bad argument");
+    for (int e = 0; e < n_total; ++e) {
+        h_out_remap[e] = 0;
+        if (h_out_cache_bias) h_out_cache_bias[e] = -1000.0f;
+    }
+    for (int sidx = 0; sidx < n_ids; ++sidx) {
+        DMOE_REQUIRE(h_expert_ids[sidx] < (uint32_t)n_total, "preload remap: expert id %u >= %d",
+                     h_expert_ids[sidx], n_total);
+        h_out_remap[h_expert_ids[sidx]] = sidx;
+        if (h_out_cache_bias) h_out_cache_bias[h_expert_ids[sidx]] = 0.0f;
+    }
+    return DMOE_OK;
+}
+
+} // extern "C"

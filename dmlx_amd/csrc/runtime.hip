@@ -1,0 +1,231 @@
+// Runtime plumbing of libdmoe: error reporting, device selection, streams, device memory, workspaces.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "common.h"
+
+namespace dmoe {
+
+static thread_local char g_err[2048] = ""; // same size as the reference's mlx error buffer
+
+void set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+int hip_fail(hipError_t e, const char *what) {
+    set_error("HIP error %d (%s) in %s", (int)e, hipGetErrorString(e), what);
+    return DMOE_ERR_HIP;
+}
+
+int workspace_reserve(dmoe_workspace ws, size_t bytes, Workspace **out) {
+    Workspace *w = (Workspace *)ws.ctx;
+    DMOE_REQUIRE(w != nullptr, "workspace handle is null");
+    if (bytes > w->bytes) {
+        // growth is rare (first call at a new size); in-flight work may still use the old block
+        DMOE_HIP(hipDeviceSynchronize());
+        if (w->base) DMOE_HIP(hipFree(w->base));
+        w->base = nullptr;
+        w->bytes = 0;
+        size_t want = bytes + bytes / 4;
+        DMOE_HIP(hipMalloc(&w->base, want));
+        w->bytes = want;
+    }
+    *out = w;
+    return DMOE_OK;
+}
+
+int stage_flush(Workspace *w) {
+    StageTimer &t = w->timer;
+    for (int i = 0; i < DMOE_STAGE_COUNT; ++i) {
+        if (!t.pending[i]) continue;
+        DMOE_HIP(hipEventSynchronize(t.stop[i]));
+        float ms = 0.0f;
+        DMOE_HIP(hipEventElapsedTime(&ms, t.start[i], t.stop[i]));
+        t.total_ms[i] += ms;
+        t.samples[i] += 1;
+        t.pending[i] = false;
+    }
+    return DMOE_OK;
+}
+
+int stage_begin(Workspace *w, int stage, hipStream_t st) {
+    StageTimer &t = w->timer;
+    if (!t.enabled) return DMOE_OK;
+    if (t.pending[stage]) DMOE_TRY(stage_flush(w)); // the event pair is about to be reused
+    DMOE_HIP(hipEventRecord(t.start[stage], st));
+    return DMOE_OK;
+}
+
+int stage_end(Workspace *w, int stage, hipStream_t st) {
+    StageTimer &t = w->timer;
+    if (!t.enabled) return DMOE_OK;
+    DMOE_HIP(hipEventRecord(t.stop[stage], st));
+    t.pending[stage] = true;
+    return DMOE_OK;
+}
+
+} // namespace dmoe
+
+using namespace dmoe;
+
+extern "C" {
+
+int dmoe_version(void) { return DMOE_VERSION; }
+
+const char *dmoe_last_error(void) { return g_err; }
+
+int dmoe_quant_mode_from_string(const char *name) {
+    if (!name) return -1;
+    if (!strcmp(name, "affine")) return DMOE_QUANT_AFFINE;
+    if (!strcmp(name, "mxfp4")) return DMOE_QUANT_MXFP4;
+    if (!strcmp(name, "fp8")) return DMOE_QUANT_FP8_ROW;
+    return -1;
+}
+
+int dmoe_init(int device) {
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0) {
+        set_error("no HIP device visible (%s)", e == hipSuccess ? "count is 0" : hipGetErrorString(e));
+        return DMOE_ERR_NO_DEVICE;
+    }
+    if (device >= 0) {
+        DMOE_REQUIRE(device < n, "device %d out of range (%d visible)", device, n);
+        DMOE_HIP(hipSetDevice(device));
+    } else {
+        DMOE_HIP(hipGetDevice(&device));
+    }
+    hipDeviceProp_t prop;
+    DMOE_HIP(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        set_error("device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
+        return DMOE_ERR_NO_DEVICE;
+    }
+    return DMOE_OK;
+}
+
+int dmoe_stream_create(dmoe_stream *out) {
+    DMOE_REQUIRE(out != nullptr, "out is null");
+    hipStream_t st;
+    DMOE_HIP(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+    out->ctx = (void *)st;
+    return DMOE_OK;
+}
+
+int dmoe_stream_destroy(dmoe_stream s) {
+    if (s.ctx) DMOE_HIP(hipStreamDestroy(to_hip(s)));
+    return DMOE_OK;
+}
+
+int dmoe_stream_synchronize(dmoe_stream s) {
+    DMOE_HIP(hipStreamSynchronize(to_hip(s)));
+    return DMOE_OK;
+}
+
+int dmoe_malloc(void **out, size_t bytes) {
+    DMOE_REQUIRE(out != nullptr, "out is null");
+    *out = nullptr;
+    if (bytes == 0) return DMOE_OK;
+    DMOE_HIP(hipMalloc(out, bytes));
+    return DMOE_OK;
+}
+
+int dmoe_free(void *p) {
+    if (p) DMOE_HIP(hipFree(p));
+    return DMOE_OK;
+}
+
+int dmoe_copy_to_device(void *dst, const void *src, size_t bytes, dmoe_stream s) {
+    if (bytes == 0) return DMOE_OK;
+    DMOE_REQUIRE(dst && src, "null pointer");
+    DMOE_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, to_hip(s)));
+    // pageable host memory: the runtime may still read `src` after returning; wait so the caller may reuse it
+    DMOE_HIP(hipStreamSynchronize(to_hip(s)));
+    return DMOE_OK;
+}
+
+int dmoe_copy_to_host(void *dst, const void *src, size_t bytes, dmoe_stream s) {
+    if (bytes == 0) return DMOE_OK;
+    DMOE_REQUIRE(dst && src, "null pointer");
+    DMOE_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, to_hip(s)));
+    DMOE_HIP(hipStreamSynchronize(to_hip(s)));
+    return DMOE_OK;
+}
+
+int dmoe_workspace_create(dmoe_workspace *out, size_t initial_bytes) {
+    DMOE_REQUIRE(out != nullptr, "out is null");
+    Workspace *w = new Workspace();
+    hipError_t e = hipGetDevice(&w->device);
+    if (e != hipSuccess) {
+        delete w;
+        return hip_fail(e, "hipGetDevice");
+    }
+    out->ctx = w;
+    if (initial_bytes) {
+        Workspace *tmp;
+        int rc = workspace_reserve(*out, initial_bytes, &tmp);
+        if (rc != DMOE_OK) {
+            delete w;
+            out->ctx = nullptr;
+            return rc;
+        }
+    }
+    return DMOE_OK;
+}
+
+int dmoe_workspace_set_stage_timing(dmoe_workspace ws, int enabled) {
+    Workspace *w = (Workspace *)ws.ctx;
+    DMOE_REQUIRE(w != nullptr, "workspace handle is null");
+    StageTimer &t = w->timer;
+    if (enabled && !t.start[0]) {
+        for (int i = 0; i < DMOE_STAGE_COUNT; ++i) {
+            DMOE_HIP(hipEventCreate(&t.start[i]));
+            DMOE_HIP(hipEventCreate(&t.stop[i]));
+        }
+    }
+    if (!enabled && t.enabled) DMOE_TRY(stage_flush(w));
+    if (enabled && !t.enabled)
+        for (int i = 0; i < DMOE_STAGE_COUNT; ++i) {
+            t.total_ms[i] = 0.0f;
+            t.samples[i] = 0;
+            t.pending[i] = false;
+        }
+    t.enabled = enabled != 0;
+    return DMOE_OK;
+}
+
+int dmoe_workspace_read_stage_times(float *h_out_total_ms, int *h_out_samples, dmoe_workspace ws) {
+    Workspace *w = (Workspace *)ws.ctx;
+    DMOE_REQUIRE(w && h_out_total_ms && h_out_samples, "null argument");
+    DMOE_TRY(stage_flush(w));
+    for (int i = 0; i < DMOE_STAGE_COUNT; ++i) {
+        h_out_total_ms[i] = w->timer.total_ms[i];
+        h_out_samples[i] = w->timer.samples[i];
+    }
+    return DMOE_OK;
+}
+
+int dmoe_workspace_destroy(dmoe_workspace ws) {
+    Workspace *w = (Workspace *)ws.ctx;
+    if (!w) return DMOE_OK;
+    for (int i = 0; i < DMOE_STAGE_COUNT; ++i) {
+        if (w->timer.start[i]) (void)hipEventDestroy(w->timer.start[i]);
+        if (w->timer.stop[i]) (void)hipEventDestroy(w->timer.stop[i]);
+    }
+    hipError_t e = w->base ? hipFree(w->base) : hipSuccess;
+    delete w;
+    if (e != hipSuccess) return hip_fail(e, "hipFree(workspace)");
+    return DMOE_OK;
+}
+
+int dmoe_workspace_reserved(size_t *out_bytes, dmoe_workspace ws) {
+    DMOE_REQUIRE(out_bytes && ws.ctx, "null argument");
+    *out_bytes = ((Workspace *)ws.ctx)->bytes;
+    return DMOE_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,249 @@
+/*
+ * dmoe — MI355X (gfx950) implementation of dmlx's quantized MoE expert-FFN path.
+ *
+ * C ABI of libdmoe.so. Conventions follow the mlx-c call style the reference binds
+ * (out-parameters first, inputs next, stream last, `int` return code, 0 = ok; see
+ * e.g. moe_router.zig:61,78 and deepseek_v4.zig:1037 in the reference):
+ *   - every pointer named `d_*` is DEVICE memory (HIP), dense row-major, owned by
+ *     the caller; inputs are borrowed for the duration of the call, outputs are
+ *     written in place. Nullable arguments say so.
+ *   - bf16 tensors are passed as `uint16_t*` bit patterns.
+ *   - all work is enqueued on the given stream and returns without waiting;
+ *     `dmoe_stream_synchronize` is the only wait. A stream with ctx == NULL is the
+ *     default HIP stream.
+ *   - a non-zero return code means nothing useful was enqueued; the message is
+ *     available (per thread) from `dmoe_last_error()`. The reference maps any
+ *     non-zero mlx-c code to one Zig error after logging the message; a binding
+ *     does the same here.
+ *   - calls that share one `dmoe_workspace` must be ordered on one stream.
+ *
+ * Each entry point names the reference interface it replaces (file:line in the
+ * reference tree).
+ */
+#ifndef DMOE_H
+#define DMOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DMOE_VERSION 100 /* 0.1.0 */
+
+typedef enum {
+    DMOE_OK = 0,
+    DMOE_ERR_INVALID = 1,     /* bad argument / unsupported shape            */
+    DMOE_ERR_HIP = 2,         /* a HIP runtime call failed                   */
+    DMOE_ERR_UNSUPPORTED = 3, /* valid request this build does not implement */
+    DMOE_ERR_NO_DEVICE = 4    /* no gfx950 device visible                    */
+} dmoe_status;
+
+/* quantization mode; the reference passes it as the C strings "affine"/"mxfp4"
+ * (deepseek_v4.zig:974, deepseek_v4_loader.zig:129) */
+typedef enum {
+    DMOE_QUANT_AFFINE = 0, /* bits 4|8, group 32|64|128, bf16 scales + bf16 biases (biases nullable = 0) */
+    DMOE_QUANT_MXFP4 = 1,  /* E2M1 nibbles, one E8M0 byte per 32 values, no biases                      */
+    DMOE_QUANT_FP8_ROW = 2 /* E4M3FN bytes, one f32 scale per output row, no biases                     */
+} dmoe_quant_mode;
+
+typedef struct dmoe_stream_ { void *ctx; } dmoe_stream;           /* ctx = hipStream_t */
+typedef struct dmoe_workspace_ { void *ctx; } dmoe_workspace;     /* grow-only device scratch */
+typedef struct dmoe_layer_ { void *ctx; } dmoe_layer;             /* resident expert weights of one MoE layer */
+
+/* "affine" -> DMOE_QUANT_AFFINE, "mxfp4" -> DMOE_QUANT_MXFP4, "fp8" -> DMOE_QUANT_FP8_ROW; -1 if unknown */
+int dmoe_quant_mode_from_string(const char *name);
+
+/* ---- runtime ------------------------------------------------------------------ */
+
+int dmoe_version(void);
+const char *dmoe_last_error(void);              /* thread-local, never NULL */
+/* replaces c.initErrorHandler() + default GPU stream set-up (src/tests.zig:66-68, main.zig:479-480):
+ * selects the device, checks it is gfx950. device < 0 keeps the current device. */
+int dmoe_init(int device);
+
+int dmoe_stream_create(dmoe_stream *out);
+int dmoe_stream_destroy(dmoe_stream s);
+int dmoe_stream_synchronize(dmoe_stream s);     /* replaces Array.eval() as the host-visible sync point */
+
+/* device memory for host languages that do not link HIP themselves (what Array.fromData /
+ * dataSlice do in the reference: copies in and out of device arrays) */
+int dmoe_malloc(void **out_d_ptr, size_t bytes);
+int dmoe_free(void *d_ptr);
+int dmoe_copy_to_device(void *d_dst, const void *h_src, size_t bytes, dmoe_stream s);
+int dmoe_copy_to_host(void *h_dst, const void *d_src, size_t bytes, dmoe_stream s);   /* waits for the copy */
+
+int dmoe_workspace_create(dmoe_workspace *out, size_t initial_bytes);
+int dmoe_workspace_destroy(dmoe_workspace ws);
+/* bytes currently reserved; growth happens inside calls (it synchronizes the device) */
+int dmoe_workspace_reserved(size_t *out_bytes, dmoe_workspace ws);
+
+/* Per-stage device timing of the layer forward calls made with this workspace (HIP events recorded on the
+ * call's stream around each stage). Off by default; while on, every forward call waits for the previous
+ * call's events, so use it for measurement runs only. No counterpart in the reference, which logs host wall
+ * time per token step (expert_stream.zig:587-610). */
+enum {
+    DMOE_STAGE_ROUTE = 0,        /* dmoe_gate_route inside dmoe_moe_layer_forward */
+    DMOE_STAGE_PACK = 1,         /* remap + counting sort                         */
+    DMOE_STAGE_GATE_UP = 2,      /* grouped gate/up GEMM + SwiGLU                 */
+    DMOE_STAGE_DOWN = 3,         /* grouped down GEMM                             */
+    DMOE_STAGE_SHARED = 4,       /* shared expert (both GEMMs)                    */
+    DMOE_STAGE_COMBINE = 5,      /* weighted sum over k + shared add              */
+    DMOE_STAGE_COUNT = 6
+};
+int dmoe_workspace_set_stage_timing(dmoe_workspace ws, int enabled);
+/* total milliseconds and number of samples per stage since timing was enabled; arrays of DMOE_STAGE_COUNT */
+int dmoe_workspace_read_stage_times(float *h_out_total_ms, int *h_out_samples, dmoe_workspace ws);
+
+/* ---- router ------------------------------------------------------------------- */
+
+/* MoERouter.topkRoute (moe_router.zig:55-103): per token, the K largest of E scores.
+ * Columns are in ASCENDING score order (the reference slices the last K columns of an
+ * ascending argsort); among equal scores the higher expert index wins. Weights are the
+ * selected scores, divided by (sum_k + 1e-20) when `normalize` != 0.
+ *   d_out_indices u32 [T,K], d_out_weights f32 [T,K], d_scores f32 [T,E]; 1 <= K <= E <= 1024 */
+int dmoe_topk_route(uint32_t *d_out_indices, float *d_out_weights, const float *d_scores,
+                    int T, int E, int K, int normalize, dmoe_stream s);
+
+/* DSV4Gate.forward from the scores on (deepseek_v4.zig:589-678): selection on
+ * scores + bias[E] (+ -1e9 where resident_mask[e] == 0), weights gathered from the
+ * unbiased scores, divided by (sum_k + 1e-20) when `renorm` != 0 (the reference does so
+ * for every scoring function except softmax, :663), then * route_scale (:676-678).
+ *   d_bias f32 [E] nullable; d_resident_mask u8 [E] nullable (Smelt mask, :601-615) */
+int dmoe_gate_route(uint32_t *d_out_indices, float *d_out_weights, const float *d_scores,
+                    const float *d_bias, const uint8_t *d_resident_mask,
+                    int T, int E, int K, int renorm, float route_scale, dmoe_stream s);
+
+/* mlx_take(remap, indices).astype(u32) (deepseek_v4.zig:1035-1039, expert_preload.zig:200-206):
+ * d_out[i] = (u32) d_remap[d_indices[i]], n elements, every index < n_total. */
+int dmoe_remap_indices(uint32_t *d_out, const int32_t *d_remap, const uint32_t *d_indices,
+                       size_t n, int n_total, dmoe_stream s);
+
+/* MoERouter.expandTokens (moe_router.zig:111-132): out[t*K+k, :] = x[t, :]; elem_size in bytes (2 or 4) */
+int dmoe_expand_tokens(void *d_out, const void *d_x, int T, int D, int K, int elem_size, dmoe_stream s);
+
+/* MoERouter.reduceExperts (moe_router.zig:139-164): out[t,:] = sum_k w[t,k] * expert_outs[t*K+k,:], f32,
+ * summed over k left to right. expert_outs is f32 (outs_are_bf16 == 0) or bf16. */
+int dmoe_reduce_experts(float *d_out, const void *d_expert_outs, int outs_are_bf16, const float *d_weights,
+                        int T, int K, int D, dmoe_stream s);
+
+/* SmeltConfig.buildMask (deepseek_v4_loader.zig:272-293), host side: h_out_mask u8 [n_experts];
+ * strategy 0 = uniform, 1 = first. Returns the number of resident experts in *out_n_resident. */
+int dmoe_smelt_build_mask(uint8_t *h_out_mask, int *out_n_resident, int n_experts, float load_fraction,
+                          int strategy, int enabled);
+/* expert_remap construction (deepseek_v4_loader.zig:2151-2168), host side: running slot index over the
+ * mask, non-resident experts map to slot 0. */
+int dmoe_build_remap(int32_t *h_out_remap, const uint8_t *h_mask, int n_experts);
+/* ExpertPreloadProvider.init remap + cache bias (expert_preload.zig:141-160), host side:
+ * remap[ids[s]] = s (others 0); cache_bias 0 for loaded ids, -1000 otherwise (nullable). */
+int dmoe_preload_remap(int32_t *h_out_remap, float *h_out_cache_bias, const uint32_t *h_expert_ids,
+                       int n_ids, int n_total);
+
+/* ---- packing (token -> expert segments) --------------------------------------------- */
+
+/* The sort block of DSV4SwitchGLU.forward (deepseek_v4.zig:749-784) as one stable counting sort:
+ *   order[p]     = flat index (t*K+k) of the p-th row when rows are grouped by expert, ties in
+ *                  ascending flat index                                (argsort(flat_indices), :753)
+ *   inv_order[i] = position of flat index i                            (argsort(order), :758)
+ *   token[p]     = order[p] / K                                        (:765-772)
+ *   sorted_expert[p] = indices[order[p]]                               (:777-779)
+ *   counts[e], offsets[e] = rows of expert e and their exclusive scan; offsets[E] = T*K
+ * plus what expert_stream.zig:449-465 derives on the host: live_experts = ascending ids with
+ * counts > 0 and *n_live their number (d_out_n_live is a device u32).
+ * Any output pointer except d_out_order may be NULL. indices < E <= 1024. */
+int dmoe_pack(uint32_t *d_out_order, uint32_t *d_out_inv_order, uint32_t *d_out_token,
+              uint32_t *d_out_sorted_expert, uint32_t *d_out_counts, uint32_t *d_out_offsets,
+              uint32_t *d_out_live_experts, uint32_t *d_out_n_live,
+              const uint32_t *d_indices, int T, int K, int E, dmoe_workspace ws, dmoe_stream s);
+
+/* ---- quantized weights ------------------------------------------------------------------ */
+
+/* one stack [n_mats, rows, cols] of quantized matrices in MLX layout (out-features = rows):
+ *   affine : w u32 [n, rows, cols*bits/32]; scales, biases bf16 [n, rows, cols/group_size]
+ *   mxfp4  : w u32 [n, rows, cols/8];       scales u8 [n, rows, cols/32]; biases NULL
+ *   fp8row : w u8  [n, rows, cols];         scales f32 [n, rows];         biases NULL
+ * (QuantizedWeight / QuantConfig of mlx-zig as used at deepseek_v4.zig:474-481, :971-976) */
+typedef struct {
+    const void *w;
+    const void *scales;
+    const void *biases; /* nullable */
+    int n_mats, rows, cols;
+    int mode;           /* dmoe_quant_mode */
+    int bits;           /* 4 | 8 (affine), 4 (mxfp4), 8 (fp8row) */
+    int group_size;     /* 32 | 64 | 128 (affine), 32 (mxfp4), ignored (fp8row) */
+} dmoe_qweight;
+
+/* mlx_dequantize(..., dtype = bf16) (deepseek_v4_loader.zig:129): d_out bf16 [rows, cols] of matrix
+ * `mat_index`; value = q*scale + bias evaluated in f32 and rounded once to bf16 (affine),
+ * E2M1 * 2^(s-127) (mxfp4, exact), e4m3 * row_scale rounded to bf16 (fp8row). Device pointers in `qw`. */
+int dmoe_dequantize(uint16_t *d_out, const dmoe_qweight *qw, int mat_index, dmoe_stream s);
+
+/* quantize_mod.gatherQmm(x, w, scales, biases, lhs_indices, rhs_indices, transpose = true, cfg, sorted)
+ * (call shape deepseek_v4.zig:976, expert_preload.zig:265; mlx.core.gather_qmm):
+ *   out[r, :] = x[lhs ? lhs[r] : r, :] . dequant(W[rhs[r]])^T     r < R
+ * x bf16 [*, cols], out bf16 [R, rows], f32 accumulation. d_lhs_indices nullable. `sorted` != 0 promises
+ * non-decreasing rhs_indices (as the reference's sorted=true); the result is the same either way. */
+int dmoe_gather_qmm(uint16_t *d_out, const uint16_t *d_x, const dmoe_qweight *qw,
+                    const uint32_t *d_lhs_indices, const uint32_t *d_rhs_indices, int R, int sorted,
+                    dmoe_workspace ws, dmoe_stream s);
+
+/* ---- resident MoE layer -------------------------------------------------------------------- */
+
+typedef enum {
+    DMOE_WEIGHTS_COPY_FROM_HOST = 0,   /* pointers in the descriptor are host memory; copied to HBM   */
+    DMOE_WEIGHTS_COPY_FROM_DEVICE = 1, /* device memory; copied, caller may free its copy afterwards  */
+    DMOE_WEIGHTS_BORROW_DEVICE = 2     /* device memory used in place; must outlive the layer         */
+} dmoe_weight_source;
+
+/* DSV4SwitchGLU fields (deepseek_v4.zig:687-705) + DSV4Expert fields for the shared expert (:442-457)
+ * + DSV4MoE.expert_remap (:991-993). Replaces LayerExpertMeta + the SSD/LFU expert cache of
+ * expert_stream.zig / expert_cache.zig: all `n_mats` expert slots stay resident in HBM. */
+typedef struct {
+    int hidden;                 /* D */
+    int ffn;                    /* F (routed experts)                         */
+    int top_k;                  /* K                                          */
+    dmoe_qweight gate, up, down;/* gate/up: rows=F, cols=D; down: rows=D, cols=F; n_mats = resident slots */
+    float swiglu_limit;         /* limitedSwiGLU clamp, 0 = none (:947-966)   */
+    int score_before_down;      /* 1 = DSV4SwitchGLU.forward (:796-806); 0 = provider paths
+                                   (expert_stream.zig:575-580, expert_preload.zig:283-289) */
+    int has_shared;             /* shared expert (DSV4Expert, :489-517), n_mats = 1, rows/cols as above with its own F */
+    dmoe_qweight shared_gate, shared_up, shared_down;
+    float shared_swiglu_limit;  /* the reference builds the shared expert with 0 (deepseek_v4_loader.zig:1893) */
+    const int32_t *remap;       /* nullable HOST i32 [n_experts_total]: router id -> slot (:1035-1039) */
+    int n_experts_total;        /* length of remap; ignored when remap is NULL */
+    int weight_source;          /* dmoe_weight_source */
+} dmoe_layer_desc;
+
+int dmoe_layer_create(dmoe_layer *out, const dmoe_layer_desc *desc, dmoe_stream s);
+int dmoe_layer_destroy(dmoe_layer layer);
+
+/* ExpertProvider.VTable.forward(ptr, layer_idx, flat_x, indices, scores) (expert_provider.zig:21) ==
+ * ExpertStreamProvider.streamForward (expert_stream.zig:245-261) == the provider arm of DSV4MoE.forward
+ * (deepseek_v4.zig:1030-1047), plus the shared expert and the final add (:1021, :1050-1052) when the layer
+ * has one: remap -> pack -> grouped gate/up + limited SwiGLU -> grouped down -> weighted sum over k.
+ *   d_out bf16 [T,D]; d_x bf16 [T,D]; d_indices u32 [T,K] router expert ids; d_scores f32 [T,K] */
+int dmoe_moe_forward(uint16_t *d_out, dmoe_layer layer, const uint16_t *d_x, const uint32_t *d_indices,
+                     const float *d_scores, int T, dmoe_workspace ws, dmoe_stream s);
+
+/* DSV4SwitchGLU.forwardNoScores (deepseek_v4.zig:855-945): expert outputs without score weighting,
+ * d_out bf16 [T,K,D] in (t,k) order; indices are slot ids (no remap applied, no shared expert). */
+int dmoe_switch_glu_forward_no_scores(uint16_t *d_out, dmoe_layer layer, const uint16_t *d_x,
+                                      const uint32_t *d_slot_indices, int T, dmoe_workspace ws, dmoe_stream s);
+
+/* DSV4MoE.forward from the gate scores on (deepseek_v4.zig:1021-1052): dmoe_gate_route followed by
+ * dmoe_moe_forward. d_scores f32 [T,E_total]; d_bias, d_resident_mask nullable as in dmoe_gate_route.
+ * d_out_indices / d_out_weights (nullable) receive the routing for inspection. */
+int dmoe_moe_layer_forward(uint16_t *d_out, uint32_t *d_out_indices, float *d_out_weights, dmoe_layer layer,
+                           const uint16_t *d_x, const float *d_scores, const float *d_bias,
+                           const uint8_t *d_resident_mask, int T, int E_total, int renorm, float route_scale,
+                           dmoe_workspace ws, dmoe_stream s);
+
+/* Inspection of the last dmoe_moe_forward / dmoe_switch_glu_forward_no_scores on this workspace:
+ * the SwiGLU activations in flat (t*K+k) row order, bf16 [T*K, F]. For parity tests. */
+int dmoe_debug_last_activations(uint16_t *d_out, dmoe_layer layer, int T, dmoe_workspace ws, dmoe_stream s);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DMOE_H */

@@ -1,0 +1,184 @@
+"""GPU parity: dequantize (bit-exact), gather_qmm and the MoE layer forward (bf16 outputs within
+max-abs-rel 1e-2 of the fp32-accumulating oracle), through the C ABI, for every weight format and for both
+GEMM paths (small-M decode kernel, MFMA prefill kernel)."""
+import numpy as np
+import pytest
+import torch
+
+from dmlx_amd import quantize as Q
+from dmlx_amd import workloads
+from dmlx_amd.capi import QUANT_AFFINE, QUANT_FP8_ROW, QUANT_MXFP4, QWeight
+from tests.helpers import bf16_bits, max_abs_rel, oracle_forward, qmat, to_np_u32
+
+pytestmark = pytest.mark.gpu
+
+OUT_TOL = 1e-2   # max |gpu - oracle| / max |oracle| on bf16 outputs
+
+
+def _stack(fmt, n, rows, cols, seed):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    w = torch.randn((n, rows, cols), generator=g, device="cuda") * 0.02
+    if fmt == "affine4":
+        a, s, b = Q.quantize_affine(w, 64, 4)
+        return QWeight(a, s, b, rows, cols, QUANT_AFFINE, 4, 64)
+    if fmt == "affine4g32":
+        a, s, b = Q.quantize_affine(w, 32, 4)
+        return QWeight(a, s, b, rows, cols, QUANT_AFFINE, 4, 32)
+    if fmt == "affine4g128":
+        a, s, b = Q.quantize_affine(w, 128, 4)
+        return QWeight(a, s, b, rows, cols, QUANT_AFFINE, 4, 128)
+    if fmt == "affine8":
+        a, s, b = Q.quantize_affine(w, 64, 8)
+        return QWeight(a, s, b, rows, cols, QUANT_AFFINE, 8, 64)
+    if fmt == "mxfp4":
+        a, s = Q.quantize_mxfp4(w)
+        return QWeight(a, s, None, rows, cols, QUANT_MXFP4, 4, 32)
+    a, s = Q.quantize_fp8_row(w)
+    return QWeight(a, s, None, rows, cols, QUANT_FP8_ROW, 8, 0)
+
+
+FORMATS = ["affine4", "affine4g32", "affine4g128", "affine8", "mxfp4", "fp8row"]
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+def test_dequantize_bit_exact(dmoe, orc, fmt):
+    qw = _stack(fmt, 3, 96, 512, 1)
+    if fmt == "mxfp4":   # exercise extreme shared exponents and every code
+        qw.scales[0, 0, :4] = torch.tensor([0, 1, 254, 200], dtype=torch.uint8, device="cuda")
+        qw.w[0, 0, :4] = torch.tensor([0x76543210, -19088744, 0x0F0F0F0F, 0x7F7F7F7F], dtype=torch.int32, device="cuda")
+    if fmt == "fp8row":  # every byte value, NaN codes included
+        qw.w[0, 0, :256] = torch.arange(256, dtype=torch.uint8, device="cuda")
+    qm = qmat(qw)
+    for m in range(3):
+        got = bf16_bits(dmoe.dequantize(qw, m))
+        want = orc.dequantize(qm, m)
+        nan = (want & 0x7FFF) > 0x7F80
+        np.testing.assert_array_equal(got[~nan], want[~nan])
+        assert ((got[nan] & 0x7FFF) > 0x7F80).all()
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("R,n_mats,rows,cols", [(24, 8, 256, 1024),     # small-M path (<= 4 rows per expert on average)
+                                                (700, 4, 256, 512),     # MFMA path, ragged segments
+                                                (130, 1, 128, 2048)])   # single expert, MFMA, partial tile
+def test_gather_qmm_matches_oracle(dmoe, orc, ws, fmt, R, n_mats, rows, cols):
+    qw = _stack(fmt, n_mats, rows, cols, 2)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn((R + 5, cols), generator=g, device="cuda").to(torch.bfloat16)
+    rhs = torch.randint(0, n_mats, (R,), generator=g, device="cuda", dtype=torch.int32)
+    lhs = torch.randint(0, R + 5, (R,), generator=g, device="cuda", dtype=torch.int32)
+    qm = qmat(qw)
+    for use_lhs in (False, True):
+        got = dmoe.gather_qmm(x, qw, rhs, ws, lhs if use_lhs else None).float().cpu().numpy()
+        want = orc.gather_qmm(bf16_bits(x), qm, to_np_u32(rhs), to_np_u32(lhs) if use_lhs else None)
+        assert max_abs_rel(got, want) < OUT_TOL, (fmt, use_lhs, max_abs_rel(got, want))
+    # sorted indices (the reference's sorted=true call) give the same rows
+    srt = torch.sort(rhs).values.to(torch.int32)
+    got_s = dmoe.gather_qmm(x, qw, srt, ws, None, sorted_indices=True).float().cpu().numpy()
+    want_s = orc.gather_qmm(bf16_bits(x), qm, to_np_u32(srt), None)
+    assert max_abs_rel(got_s, want_s) < OUT_TOL
+
+
+def _route(dmoe, orc, wl):
+    idx, w = dmoe.gate_route(wl.scores, wl.bias, wl.resident_mask, wl.K, wl.renorm, wl.route_scale)
+    want_idx, want_w = orc.gate_route(wl.scores.cpu().numpy(), None if wl.bias is None else wl.bias.cpu().numpy(),
+                                      None if wl.resident_mask is None else wl.resident_mask.cpu().numpy(),
+                                      wl.K, wl.renorm, wl.route_scale)
+    np.testing.assert_array_equal(to_np_u32(idx), want_idx)
+    np.testing.assert_array_equal(w.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
+    return idx, w, want_idx, want_w
+
+
+def _check_layer(dmoe, orc, ws, wl, check_h=True):
+    layer = dmoe.Layer(wl.D, wl.F, wl.K, wl.gate, wl.up, wl.down, swiglu_limit=wl.swiglu_limit,
+                       score_before_down=wl.score_before_down, shared=wl.shared,
+                       shared_swiglu_limit=wl.shared_swiglu_limit, remap=wl.remap)
+    idx, w, want_idx, want_w = _route(dmoe, orc, wl)
+    out = layer.forward(wl.x, idx, w, ws)
+    slots = want_idx if wl.remap is None else orc.remap(np.array(wl.remap, np.int32), want_idx)
+    want, want_h = oracle_forward(wl, slots, want_w, want_h=True)
+    err = max_abs_rel(out.float().cpu().numpy(), want)
+    assert err < OUT_TOL, (wl.name, err)
+    if check_h:
+        h = layer.last_activations(wl.T, ws).float().cpu().numpy()
+        scale = want_w.reshape(-1, 1) if wl.score_before_down else 1.0
+        assert max_abs_rel(h, want_h * scale) < OUT_TOL
+    # one call from the gate scores on gives the same bytes as route + forward
+    out2, idx2, w2 = layer.layer_forward(wl.x, wl.scores, wl.bias, wl.resident_mask, wl.renorm, wl.route_scale, ws,
+                                         want_routing=True)
+    assert torch.equal(out2, out) and torch.equal(idx2, idx) and torch.equal(w2, w)
+    layer.close()
+    return err
+
+
+def test_c0_small_layer_full_size(dmoe, orc, ws):
+    """BASELINE config 0 at its real size: 16 tokens, D=1024, E=8, top-2, F=2048, affine-4 g64, softmax scores
+    renormalised over the top-k (MoERouter.topkRoute)."""
+    wl = workloads.make(0)
+    idx, w = dmoe.topk_route(wl.scores, wl.K, True)
+    want_idx, want_w = orc.topk_route(wl.scores.cpu().numpy(), wl.K, True)
+    np.testing.assert_array_equal(to_np_u32(idx), want_idx)
+    np.testing.assert_array_equal(w.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
+    layer = dmoe.Layer(wl.D, wl.F, wl.K, wl.gate, wl.up, wl.down)
+    out = layer.forward(wl.x, idx, w, ws)
+    want = oracle_forward(wl, want_idx, want_w)
+    assert max_abs_rel(out.float().cpu().numpy(), want) < OUT_TOL
+    # MoERouter surface: expand -> (expert fn) -> reduce reproduces the same layer output
+    y = layer.forward_no_scores(wl.x, idx, ws)                       # [T, K, D]
+    red = dmoe.reduce_experts(y.reshape(wl.T * wl.K, wl.D), w)
+    assert max_abs_rel(red.cpu().numpy(), want) < OUT_TOL
+    layer.close()
+
+
+@pytest.mark.parametrize("config,scale", [(1, 0.125), (1, 0.5), (2, 0.125), (2, 0.5), (3, 0.125), (4, 0.125)])
+def test_configs_reduced_size(dmoe, orc, ws, config, scale):
+    """Configurations 1-4 with E, D, F shrunk (same formats, routing rules and raggedness). Scale 0.5 keeps
+    the decode configurations on the small-M kernel, 0.125 puts them on the MFMA kernel."""
+    wl = workloads.make(config, scale=scale)
+    _check_layer(dmoe, orc, ws, wl)
+
+
+@pytest.mark.parametrize("before", [False, True])
+def test_score_position_variants(dmoe, orc, ws, before):
+    wl = workloads.make(1, scale=0.125)
+    wl.score_before_down = before
+    _check_layer(dmoe, orc, ws, wl)
+
+
+def test_c1_decode_full_size(dmoe, orc, ws):
+    """BASELINE config 1 at full size (64 x 1 tokens, D=4096, 256 experts top-6 + shared, F=2048, affine-4)."""
+    wl = workloads.make(1)
+    _check_layer(dmoe, orc, ws, wl, check_h=True)
+
+
+def test_c2_decode_mxfp4_smelt_full_size(dmoe, orc, ws):
+    wl = workloads.make(2)
+    assert wl.E == 51 and int(wl.resident_mask.sum()) == 51
+    _check_layer(dmoe, orc, ws, wl)
+
+
+def test_forward_edge_cases(dmoe, orc, ws):
+    wl = workloads.make(1, scale=0.125)
+    layer = dmoe.Layer(wl.D, wl.F, wl.K, wl.gate, wl.up, wl.down, swiglu_limit=wl.swiglu_limit, shared=wl.shared)
+    # empty batch: nothing enqueued, no error
+    empty = layer.forward(wl.x[:0], torch.empty((0, wl.K), dtype=torch.int32, device="cuda"),
+                          torch.empty((0, wl.K), dtype=torch.float32, device="cuda"), ws)
+    assert empty.shape == (0, wl.D)
+    # every token on the same K experts (maximally unbalanced segments)
+    T = 40
+    idx = torch.arange(wl.K, dtype=torch.int32, device="cuda").repeat(T, 1)
+    w = torch.full((T, wl.K), 1.0 / wl.K, device="cuda")
+    x = wl.x[:T].contiguous()
+    out = layer.forward(x, idx, w, ws)
+    wl.x, wl.T = x, T
+    want = oracle_forward(wl, to_np_u32(idx), w.cpu().numpy())
+    assert max_abs_rel(out.float().cpu().numpy(), want) < OUT_TOL
+    # a single token
+    out1 = layer.forward(x[:1].contiguous(), idx[:1].contiguous(), w[:1].contiguous(), ws)
+    assert max_abs_rel(out1.float().cpu().numpy(), want[:1]) < OUT_TOL
+    # bad arguments are rejected with a message, nothing is launched
+    with pytest.raises(dmoe.DmoeError):
+        dmoe.topk_route(wl.scores, 2000, True)
+    with pytest.raises(dmoe.DmoeError):
+        dmoe.Layer(wl.D, wl.F + 8, wl.K, wl.gate, wl.up, wl.down)
+    layer.close()
