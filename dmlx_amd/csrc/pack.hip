@@ -218,7 +218,7 @@ int launch_pack(const PackOut &o, const uint32_t *d_idx, size_t n, int K, int E,
     DMOE_REQUIRE(E >= 1 && E <= kPackThreads, "pack: E=%d out of range [1,%d]", E, kPackThreads);
     DMOE_REQUIRE(K >= 1, "pack: K=%d", K);
     DMOE_REQUIRE(n < (1ull << 31), "pack: too many rows");
-    DMOE_REQUIRE(o.order != nullptr && (d_idx != nullptr || n == 0), "pack: null pointer");
+    DMOE_REQUIRE(n == 0 || (o.order != nullptr && d_idx != nullptr), "pack: null pointer");
     if (n <= (size_t)kPackThreads) {
         // also covers n == 0: counts/offsets/n_tiles/n_live are still written (all zero)
         size_t lds = sizeof(uint32_t) * (size_t)kPackWaves * E;

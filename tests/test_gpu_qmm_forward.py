@@ -102,7 +102,11 @@ def _check_layer(dmoe, orc, ws, wl, check_h=True):
     if check_h:
         h = layer.last_activations(wl.T, ws).float().cpu().numpy()
         scale = want_w.reshape(-1, 1) if wl.score_before_down else 1.0
-        assert max_abs_rel(h, want_h * scale) < OUT_TOL
+        # an intermediate, not an output: the oracle rounds sigmoid, silu and the product to bf16 one by
+        # one, the kernel rounds once, so the bar here is two bf16 roundings wider than OUT_TOL
+        err_h = max_abs_rel(h, want_h * scale)
+        assert err_h < 2e-2, (wl.name, "activations", err_h)
+    print(f"[parity] {wl.name}: T={wl.T} out max-abs-rel {err:.3e}")
     # one call from the gate scores on gives the same bytes as route + forward
     out2, idx2, w2 = layer.layer_forward(wl.x, wl.scores, wl.bias, wl.resident_mask, wl.renorm, wl.route_scale, ws,
                                          want_routing=True)
