@@ -126,6 +126,7 @@ __global__ void combine_kernel(uint16_t *__restrict__ out, const uint16_t *__res
 
 // average rows per expert at or below this run on the small-M path
 constexpr int kSmallAvgRows = 4;
+constexpr int kSharedSmallRows = 64;
 
 static bool use_small_path(size_t rows, int n_experts, const QView &b) {
     return qgemm_small_supports(b) && rows <= (size_t)kSmallAvgRows * (size_t)n_experts;
@@ -224,7 +225,9 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
 
 static int shared_forward(const Layer *L, Workspace *w, const FwdLayout &f, const uint16_t *d_x, int T,
                           hipStream_t st) {
-    const bool small = T <= kSmallTileM && qgemm_small_supports(L->sgate.view) && qgemm_small_supports(L->sdown.view);
+    // up to 64 rows the dense expert is streamed by the small-M kernel in 4-row tiles (many workgroups per
+    // weight row block); above that the MFMA kernel amortises the dequantization
+    const bool small = T <= kSharedSmallRows && qgemm_small_supports(L->sgate.view) && qgemm_small_supports(L->sdown.view);
     const int tile_m = small ? kSmallTileM : kMfmaTileM;
     GemmArgs gu;
     gu.b0 = L->sgate.view;

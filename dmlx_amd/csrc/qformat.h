@@ -57,6 +57,19 @@ struct FmtAffine4 {
         m.b = row_b ? bf16_bits_to_f32(((const uint16_t *)row_b)[g]) : 0.0f;
         return m;
     }
+    // the same two values as raw 16-bit words (kept unconverted while a load is in flight)
+    __device__ static __forceinline__ void load_meta_raw(const QView &q, const uint8_t *row_s, const uint8_t *row_b,
+                                                         int k0, uint32_t *sb) {
+        int g = k0 / q.group;
+        sb[0] = ((const uint16_t *)row_s)[g];
+        sb[1] = row_b ? ((const uint16_t *)row_b)[g] : 0u;
+    }
+    __device__ static __forceinline__ Meta meta_from_raw(const uint32_t *sb) {
+        Meta m;
+        m.s = bf16_bits_to_f32(sb[0]);
+        m.b = bf16_bits_to_f32(sb[1]);
+        return m;
+    }
     __device__ static __forceinline__ void decode_word(uint32_t w, Meta m, uint32_t *out /*[4]*/) {
         uint32_t lo = w & 0x0f0f0f0fu, hi = (w >> 4) & 0x0f0f0f0fu; // nibbles 0,2,4,6 / 1,3,5,7 as bytes
         out[0] = pack_bf16x2(fmaf((float)(lo & 0xffu), m.s, m.b), fmaf((float)(hi & 0xffu), m.s, m.b));
@@ -70,6 +83,7 @@ struct FmtAffine4 {
         decode_word(raw.z, m, out + 8);
         decode_word(raw.w, m, out + 12);
     }
+    __device__ static __forceinline__ void decode_fast(const uint4 &raw, Meta m, uint32_t *out) { decode(raw, m, out); }
 };
 
 struct FmtAffine8 {
@@ -79,6 +93,11 @@ struct FmtAffine8 {
                                                      int k0) {
         return FmtAffine4::load_meta(q, row_s, row_b, k0);
     }
+    __device__ static __forceinline__ void load_meta_raw(const QView &q, const uint8_t *row_s, const uint8_t *row_b,
+                                                         int k0, uint32_t *sb) {
+        FmtAffine4::load_meta_raw(q, row_s, row_b, k0, sb);
+    }
+    __device__ static __forceinline__ Meta meta_from_raw(const uint32_t *sb) { return FmtAffine4::meta_from_raw(sb); }
     __device__ static __forceinline__ void decode_word(uint32_t w, Meta m, uint32_t *out /*[2]*/) {
         out[0] = pack_bf16x2(fmaf((float)(w & 0xffu), m.s, m.b), fmaf((float)((w >> 8) & 0xffu), m.s, m.b));
         out[1] = pack_bf16x2(fmaf((float)((w >> 16) & 0xffu), m.s, m.b), fmaf((float)(w >> 24), m.s, m.b));
@@ -89,6 +108,7 @@ struct FmtAffine8 {
         decode_word(raw.z, m, out + 4);
         decode_word(raw.w, m, out + 6);
     }
+    __device__ static __forceinline__ void decode_fast(const uint4 &raw, Meta m, uint32_t *out) { decode(raw, m, out); }
 };
 
 struct FmtMxfp4 {
@@ -97,6 +117,17 @@ struct FmtMxfp4 {
     __device__ static __forceinline__ Meta load_meta(const QView &, const uint8_t *row_s, const uint8_t *, int k0) {
         Meta m;
         m.s = e8m0_to_f32(row_s[k0 >> 5]);
+        m.b = 0.0f;
+        return m;
+    }
+    __device__ static __forceinline__ void load_meta_raw(const QView &, const uint8_t *row_s, const uint8_t *, int k0,
+                                                         uint32_t *sb) {
+        sb[0] = row_s[k0 >> 5];
+        sb[1] = 0u;
+    }
+    __device__ static __forceinline__ Meta meta_from_raw(const uint32_t *sb) {
+        Meta m;
+        m.s = e8m0_to_f32(sb[0]);
         m.b = 0.0f;
         return m;
     }
@@ -114,12 +145,36 @@ struct FmtMxfp4 {
         decode_word(raw.z, m, out + 8);
         decode_word(raw.w, m, out + 12);
     }
+    // same values through the packed FP4 -> bf16 conversion (it scales by the exponent of `scale`)
+    __device__ static __forceinline__ void fast_word(uint32_t w, float scale, uint32_t *out /*[4]*/) {
+        out[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 0));
+        out[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 1));
+        out[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 2));
+        out[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 3));
+    }
+    __device__ static __forceinline__ void decode_fast(const uint4 &raw, Meta m, uint32_t *out /*[16]*/) {
+        fast_word(raw.x, m.s, out);
+        fast_word(raw.y, m.s, out + 4);
+        fast_word(raw.z, m.s, out + 8);
+        fast_word(raw.w, m.s, out + 12);
+    }
 };
 
 struct FmtFp8Row {
     static constexpr int kVals = 16;
     static constexpr bool kRowScale = true; // scales: one f32 per row, applied after the reduction
     __device__ static __forceinline__ Meta load_meta(const QView &, const uint8_t *, const uint8_t *, int) {
+        Meta m;
+        m.s = 1.0f;
+        m.b = 0.0f;
+        return m;
+    }
+    __device__ static __forceinline__ void load_meta_raw(const QView &, const uint8_t *, const uint8_t *, int,
+                                                         uint32_t *sb) {
+        sb[0] = 0u;
+        sb[1] = 0u;
+    }
+    __device__ static __forceinline__ Meta meta_from_raw(const uint32_t *) {
         Meta m;
         m.s = 1.0f;
         m.b = 0.0f;
@@ -134,6 +189,16 @@ struct FmtFp8Row {
         decode_word(raw.y, m, out + 2);
         decode_word(raw.z, m, out + 4);
         decode_word(raw.w, m, out + 6);
+    }
+    __device__ static __forceinline__ void fast_word(uint32_t w, uint32_t *out /*[2]*/) {
+        out[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false));
+        out[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true));
+    }
+    __device__ static __forceinline__ void decode_fast(const uint4 &raw, Meta, uint32_t *out /*[8]*/) {
+        fast_word(raw.x, out);
+        fast_word(raw.y, out + 2);
+        fast_word(raw.z, out + 4);
+        fast_word(raw.w, out + 6);
     }
 };
 

@@ -127,7 +127,7 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void qgemm_mfma_kernel(GemmArgs g)
         const int cur = ss & 1;
         uint32_t wp[NT][KV / 2];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) Fmt::decode(b_raw[nt], b_meta[nt], wp[nt]);
+        for (int nt = 0; nt < NT; ++nt) Fmt::decode_fast(b_raw[nt], b_meta[nt], wp[nt]);
         const bool more = ss + 1 < n_sub;
         if (more) {
             load_a(ss + 1);

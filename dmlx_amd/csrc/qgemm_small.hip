@@ -1,14 +1,18 @@
 // Grouped quantized GEMM, small-M path (decode): at most kSmallTileM rows per expert tile.
 //
 // The step is bound by streaming every live expert's packed weights once from HBM, so the layout is
-// built around the weight stream: one wavefront owns a run of output columns; for each column its 64
-// lanes read one contiguous 1 KiB piece of the packed row (16 bytes per lane), so every lane always
-// covers the SAME slice of the reduction dimension and keeps the matching activations of the tile's
-// rows in registers for the whole kernel. Products are formed with packed-bf16 dot instructions, f32
-// accumulation, and one cross-lane sum per output value.
+// built around the weight stream. A workgroup has four wavefronts; the reduction dimension is cut into
+// KS slices of 64 chunks (a chunk = 16 bytes of one packed row), one slice per wavefront, so a wavefront
+// reads one contiguous 1 KiB piece of a weight row per load instruction and every lane always covers
+// the SAME columns of the reduction dimension: the matching activations of the tile's rows are loaded
+// once and stay in registers. The 4 / KS wavefronts that share a slice take different output columns.
+// Loads run one batch of columns ahead of the arithmetic. Products are formed with packed-bf16 dot
+// instructions and f32 accumulation; the per-lane partial sums of a batch are reduced across the
+// wavefront with a transposing butterfly (V values cost V + 5 - log2 V shuffles instead of 6 V), the
+// slices meet in LDS, and the epilogue (row scale, SwiGLU, routing weight, bf16) stores coalesced rows.
 //
-// 4-bit affine weights are never multiplied out: codes are turned into the bf16 numbers (128 + q) with
-// one AND-OR per pair, and   sum_k x_k (q_k s + b) = s * sum_k x_k (128 + q_k) + (b - 128 s) * sum_k x_k
+// 4-bit affine weights are never multiplied out: codes become the bf16 numbers (128 + q) with one
+// AND-OR per pair, and   sum_k x_k (q_k s + b) = s * sum_k x_k (128 + q_k) + (b - 128 s) * sum_k x_k
 // is applied once per 32-value chunk.
 #include "common.h"
 #include "qformat.h"
@@ -16,14 +20,18 @@
 namespace dmoe {
 
 constexpr int kSmallWaves = 4;
-constexpr int kColsGateUp = 16; // output columns per wavefront (each needs a gate row and an up row)
-constexpr int kColsPlain = 32;
+constexpr int kColsGateUp = 32; // output columns per wavefront (each needs a gate row and an up row)
+constexpr int kColsPlain = 64;
+constexpr int kBatch = 2;       // columns per load batch
+constexpr int kStages = 4;      // batches in the load ring (kStages - 1 in flight ahead of the arithmetic)
+
+__device__ __forceinline__ uint32_t vgpr_const(uint32_t c);
 
 template <typename Fmt>
 struct SmallTraits {
     static constexpr bool kFactored = false;
     __device__ static __forceinline__ void unpack(const uint4 &raw, Meta m, uint32_t *pairs) {
-        Fmt::decode(raw, m, pairs);
+        Fmt::decode_fast(raw, m, pairs);
     }
     __device__ static __forceinline__ void arrange_x(uint32_t *) {}
 };
@@ -32,17 +40,18 @@ template <>
 struct SmallTraits<FmtAffine4> {
     static constexpr bool kFactored = true;
     // pairs (q_i, q_{i+4}) of each 8-code word as bf16 (128 + q)
-    __device__ static __forceinline__ void unpack_word(uint32_t w, uint32_t *o) {
-        o[0] = (w & 0x000f000fu) | 0x43004300u;
-        o[1] = ((w >> 4) & 0x000f000fu) | 0x43004300u;
-        o[2] = ((w >> 8) & 0x000f000fu) | 0x43004300u;
-        o[3] = ((w >> 12) & 0x000f000fu) | 0x43004300u;
+    __device__ static __forceinline__ void unpack_word(uint32_t w, uint32_t mask, uint32_t magic, uint32_t *o) {
+        o[0] = (w & mask) | magic;
+        o[1] = ((w >> 4) & mask) | magic;
+        o[2] = ((w >> 8) & mask) | magic;
+        o[3] = ((w >> 12) & mask) | magic;
     }
     __device__ static __forceinline__ void unpack(const uint4 &raw, Meta, uint32_t *pairs) {
-        unpack_word(raw.x, pairs);
-        unpack_word(raw.y, pairs + 4);
-        unpack_word(raw.z, pairs + 8);
-        unpack_word(raw.w, pairs + 12);
+        const uint32_t mask = vgpr_const(0x000f000fu), magic = vgpr_const(0x43004300u);
+        unpack_word(raw.x, mask, magic, pairs);
+        unpack_word(raw.y, mask, magic, pairs + 4);
+        unpack_word(raw.z, mask, magic, pairs + 8);
+        unpack_word(raw.w, mask, magic, pairs + 12);
     }
     // natural pairs (x0,x1)(x2,x3)(x4,x5)(x6,x7) -> (x0,x4)(x1,x5)(x2,x6)(x3,x7), per 8 values
     __device__ static __forceinline__ void arrange_x(uint32_t *x /*[16]*/) {
@@ -62,147 +71,211 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
                                            false);
 }
 
-template <typename Fmt, int ITERS, int NM>
-struct ColData {
-    uint4 raw[NM][ITERS];
-    Meta meta[NM][ITERS];
+// Sum V per-lane values over the 64 lanes; afterwards lane l holds the total of value (l mod V).
+template <int V>
+__device__ __forceinline__ float transpose_reduce(float (&v)[V], int lane) {
+    int n = V, bit = 1;
+#pragma unroll
+    for (int level = 0; level < 6; ++level) {
+        if (n > 1) {
+#pragma unroll
+            for (int i = 0; i < V / 2; ++i) {
+                if (i < n / 2) {
+                    const bool up = (lane & bit) != 0;
+                    float send = up ? v[2 * i] : v[2 * i + 1];
+                    float keep = up ? v[2 * i + 1] : v[2 * i];
+                    v[i] = keep + __shfl_xor(send, bit, 64);
+                }
+            }
+            n >>= 1;
+        } else {
+            v[0] += __shfl_xor(v[0], bit, 64);
+        }
+        bit <<= 1;
+    }
+    return v[0];
+}
+
+template <int NM>
+struct Batch {
+    uint4 raw[kBatch][NM];
+    uint32_t sb[kBatch][NM][2]; // raw scale / bias words (converted when the batch is consumed)
 };
 
-template <typename Fmt, int ITERS, bool GATE_UP, int M>
-__device__ __forceinline__ void small_run(const GemmArgs &g, const Tile &t, int wave, int lane) {
-    using ST = SmallTraits<Fmt>;
-    constexpr int NP = Fmt::kVals / 2;       // packed pairs per chunk
-    constexpr int KSTEP = 64 * Fmt::kVals;   // reduction elements one wavefront covers per iteration
-    constexpr int NM = GATE_UP ? 2 : 1;
-    constexpr int CPW = GATE_UP ? kColsGateUp : kColsPlain;
-    const int cols = g.b0.cols;
-    const int n_out = g.b0.rows;
+// a 32-bit constant the compiler must keep in a vector register (VOP3 on gfx9 reads one scalar at most,
+// so "(w & mask) | magic" only becomes a single v_and_or_b32 when the constants are vector operands)
+__device__ __forceinline__ uint32_t vgpr_const(uint32_t c) {
+    uint32_t v;
+    asm volatile("v_mov_b32 %0, %1" : "=v"(v) : "s"(c));
+    return v;
+}
 
-    // ---- activations of the tile's rows, this lane's slices, kept in registers -------------------
-    uint32_t xp[M][ITERS][NP];
-    float xs[M][ITERS];
+template <typename Fmt, int KS, bool GATE_UP, int M>
+__device__ __forceinline__ void small_run(const GemmArgs &g, const Tile &t, float *part) {
+    using ST = SmallTraits<Fmt>;
+    constexpr int NP = Fmt::kVals / 2;          // packed pairs per chunk
+    constexpr int NM = GATE_UP ? 2 : 1;
+    constexpr int CG = kSmallWaves / KS;        // wavefronts (column groups) per slice
+    constexpr int CPW = GATE_UP ? kColsGateUp : kColsPlain;
+    constexpr int CPB = CG * CPW;               // output columns per workgroup
+    constexpr int NB = CPW / kBatch;            // batches per wavefront
+    constexpr int MP = M == 3 ? 4 : M;          // rows padded to a power of two for the butterfly
+    constexpr int V = kBatch * NM * MP;
+    const int tid = (int)threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // wave-uniform: keeps addressing scalar
+    const int slice = wave % KS, cg = wave / KS;
+    const int cols = g.b0.cols, n_out = g.b0.rows;
+    const int k0 = (slice * 64 + lane) * Fmt::kVals;   // first reduction element of this lane's chunk
+    const bool k_on = k0 < cols;
+    // lanes past the end of the row read chunk 0 instead (valid memory) and multiply it by zero activations
+    const uint32_t w_off = k_on ? (uint32_t)(slice * 64 + lane) * 16u : 0u;
+    const int k_meta = k_on ? k0 : 0;
+
+    const size_t e = t.expert;
+    const int block_col0 = (int)blockIdx.x * CPB;
+    const int wave_col0 = block_col0 + cg * CPW;
+    // scalar bases of this expert's matrices; per-column offsets are added as scalars too
+    const uint8_t *wbase[NM], *sbase[NM], *bbase[NM];
+#pragma unroll
+    for (int mi = 0; mi < NM; ++mi) {
+        const QView &q = mi == 0 ? g.b0 : g.b1;
+        wbase[mi] = q.w + e * q.w_mat;
+        sbase[mi] = q.scales + e * q.s_mat;
+        bbase[mi] = q.biases ? q.biases + e * q.s_mat : nullptr;
+    }
+
+    auto load_batch = [&](int n0, Batch<NM> &b) {
+#pragma unroll
+        for (int c = 0; c < kBatch; ++c) {
+            int n = n0 + c;
+            if (n >= n_out) n = n_out - 1; // stay inside the matrix; such columns are never stored
+#pragma unroll
+            for (int mi = 0; mi < NM; ++mi) {
+                const QView &q = mi == 0 ? g.b0 : g.b1;
+                b.raw[c][mi] = *(const uint4 *)(wbase[mi] + (size_t)n * q.w_row + w_off);
+                Fmt::load_meta_raw(q, sbase[mi] + (size_t)n * q.s_row,
+                                   bbase[mi] ? bbase[mi] + (size_t)n * q.s_row : nullptr, k_meta, b.sb[c][mi]);
+            }
+        }
+    };
+
+    Batch<NM> ring[kStages];
+    const bool wave_on = wave_col0 < n_out;
+    if (wave_on) {
+#pragma unroll
+        for (int j = 0; j < kStages - 1; ++j)
+            if (j < NB) load_batch(wave_col0 + j * kBatch, ring[j]);
+    }
+
+    // ---- activations of the tile's rows: this lane's chunk, kept in registers ---------------------------
+    // (issued after the first weight loads, which depend on the tile only, so both latencies overlap)
+    uint32_t xp[M][NP];
+    float xs[M];
 #pragma unroll
     for (int r = 0; r < M; ++r) {
         const uint32_t p = t.row0 + (uint32_t)r;
         const size_t src = g.a_rows ? g.a_rows[p] : p;
         const uint16_t *xrow = g.a + src * (size_t)cols;
 #pragma unroll
-        for (int it = 0; it < ITERS; ++it) {
-            const int k0 = it * KSTEP + lane * Fmt::kVals;
-            float sum = 0.0f;
-#pragma unroll
-            for (int v = 0; v < NP / 4; ++v) {
-                uint4 q = make_uint4(0, 0, 0, 0);
-                if (k0 < cols) q = *(const uint4 *)(xrow + k0 + 8 * v);
-                xp[r][it][4 * v] = q.x;
-                xp[r][it][4 * v + 1] = q.y;
-                xp[r][it][4 * v + 2] = q.z;
-                xp[r][it][4 * v + 3] = q.w;
-            }
-            if (ST::kFactored) {
-#pragma unroll
-                for (int i = 0; i < NP; ++i)
-                    sum += bf16_bits_to_f32(xp[r][it][i] & 0xffffu) + bf16_bits_to_f32(xp[r][it][i] >> 16);
-            }
-            xs[r][it] = sum;
-            ST::arrange_x(xp[r][it]);
+        for (int v = 0; v < NP / 4; ++v) {
+            uint4 q = make_uint4(0, 0, 0, 0);
+            if (k_on) q = *(const uint4 *)(xrow + k0 + 8 * v);
+            xp[r][4 * v] = q.x;
+            xp[r][4 * v + 1] = q.y;
+            xp[r][4 * v + 2] = q.z;
+            xp[r][4 * v + 3] = q.w;
         }
+        float sum = 0.0f;
+        if (ST::kFactored) {
+#pragma unroll
+            for (int i = 0; i < NP; ++i) sum = dot2_bf16(xp[r][i], 0x3f803f80u, sum); // x . (1, 1)
+        }
+        xs[r] = sum;
+        ST::arrange_x(xp[r]);
     }
 
-    const size_t e = t.expert;
-    const int n_base = ((int)blockIdx.x * kSmallWaves + wave) * CPW;
-
-    auto load_col = [&](int n, ColData<Fmt, ITERS, NM> &c) {
+    auto compute_batch = [&](int col_in_wave, const Batch<NM> &b) {
+        float v[V];
 #pragma unroll
-        for (int mi = 0; mi < NM; ++mi) {
-            const QView &b = mi == 0 ? g.b0 : g.b1;
-            const uint8_t *wrow = b.w + e * b.w_mat + (size_t)n * b.w_row;
-            const uint8_t *srow = b.scales + e * b.s_mat + (size_t)n * b.s_row;
-            const uint8_t *brow = b.biases ? b.biases + e * b.s_mat + (size_t)n * b.s_row : nullptr;
+        for (int c = 0; c < kBatch; ++c) {
 #pragma unroll
-            for (int it = 0; it < ITERS; ++it) {
-                const int k0 = it * KSTEP + lane * Fmt::kVals;
-                if (k0 < cols) {
-                    c.raw[mi][it] = *(const uint4 *)(wrow + (size_t)(it * 64 + lane) * 16);
-                    c.meta[mi][it] = Fmt::load_meta(b, srow, brow, k0);
-                } else {
-                    c.raw[mi][it] = make_uint4(0, 0, 0, 0);
-                    c.meta[mi][it].s = 0.0f;
-                    c.meta[mi][it].b = 0.0f;
-                }
-            }
-        }
-    };
-
-    auto compute_col = [&](int n, const ColData<Fmt, ITERS, NM> &c) {
-        float acc[NM][M];
-#pragma unroll
-        for (int mi = 0; mi < NM; ++mi)
-#pragma unroll
-            for (int r = 0; r < M; ++r) acc[mi][r] = 0.0f;
-#pragma unroll
-        for (int mi = 0; mi < NM; ++mi) {
-#pragma unroll
-            for (int it = 0; it < ITERS; ++it) {
+            for (int mi = 0; mi < NM; ++mi) {
                 uint32_t pairs[NP];
-                ST::unpack(c.raw[mi][it], c.meta[mi][it], pairs);
-                const float s = c.meta[mi][it].s;
-                const float boff = fmaf(-128.0f, s, c.meta[mi][it].b);
+                const Meta meta = Fmt::meta_from_raw(b.sb[c][mi]);
+                ST::unpack(b.raw[c][mi], meta, pairs);
+                const float s = meta.s;
+                const float boff = fmaf(-128.0f, s, meta.b);
 #pragma unroll
-                for (int r = 0; r < M; ++r) {
-                    float p0 = 0.0f, p1 = 0.0f; // two chains for instruction-level parallelism
+                for (int r = 0; r < MP; ++r) {
+                    float val = 0.0f;
+                    if (r < M) {
+                        float p0 = 0.0f, p1 = 0.0f; // two chains for instruction-level parallelism
 #pragma unroll
-                    for (int i = 0; i < NP; i += 2) {
-                        p0 = dot2_bf16(pairs[i], xp[r][it][i], p0);
-                        p1 = dot2_bf16(pairs[i + 1], xp[r][it][i + 1], p1);
+                        for (int i = 0; i < NP; i += 2) {
+                            p0 = dot2_bf16(pairs[i], xp[r][i], p0);
+                            p1 = dot2_bf16(pairs[i + 1], xp[r][i + 1], p1);
+                        }
+                        val = ST::kFactored ? fmaf(s, p0 + p1, boff * xs[r]) : p0 + p1;
                     }
-                    if (ST::kFactored) acc[mi][r] = fmaf(s, p0 + p1, fmaf(boff, xs[r][it], acc[mi][r]));
-                    else acc[mi][r] += p0 + p1;
+                    v[(c * NM + mi) * MP + r] = val;
                 }
             }
         }
-#pragma unroll
-        for (int mi = 0; mi < NM; ++mi) {
-            float rs = 1.0f;
-            if (Fmt::kRowScale) {
-                const QView &b = mi == 0 ? g.b0 : g.b1;
-                rs = *(const float *)(b.scales + e * b.s_mat + (size_t)n * b.s_row);
-            }
-#pragma unroll
-            for (int r = 0; r < M; ++r) acc[mi][r] = wave_sum(acc[mi][r]) * rs;
-        }
-#pragma unroll
-        for (int r = 0; r < M; ++r) {
-            if (lane == r) {
-                const uint32_t p = t.row0 + (uint32_t)r;
-                float v = GATE_UP ? limited_swiglu(acc[0][r], acc[NM - 1][r], g.swiglu_limit) : acc[0][r];
-                if (g.row_scale) v *= g.row_scale[g.row_scale_idx ? g.row_scale_idx[p] : p];
-                const size_t dst = g.out_rows ? g.out_rows[p] : p;
-                g.out[dst * (size_t)g.ldo + n] = f32_to_bf16_bits(v);
-            }
+        float tot = transpose_reduce<V>(v, lane);
+        if (lane < V) {
+            const int r = lane % MP, mi = (lane / MP) % NM, c = lane / (MP * NM);
+            if (r < M) part[((slice * CPB + cg * CPW + col_in_wave + c) * NM + mi) * 4 + r] = tot;
         }
     };
 
-    ColData<Fmt, ITERS, NM> cur, nxt;
-    if (n_base < n_out) load_col(n_base, cur);
-#pragma unroll 2
-    for (int c = 0; c < CPW; ++c) {
-        const int n = n_base + c;
-        if (n >= n_out) break;
-        const bool more = (c + 1 < CPW) && (n + 1 < n_out);
-        if (more) load_col(n + 1, nxt);
-        compute_col(n, cur);
-        if (more) cur = nxt;
+    // software pipeline over the batches of this wavefront: kStages - 1 batches of loads stay in flight
+    // while one is consumed; the ring indices are compile-time constants
+#pragma unroll 1
+    for (int b0 = 0; b0 < NB; b0 += kStages) {
+#pragma unroll
+        for (int j = 0; j < kStages; ++j) {
+            const int b = b0 + j;
+            if (wave_on && b + kStages - 1 < NB)
+                load_batch(wave_col0 + (b + kStages - 1) * kBatch, ring[(j + kStages - 1) % kStages]);
+            if (wave_on && b < NB && wave_col0 + b * kBatch < n_out) compute_batch(b * kBatch, ring[j]);
+        }
+    }
+    __syncthreads();
+
+    // ---- epilogue: add the slices, scale, activate, store rows of consecutive columns ----------------
+    for (int i = tid; i < CPB * M; i += kSmallWaves * 64) {
+        const int col = i % CPB, r = i / CPB;
+        const int n = block_col0 + col;
+        if (n >= n_out) continue;
+        float acc[NM];
+#pragma unroll
+        for (int mi = 0; mi < NM; ++mi) {
+            float a = 0.0f;
+#pragma unroll
+            for (int sl = 0; sl < KS; ++sl) a += part[((sl * CPB + col) * NM + mi) * 4 + r];
+            if (Fmt::kRowScale) {
+                const QView &q = mi == 0 ? g.b0 : g.b1;
+                a *= *(const float *)(q.scales + e * q.s_mat + (size_t)n * q.s_row);
+            }
+            acc[mi] = a;
+        }
+        const uint32_t p = t.row0 + (uint32_t)r;
+        float val = GATE_UP ? limited_swiglu(acc[0], acc[NM - 1], g.swiglu_limit) : acc[0];
+        if (g.row_scale) val *= g.row_scale[g.row_scale_idx ? g.row_scale_idx[p] : p];
+        const size_t dst = g.out_rows ? g.out_rows[p] : p;
+        g.out[dst * (size_t)g.ldo + n] = f32_to_bf16_bits(val);
     }
 }
 
-template <typename Fmt, int ITERS, bool GATE_UP>
+template <typename Fmt, int KS, bool GATE_UP>
 __global__ __launch_bounds__(kSmallWaves * 64) void qgemm_small_kernel(GemmArgs g) {
+    __shared__ float part[2048];
     Tile t;
     const uint32_t slot = blockIdx.y;
     if (g.tiles) {
-        if (slot >= *g.n_tiles) return;
-        t = g.tiles[slot];
+        const uint32_t n_tiles = *g.n_tiles; // both loads are issued before either is needed
+        t = g.tiles[slot];                   // the list has room for every launched slot
+        if (slot >= n_tiles) return;
     } else {
         t.expert = 0;
         t.row0 = slot * (uint32_t)kSmallTileM;
@@ -211,42 +284,45 @@ __global__ __launch_bounds__(kSmallWaves * 64) void qgemm_small_kernel(GemmArgs 
         t.nrows = left < (uint32_t)kSmallTileM ? left : (uint32_t)kSmallTileM;
         t.pad = 0;
     }
-    const int wave = (int)(threadIdx.x >> 6), lane = lane_id();
-    switch (t.nrows) {
-    case 1: small_run<Fmt, ITERS, GATE_UP, 1>(g, t, wave, lane); break;
-    case 2: small_run<Fmt, ITERS, GATE_UP, 2>(g, t, wave, lane); break;
-    case 3: small_run<Fmt, ITERS, GATE_UP, 3>(g, t, wave, lane); break;
-    case 4: small_run<Fmt, ITERS, GATE_UP, 4>(g, t, wave, lane); break;
+    switch (t.nrows) { // uniform over the workgroup
+    case 1: small_run<Fmt, KS, GATE_UP, 1>(g, t, part); break;
+    case 2: small_run<Fmt, KS, GATE_UP, 2>(g, t, part); break;
+    case 3: small_run<Fmt, KS, GATE_UP, 3>(g, t, part); break;
+    case 4: small_run<Fmt, KS, GATE_UP, 4>(g, t, part); break;
     default: break;
     }
 }
 
-static int small_iters(const QView &b, int vals) { return ceil_div(b.cols, 64 * vals); }
+static int small_slices(const QView &b, int vals) {
+    int s = ceil_div(b.cols, 64 * vals);
+    return s <= 1 ? 1 : (s == 2 ? 2 : (s <= 4 ? 4 : 0));
+}
 
 bool qgemm_small_supports(const QView &b) {
     int vals = (b.mode == DMOE_QUANT_AFFINE && b.bits == 4) || b.mode == DMOE_QUANT_MXFP4 ? 32 : 16;
-    int it = small_iters(b, vals);
-    return b.cols % vals == 0 && (it == 1 || it == 2 || (vals == 16 && it <= 4));
+    return b.cols % vals == 0 && small_slices(b, vals) != 0;
 }
 
 struct SmallLaunch {
     const GemmArgs &g;
     hipStream_t st;
-    template <typename Fmt, int ITERS>
+    template <typename Fmt, int KS>
     int go() {
-        const int cpw = g.gate_up ? kColsGateUp : kColsPlain;
-        dim3 grid((unsigned)ceil_div(g.b0.rows, kSmallWaves * cpw), (unsigned)g.max_tiles), block(kSmallWaves * 64);
-        if (g.gate_up) hipLaunchKernelGGL((qgemm_small_kernel<Fmt, ITERS, true>), grid, block, 0, st, g);
-        else hipLaunchKernelGGL((qgemm_small_kernel<Fmt, ITERS, false>), grid, block, 0, st, g);
+        const int cpb = (kSmallWaves / KS) * (g.gate_up ? kColsGateUp : kColsPlain);
+        dim3 grid((unsigned)ceil_div(g.b0.rows, cpb), (unsigned)g.max_tiles), block(kSmallWaves * 64);
+        if (g.gate_up) hipLaunchKernelGGL((qgemm_small_kernel<Fmt, KS, true>), grid, block, 0, st, g);
+        else hipLaunchKernelGGL((qgemm_small_kernel<Fmt, KS, false>), grid, block, 0, st, g);
         DMOE_LAUNCH_CHECK();
         return DMOE_OK;
     }
     template <typename Fmt>
     int operator()() {
-        int it = small_iters(g.b0, Fmt::kVals);
-        if (it == 1) return go<Fmt, 1>();
-        if (it == 2) return go<Fmt, 2>();
-        if (Fmt::kVals == 16 && it <= 4) return go<Fmt, (Fmt::kVals == 16 ? 4 : 2)>();
+        switch (small_slices(g.b0, Fmt::kVals)) {
+        case 1: return go<Fmt, 1>();
+        case 2: return go<Fmt, 2>();
+        case 4: return go<Fmt, 4>();
+        default: break;
+        }
         set_error("small-M GEMM: reduction length %d not supported", g.b0.cols);
         return DMOE_ERR_UNSUPPORTED;
     }
