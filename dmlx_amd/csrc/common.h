@@ -111,7 +111,18 @@ struct QView { // device view of one dmoe_qweight stack
     size_t w_row = 0, s_row = 0;   // bytes between consecutive rows
     int rows = 0, cols = 0, n_mats = 0;
     int mode = 0, bits = 4, group = 64;
+    // packed (resident) layout, see qformat.h: w holds the re-ordered chunks, meta the interleaved
+    // scale/bias words (affine) or exponents (mxfp4); scales still holds the per-row f32 scales of fp8row
+    bool packed = false;
+    const uint8_t *meta = nullptr;
+    size_t m_mat = 0;
 };
+// bytes of the packed copies of a stack (rows must be a multiple of 32)
+size_t packed_w_bytes(const QView &v);
+size_t packed_meta_bytes(const QView &v);
+bool can_pack(const QView &v);
+// d_w / d_meta receive the packed layout of the MLX-layout stack `src` (all device memory)
+int launch_repack(void *d_w, void *d_meta, const QView &src, hipStream_t st);
 int make_qview(QView *out, const dmoe_qweight *q, const char *name);
 size_t qweight_w_bytes(const dmoe_qweight *q);
 size_t qweight_s_bytes(const dmoe_qweight *q);
@@ -134,11 +145,11 @@ struct GemmArgs {
     float swiglu_limit = 0.0f;
 };
 // tile_m the kernels were built for
-constexpr int kSmallTileM = 4;
+constexpr int kSkinnyTileM = 8;
 constexpr int kMfmaTileM = 128;
-int launch_qgemm_small(const GemmArgs &g, hipStream_t st);
+int launch_qgemm_skinny(const GemmArgs &g, hipStream_t st);
 int launch_qgemm_mfma(const GemmArgs &g, hipStream_t st);
-bool qgemm_small_supports(const QView &b);
+bool qgemm_skinny_supports(const QView &b);
 bool qgemm_mfma_supports(const QView &b);
 
 } // namespace dmoe

@@ -10,9 +10,9 @@
 namespace dmoe {
 
 struct QOwned {
-    dmoe_qweight q;        // device pointers
-    void *own[3] = {nullptr, nullptr, nullptr};
-    QView view;
+    dmoe_qweight q;        // device pointers (MLX layout) while the layer is being built
+    void *own[5] = {nullptr, nullptr, nullptr, nullptr, nullptr}; // w, scales, biases (MLX layout); packed w, packed meta
+    QView view;            // what the kernels read: the packed layout whenever the shape allows it
 };
 
 struct Layer {
@@ -66,7 +66,28 @@ static int adopt(QOwned *dst, const dmoe_qweight *src, int source, const char *n
         dst->q.scales = dst->own[1];
         dst->q.biases = dst->own[2];
     }
-    return make_qview(&dst->view, &dst->q, name);
+    DMOE_TRY(make_qview(&dst->view, &dst->q, name));
+    if (!can_pack(dst->view)) return DMOE_OK; // odd shapes stay in the MLX layout (slower addressing, same results)
+    // resident layout: re-order once so that every wavefront streams its 32 weight rows linearly
+    const size_t wb = packed_w_bytes(dst->view), mb = packed_meta_bytes(dst->view);
+    DMOE_HIP(hipMalloc(&dst->own[3], wb));
+    if (mb) DMOE_HIP(hipMalloc(&dst->own[4], mb));
+    DMOE_TRY(launch_repack(dst->own[3], dst->own[4], dst->view, st));
+    DMOE_HIP(hipStreamSynchronize(st));
+    // the MLX-layout copies are no longer needed (fp8 keeps its per-row scales)
+    const bool keep_scales = dst->view.mode == DMOE_QUANT_FP8_ROW;
+    for (int i = 0; i < 3; ++i) {
+        if (i == 1 && keep_scales) continue;
+        if (dst->own[i]) DMOE_HIP(hipFree(dst->own[i]));
+        dst->own[i] = nullptr;
+    }
+    dst->view.packed = true;
+    dst->view.w = (const uint8_t *)dst->own[3];
+    dst->view.meta = (const uint8_t *)dst->own[4];
+    dst->view.m_mat = mb / (size_t)dst->view.n_mats;
+    if (!keep_scales) dst->view.scales = nullptr;
+    dst->view.biases = nullptr;
+    return DMOE_OK;
 }
 
 // ---- small kernels ----------------------------------------------------------------------------------
@@ -124,12 +145,12 @@ __global__ void combine_kernel(uint16_t *__restrict__ out, const uint16_t *__res
 
 // ---- forward -------------------------------------------------------------------------------------------
 
-// average rows per expert at or below this run on the small-M path
-constexpr int kSmallAvgRows = 4;
-constexpr int kSharedSmallRows = 64;
+// at or below this many rows per expert on average the skinny (weight-streaming) kernel runs every tile
+constexpr int kSkinnyAvgRows = 8;
+constexpr int kSharedSkinnyRows = 64;
 
 static bool use_small_path(size_t rows, int n_experts, const QView &b) {
-    return qgemm_small_supports(b) && rows <= (size_t)kSmallAvgRows * (size_t)n_experts;
+    return qgemm_skinny_supports(b) && rows <= (size_t)kSkinnyAvgRows * (size_t)n_experts;
 }
 
 struct FwdLayout {
@@ -143,8 +164,8 @@ static FwdLayout forward_layout(const Layer *L, int T) {
     FwdLayout f;
     Bump b;
     size_t n = (size_t)T * L->K;
-    f.small = use_small_path(n, L->E, L->gate.view) && qgemm_small_supports(L->down.view);
-    f.tile_m = f.small ? kSmallTileM : kMfmaTileM;
+    f.small = use_small_path(n, L->E, L->gate.view) && qgemm_skinny_supports(L->down.view);
+    f.tile_m = f.small ? kSkinnyTileM : kMfmaTileM;
     f.max_tiles = pack_max_tiles(n, L->E, f.tile_m);
     f.slot_idx = b.take(n * 4);
     f.order = b.take(n * 4);
@@ -167,7 +188,7 @@ static FwdLayout forward_layout(const Layer *L, int T) {
 }
 
 static int run_gemm(const GemmArgs &g, bool small, hipStream_t st) {
-    return small ? launch_qgemm_small(g, st) : launch_qgemm_mfma(g, st);
+    return small ? launch_qgemm_skinny(g, st) : launch_qgemm_mfma(g, st);
 }
 
 // routed experts on slot ids: fills ws->y ([T*K, D] bf16 in flat (t,k) order) or `y_out` when given
@@ -225,10 +246,10 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
 
 static int shared_forward(const Layer *L, Workspace *w, const FwdLayout &f, const uint16_t *d_x, int T,
                           hipStream_t st) {
-    // up to 64 rows the dense expert is streamed by the small-M kernel in 4-row tiles (many workgroups per
-    // weight row block); above that the MFMA kernel amortises the dequantization
-    const bool small = T <= kSharedSmallRows && qgemm_small_supports(L->sgate.view) && qgemm_small_supports(L->sdown.view);
-    const int tile_m = small ? kSmallTileM : kMfmaTileM;
+    // up to 64 rows the dense expert is streamed by the skinny kernel in 8-row tiles (many workgroups per
+    // block of weight rows); above that the big-tile kernel amortises the dequantization
+    const bool small = T <= kSharedSkinnyRows && qgemm_skinny_supports(L->sgate.view) && qgemm_skinny_supports(L->sdown.view);
+    const int tile_m = small ? kSkinnyTileM : kMfmaTileM;
     GemmArgs gu;
     gu.b0 = L->sgate.view;
     gu.b1 = L->sup.view;
@@ -438,7 +459,7 @@ int dmoe_gather_qmm(uint16_t *d_out, const uint16_t *d_x, const dmoe_qweight *qw
     hipStream_t st = to_hip(s);
     const bool small = use_small_path((size_t)R, v.n_mats, v);
     DMOE_REQUIRE(small || qgemm_mfma_supports(v), "gather_qmm: unsupported weight shape rows=%d cols=%d", v.rows, v.cols);
-    const int tile_m = small ? kSmallTileM : kMfmaTileM;
+    const int tile_m = small ? kSkinnyTileM : kMfmaTileM;
     const int max_tiles = pack_max_tiles((size_t)R, v.n_mats, tile_m);
     Bump b;
     size_t o_order = b.take((size_t)R * 4), o_arows = b.take((size_t)R * 4);

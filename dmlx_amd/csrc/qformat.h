@@ -3,6 +3,18 @@
 // Every format is read in 16-byte pieces ("chunks"): kVals values of one weight row that share one
 // scale (and bias). Value i of a chunk is element (k0 + i) of the row, so pairs (2p, 2p+1) are adjacent
 // along the reduction dimension.
+//
+// Two memory layouts exist for a stack of matrices:
+//   MLX layout     rows are contiguous ([n, rows, cols*bits/32] u32 words), scales/biases per row.
+//   packed layout  the resident layout of a dmoe_layer, built once at upload for the matrix-core
+//                  kernels. Rows are taken in blocks of 32 and the reduction dimension in steps of
+//                  two chunks; the 1 KiB that one wavefront consumes per step is contiguous:
+//                      chunk (row = 32*nb + ln, step, h)  ->  16 bytes at
+//                      w + mat*w_mat + (((nb*n_steps + step)*2 + h)*32 + ln) * 16
+//                  so a wavefront streams its 32 rows as one linear run of memory. Scales and biases
+//                  are interleaved the same way: affine {scale | bias << 16} words at
+//                      meta + mat*m_mat + ((nb*n_groups + g)*32 + ln) * 4
+//                  and MXFP4 exponents (one per chunk) at meta + mat*m_mat + ((nb*n_steps+step)*2+h)*32 + ln.
 #pragma once
 
 #include "common.h"
@@ -37,10 +49,13 @@ __device__ __forceinline__ float e4m3_to_f32(uint32_t v) {
 }
 
 // ---- per-chunk decoders -------------------------------------------------------------------------------
-// Fmt::kVals                         values per 16-byte chunk
-// Fmt::load_meta(b, row_s, row_b, k0) scale/bias of the chunk starting at column k0 (f32 pair)
-// Fmt::decode(raw, meta, out)        kVals/2 packed bf16 pairs, natural order, fully dequantized
-// Fmt::kRowScale                     true: an f32 per-row scale is applied to the finished dot product
+// Fmt::kVals                          values per 16-byte chunk
+// Fmt::kRowScale                      true: an f32 per-row scale is applied to the finished dot product
+// Fmt::load_meta(q, row_s, row_b, k0) scale/bias of the chunk starting at column k0 (MLX layout)
+// Fmt::load_meta_raw / meta_from_raw  the same in two steps: raw words while a load is in flight, f32 at use
+// Fmt::load_meta_packed / meta_from_packed   raw word(s) from the packed layout
+// Fmt::decode(raw, meta, out)         kVals/2 packed bf16 pairs, natural order, exact per-format arithmetic
+// Fmt::decode_fast                    same values through the gfx950 packed conversion instructions
 
 struct Meta {
     float s, b;
@@ -49,26 +64,34 @@ struct Meta {
 struct FmtAffine4 {
     static constexpr int kVals = 32;
     static constexpr bool kRowScale = false;
-    __device__ static __forceinline__ Meta load_meta(const QView &q, const uint8_t *row_s, const uint8_t *row_b,
-                                                     int k0) {
-        int g = k0 / q.group;
-        Meta m;
-        m.s = bf16_bits_to_f32(((const uint16_t *)row_s)[g]);
-        m.b = row_b ? bf16_bits_to_f32(((const uint16_t *)row_b)[g]) : 0.0f;
-        return m;
-    }
-    // the same two values as raw 16-bit words (kept unconverted while a load is in flight)
     __device__ static __forceinline__ void load_meta_raw(const QView &q, const uint8_t *row_s, const uint8_t *row_b,
                                                          int k0, uint32_t *sb) {
         int g = k0 / q.group;
         sb[0] = ((const uint16_t *)row_s)[g];
         sb[1] = row_b ? ((const uint16_t *)row_b)[g] : 0u;
     }
+    __device__ static __forceinline__ void load_meta_packed(const QView &q, size_t mat, int nb, int step, int h,
+                                                            int ln, uint32_t *sb) {
+        const int g = (step * 2 + h) * kVals / q.group, n_groups = q.cols / q.group;
+        sb[0] = *(const uint32_t *)(q.meta + mat * q.m_mat + (((size_t)nb * n_groups + g) * 32 + ln) * 4);
+    }
     __device__ static __forceinline__ Meta meta_from_raw(const uint32_t *sb) {
         Meta m;
         m.s = bf16_bits_to_f32(sb[0]);
         m.b = bf16_bits_to_f32(sb[1]);
         return m;
+    }
+    __device__ static __forceinline__ Meta meta_from_packed(const uint32_t *sb) {
+        Meta m;
+        m.s = __uint_as_float(sb[0] << 16);
+        m.b = __uint_as_float(sb[0] & 0xffff0000u);
+        return m;
+    }
+    __device__ static __forceinline__ Meta load_meta(const QView &q, const uint8_t *row_s, const uint8_t *row_b,
+                                                     int k0) {
+        uint32_t sb[2];
+        load_meta_raw(q, row_s, row_b, k0, sb);
+        return meta_from_raw(sb);
     }
     __device__ static __forceinline__ void decode_word(uint32_t w, Meta m, uint32_t *out /*[4]*/) {
         uint32_t lo = w & 0x0f0f0f0fu, hi = (w >> 4) & 0x0f0f0f0fu; // nibbles 0,2,4,6 / 1,3,5,7 as bytes
@@ -89,15 +112,21 @@ struct FmtAffine4 {
 struct FmtAffine8 {
     static constexpr int kVals = 16;
     static constexpr bool kRowScale = false;
-    __device__ static __forceinline__ Meta load_meta(const QView &q, const uint8_t *row_s, const uint8_t *row_b,
-                                                     int k0) {
-        return FmtAffine4::load_meta(q, row_s, row_b, k0);
-    }
     __device__ static __forceinline__ void load_meta_raw(const QView &q, const uint8_t *row_s, const uint8_t *row_b,
                                                          int k0, uint32_t *sb) {
         FmtAffine4::load_meta_raw(q, row_s, row_b, k0, sb);
     }
+    __device__ static __forceinline__ void load_meta_packed(const QView &q, size_t mat, int nb, int step, int h,
+                                                            int ln, uint32_t *sb) {
+        const int g = (step * 2 + h) * kVals / q.group, n_groups = q.cols / q.group;
+        sb[0] = *(const uint32_t *)(q.meta + mat * q.m_mat + (((size_t)nb * n_groups + g) * 32 + ln) * 4);
+    }
     __device__ static __forceinline__ Meta meta_from_raw(const uint32_t *sb) { return FmtAffine4::meta_from_raw(sb); }
+    __device__ static __forceinline__ Meta meta_from_packed(const uint32_t *sb) { return FmtAffine4::meta_from_packed(sb); }
+    __device__ static __forceinline__ Meta load_meta(const QView &q, const uint8_t *row_s, const uint8_t *row_b,
+                                                     int k0) {
+        return FmtAffine4::load_meta(q, row_s, row_b, k0);
+    }
     __device__ static __forceinline__ void decode_word(uint32_t w, Meta m, uint32_t *out /*[2]*/) {
         out[0] = pack_bf16x2(fmaf((float)(w & 0xffu), m.s, m.b), fmaf((float)((w >> 8) & 0xffu), m.s, m.b));
         out[1] = pack_bf16x2(fmaf((float)((w >> 16) & 0xffu), m.s, m.b), fmaf((float)(w >> 24), m.s, m.b));
@@ -114,22 +143,28 @@ struct FmtAffine8 {
 struct FmtMxfp4 {
     static constexpr int kVals = 32;
     static constexpr bool kRowScale = false;
-    __device__ static __forceinline__ Meta load_meta(const QView &, const uint8_t *row_s, const uint8_t *, int k0) {
-        Meta m;
-        m.s = e8m0_to_f32(row_s[k0 >> 5]);
-        m.b = 0.0f;
-        return m;
-    }
     __device__ static __forceinline__ void load_meta_raw(const QView &, const uint8_t *row_s, const uint8_t *, int k0,
                                                          uint32_t *sb) {
         sb[0] = row_s[k0 >> 5];
         sb[1] = 0u;
+    }
+    __device__ static __forceinline__ void load_meta_packed(const QView &q, size_t mat, int nb, int step, int h,
+                                                            int ln, uint32_t *sb) {
+        const int n_steps = q.cols / (2 * kVals);
+        sb[0] = q.meta[mat * q.m_mat + (((size_t)nb * n_steps + step) * 2 + h) * 32 + ln];
     }
     __device__ static __forceinline__ Meta meta_from_raw(const uint32_t *sb) {
         Meta m;
         m.s = e8m0_to_f32(sb[0]);
         m.b = 0.0f;
         return m;
+    }
+    __device__ static __forceinline__ Meta meta_from_packed(const uint32_t *sb) { return meta_from_raw(sb); }
+    __device__ static __forceinline__ Meta load_meta(const QView &q, const uint8_t *row_s, const uint8_t *row_b,
+                                                     int k0) {
+        uint32_t sb[2];
+        load_meta_raw(q, row_s, row_b, k0, sb);
+        return meta_from_raw(sb);
     }
     __device__ static __forceinline__ void decode_word(uint32_t w, Meta m, uint32_t *out /*[4]*/) {
 #pragma unroll
@@ -163,22 +198,23 @@ struct FmtMxfp4 {
 struct FmtFp8Row {
     static constexpr int kVals = 16;
     static constexpr bool kRowScale = true; // scales: one f32 per row, applied after the reduction
-    __device__ static __forceinline__ Meta load_meta(const QView &, const uint8_t *, const uint8_t *, int) {
-        Meta m;
-        m.s = 1.0f;
-        m.b = 0.0f;
-        return m;
-    }
     __device__ static __forceinline__ void load_meta_raw(const QView &, const uint8_t *, const uint8_t *, int,
                                                          uint32_t *sb) {
         sb[0] = 0u;
         sb[1] = 0u;
+    }
+    __device__ static __forceinline__ void load_meta_packed(const QView &, size_t, int, int, int, int, uint32_t *sb) {
+        sb[0] = 0u;
     }
     __device__ static __forceinline__ Meta meta_from_raw(const uint32_t *) {
         Meta m;
         m.s = 1.0f;
         m.b = 0.0f;
         return m;
+    }
+    __device__ static __forceinline__ Meta meta_from_packed(const uint32_t *sb) { return meta_from_raw(sb); }
+    __device__ static __forceinline__ Meta load_meta(const QView &, const uint8_t *, const uint8_t *, int) {
+        return meta_from_raw(nullptr);
     }
     __device__ static __forceinline__ void decode_word(uint32_t w, Meta, uint32_t *out /*[2]*/) {
         out[0] = pack_bf16x2(e4m3_to_f32(w & 0xffu), e4m3_to_f32((w >> 8) & 0xffu)); // exact in bf16
@@ -212,6 +248,43 @@ inline int dispatch_format(const QView &q, F &&f) {
     set_error("unsupported quantization mode %d / bits %d", q.mode, q.bits);
     return DMOE_ERR_UNSUPPORTED;
 }
+
+// ---- addressing of one lane's chunk stream (lane = (ln = row within the 32-row block, h = step half)) ----
+template <typename Fmt, bool PACKED>
+struct ChunkStream {
+    const uint8_t *w;     // first chunk of this lane
+    const uint8_t *srow;  // MLX layout: this row's scales / biases
+    const uint8_t *brow;
+    size_t mat;
+    int nb, h, ln;
+    size_t stride;        // bytes between consecutive steps
+
+    __device__ __forceinline__ void init(const QView &q, size_t mat_, int row_block, int ln_, int h_, int n_clamped) {
+        mat = mat_;
+        nb = row_block;
+        h = h_;
+        ln = ln_;
+        if (PACKED) {
+            const int n_steps = q.cols / (2 * Fmt::kVals);
+            w = q.w + mat * q.w_mat + ((size_t)nb * n_steps * 2 + h) * 512 + (size_t)ln * 16;
+            stride = 1024;
+            srow = brow = nullptr;
+        } else {
+            w = q.w + mat * q.w_mat + (size_t)n_clamped * q.w_row + (size_t)h * 16;
+            stride = 32;
+            srow = q.scales + mat * q.s_mat + (size_t)n_clamped * q.s_row;
+            brow = q.biases ? q.biases + mat * q.s_mat + (size_t)n_clamped * q.s_row : nullptr;
+        }
+    }
+    __device__ __forceinline__ uint4 load_chunk(int step) const { return *(const uint4 *)(w + (size_t)step * stride); }
+    __device__ __forceinline__ void load_meta(const QView &q, int step, uint32_t *sb) const {
+        if (PACKED) Fmt::load_meta_packed(q, mat, nb, step, h, ln, sb);
+        else Fmt::load_meta_raw(q, srow, brow, (step * 2 + h) * Fmt::kVals, sb);
+    }
+    __device__ static __forceinline__ Meta meta(const uint32_t *sb) {
+        return PACKED ? Fmt::meta_from_packed(sb) : Fmt::meta_from_raw(sb);
+    }
+};
 
 } // namespace dmoe
 #endif

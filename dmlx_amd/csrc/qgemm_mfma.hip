@@ -19,8 +19,9 @@ namespace dmoe {
 constexpr int kMfmaWaves = 4;
 constexpr int kMT = kMfmaTileM / 32; // 32-row MFMA tiles per workgroup tile
 
-template <typename Fmt, bool GATE_UP>
+template <typename Fmt, bool GATE_UP, bool PACKED>
 __global__ __launch_bounds__(kMfmaWaves * 64) void qgemm_mfma_kernel(GemmArgs g) {
+    using CS = ChunkStream<Fmt, PACKED>;
     constexpr int KV = Fmt::kVals;     // values per 16-byte chunk
     constexpr int KSUB = 2 * KV;       // reduction elements per step
     constexpr int NJ = KV / 8;         // MFMAs (K = 16) per step and tile
@@ -54,17 +55,16 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void qgemm_mfma_kernel(GemmArgs g)
     // gate_up: tile 0 = gate rows, tile 1 = up rows of the same 32 output columns; plain: 64 output columns
     const int col_base = GATE_UP ? ((int)blockIdx.x * kMfmaWaves + wave) * 32 : ((int)blockIdx.x * kMfmaWaves + wave) * 64;
     const bool wave_on = col_base < n_out;
-    const uint8_t *wrow[NT], *srow[NT], *brow[NT];
+    CS cs[NT];
     bool tile_on[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         const QView &b = (GATE_UP && nt == 1) ? g.b1 : g.b0;
-        int n = GATE_UP ? col_base + ln : col_base + 32 * nt + ln;
-        tile_on[nt] = wave_on && (GATE_UP ? true : (col_base + 32 * nt < n_out));
+        const int base = GATE_UP ? col_base : col_base + 32 * nt;
+        tile_on[nt] = wave_on && base < n_out;
+        int n = base + ln;
         if (n >= n_out) n = n_out - 1; // keep addresses valid; such rows are never stored
-        wrow[nt] = b.w + e * b.w_mat + (size_t)n * b.w_row;
-        srow[nt] = b.scales + e * b.s_mat + (size_t)n * b.s_row;
-        brow[nt] = b.biases ? b.biases + e * b.s_mat + (size_t)n * b.s_row : nullptr;
+        cs[nt].init(b, e, (tile_on[nt] ? base : 0) >> 5, ln, h, n);
     }
 
     // ---- activation staging: thread -> (row within pass, 16-byte piece) ------------------------------
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void qgemm_mfma_kernel(GemmArgs g)
 
     uint4 a_reg[PASSES];
     uint4 b_raw[NT];
-    Meta b_meta[NT];
+    uint32_t b_sb[NT][2];
 
     auto load_a = [&](int ss) {
 #pragma unroll
@@ -107,14 +107,8 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void qgemm_mfma_kernel(GemmArgs g)
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             const QView &b = (GATE_UP && nt == 1) ? g.b1 : g.b0;
-            if (tile_on[nt]) {
-                b_raw[nt] = *(const uint4 *)(wrow[nt] + (size_t)(ss * 2 + h) * 16);
-                b_meta[nt] = Fmt::load_meta(b, srow[nt], brow[nt], ss * KSUB + h * KV);
-            } else {
-                b_raw[nt] = make_uint4(0, 0, 0, 0);
-                b_meta[nt].s = 0.0f;
-                b_meta[nt].b = 0.0f;
-            }
+            b_raw[nt] = cs[nt].load_chunk(ss); // rows of a switched-off tile alias valid memory and are never stored
+            cs[nt].load_meta(b, ss, b_sb[nt]);
         }
     };
 
@@ -127,7 +121,7 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void qgemm_mfma_kernel(GemmArgs g)
         const int cur = ss & 1;
         uint32_t wp[NT][KV / 2];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) Fmt::decode_fast(b_raw[nt], b_meta[nt], wp[nt]);
+        for (int nt = 0; nt < NT; ++nt) Fmt::decode_fast(b_raw[nt], CS::meta(b_sb[nt]), wp[nt]);
         const bool more = ss + 1 < n_sub;
         if (more) {
             load_a(ss + 1);
@@ -219,8 +213,13 @@ struct MfmaLaunch {
     int operator()() {
         const int cols_per_block = kMfmaWaves * (g.gate_up ? 32 : 64);
         dim3 grid((unsigned)ceil_div(g.b0.rows, cols_per_block), (unsigned)g.max_tiles), block(kMfmaWaves * 64);
-        if (g.gate_up) hipLaunchKernelGGL((qgemm_mfma_kernel<Fmt, true>), grid, block, 0, st, g);
-        else hipLaunchKernelGGL((qgemm_mfma_kernel<Fmt, false>), grid, block, 0, st, g);
+        if (g.b0.packed) {
+            if (g.gate_up) hipLaunchKernelGGL((qgemm_mfma_kernel<Fmt, true, true>), grid, block, 0, st, g);
+            else hipLaunchKernelGGL((qgemm_mfma_kernel<Fmt, false, true>), grid, block, 0, st, g);
+        } else {
+            if (g.gate_up) hipLaunchKernelGGL((qgemm_mfma_kernel<Fmt, true, false>), grid, block, 0, st, g);
+            else hipLaunchKernelGGL((qgemm_mfma_kernel<Fmt, false, false>), grid, block, 0, st, g);
+        }
         DMOE_LAUNCH_CHECK();
         return DMOE_OK;
     }
@@ -235,7 +234,7 @@ int launch_qgemm_mfma(const GemmArgs &g, hipStream_t st) {
                  "MFMA GEMM: bad output / activation pointer or pitch");
     if (g.gate_up)
         DMOE_REQUIRE(g.b1.rows == g.b0.rows && g.b1.cols == g.b0.cols && g.b1.mode == g.b0.mode &&
-                         g.b1.bits == g.b0.bits && g.b1.group == g.b0.group,
+                         g.b1.bits == g.b0.bits && g.b1.group == g.b0.group && g.b1.packed == g.b0.packed,
                      "MFMA GEMM: gate and up projections differ in shape or format");
     if (g.max_tiles == 0) return DMOE_OK;
     return dispatch_format(g.b0, MfmaLaunch{g, st});

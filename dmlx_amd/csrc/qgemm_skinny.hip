@@ -1,0 +1,288 @@
+// Grouped quantized GEMM, skinny path (decode): at most kSkinnyTileM rows per expert tile.
+//
+// The step is bound by streaming every live expert's packed weights once from HBM. Each of the four
+// wavefronts of a workgroup owns 32 weight rows (per projection) and walks the whole reduction
+// dimension on its own: lane (n = lane % 32, h = lane / 32) loads the 16-byte chunk h of row n for the
+// current 64-wide step straight into registers, a ring of kSkinnyStages steps deep, so ~14 KiB per
+// wavefront are in flight while one step is consumed and the wavefronts never wait for each other.
+// The tile's activations (<= 8 rows) sit in LDS for the whole kernel and feed the A operand of
+// v_mfma_f32_32x32x16_bf16; the weights feed the B operand, so every lane's accumulators belong to ITS
+// weight row and rows 4h..4h+3 of the tile, and nothing has to be reduced across lanes.
+//
+// 4-bit affine weights (group >= 64) are never multiplied out. Codes become the bf16 numbers (128 + q)
+// with one AND-OR per pair; both halves of a step lie in the same scale group, so the matrix core
+// produces P[m][n] = sum_k x[m][k] (128 + q[n][k]) for one group and the lane applies
+//     acc += s[n] * P + (b[n] - 128 s[n]) * sum_k x[m][k]
+// with its own row's scale and bias: two FMAs per accumulator and group. The AND-OR leaves the codes of
+// a word in the order (0,4,1,5,2,6,3,7); the activations are stored in LDS in the same order, which a
+// sum does not see. Other formats are decoded to bf16 values and accumulated directly.
+#include "common.h"
+#include <type_traits>
+
+#include "qformat.h"
+
+namespace dmoe {
+
+constexpr int kSkinnyWaves = 4;
+constexpr int kSkinnyStages = 8;
+
+__device__ __forceinline__ uint32_t vgpr_const32(uint32_t c) {
+    uint32_t v;
+    asm volatile("v_mov_b32 %0, %1" : "=v"(v) : "s"(c));
+    return v;
+}
+
+// (q_i, q_{i+4}) of each 8-code word as packed bf16 (128 + q): element order 0,4,1,5,2,6,3,7
+__device__ __forceinline__ void codes_to_bf16(uint32_t w, uint32_t mask, uint32_t magic, uint32_t *o) {
+    o[0] = (w & mask) | magic;
+    o[1] = ((w >> 4) & mask) | magic;
+    o[2] = ((w >> 8) & mask) | magic;
+    o[3] = ((w >> 12) & mask) | magic;
+}
+
+template <int NM>
+struct SkinnyStage {
+    uint4 raw[NM];
+    uint32_t sb[NM][2];
+};
+
+template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED>
+__global__ __launch_bounds__(kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArgs g) {
+    using CS = ChunkStream<Fmt, PACKED>;
+    constexpr int KV = Fmt::kVals;   // values per 16-byte chunk
+    constexpr int KSTEP = 2 * KV;    // reduction elements per step (both lane halves)
+    constexpr int NJ = KV / 8;       // MFMAs (K = 16) per step
+    constexpr int NM = GATE_UP ? 2 : 1;
+    extern __shared__ __attribute__((aligned(16))) uint8_t skinny_lds[];
+
+    Tile t;
+    const uint32_t slot = blockIdx.y;
+    if (g.tiles) {
+        const uint32_t n_tiles = *g.n_tiles; // both loads are issued before either is needed
+        t = g.tiles[slot];                   // the list has room for every launched slot
+        if (slot >= n_tiles) return;
+    } else {
+        t.expert = 0;
+        t.row0 = slot * (uint32_t)kSkinnyTileM;
+        if ((int)t.row0 >= g.dense_rows) return;
+        uint32_t left = (uint32_t)g.dense_rows - t.row0;
+        t.nrows = left < (uint32_t)kSkinnyTileM ? left : (uint32_t)kSkinnyTileM;
+    }
+    const int tid = (int)threadIdx.x, lane = tid & 63, ln = lane & 31, h = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int cols = g.b0.cols, n_out = g.b0.rows;
+    const int n_steps = cols / KSTEP;
+    const size_t e = t.expert;
+
+    // ---- this lane's weight row ------------------------------------------------------------------------
+    const int col0 = ((int)blockIdx.x * kSkinnyWaves + wave) * 32;
+    const bool wave_on = col0 < n_out;
+    int n = col0 + ln;
+    if (n >= n_out) n = n_out - 1; // stay inside the matrix; such rows are never stored
+    CS cs[NM];
+#pragma unroll
+    for (int mi = 0; mi < NM; ++mi) cs[mi].init(mi == 0 ? g.b0 : g.b1, e, col0 >> 5, ln, h, n);
+    auto load_stage = [&](int step, SkinnyStage<NM> &s) {
+#pragma unroll
+        for (int mi = 0; mi < NM; ++mi) {
+            s.raw[mi] = cs[mi].load_chunk(step);
+            cs[mi].load_meta(mi == 0 ? g.b0 : g.b1, step, s.sb[mi]);
+        }
+    };
+
+    // the first weight loads depend on the tile only: issue them before anything else
+    SkinnyStage<NM> ring[kSkinnyStages];
+    if (wave_on) {
+#pragma unroll
+        for (int j = 0; j < kSkinnyStages - 1; ++j)
+            if (j < n_steps) load_stage(j, ring[j]);
+    }
+
+    // ---- activations of the tile -> LDS (rows past the tile are zero) -----------------------------------
+    const int pitch = cols * 2 + 16; // bytes per LDS row; +16 keeps the 8 rows on different banks
+    uint8_t *xs_lds = skinny_lds;
+    float *gs_lds = (float *)(skinny_lds + kSkinnyTileM * pitch); // [n_steps][8]: per-step sums of x (factored)
+    {
+        const int pieces = cols / 8; // 16-byte pieces per row
+        for (int idx = tid; idx < kSkinnyTileM * pieces; idx += kSkinnyWaves * 64) {
+            const int r = idx / pieces, pc = idx - r * pieces;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (r < (int)t.nrows) {
+                const uint32_t p = t.row0 + (uint32_t)r;
+                const size_t src = g.a_rows ? g.a_rows[p] : p;
+                v = *(const uint4 *)(g.a + src * (size_t)cols + pc * 8);
+            }
+            if (FACTORED) { // (x0..x7) -> (x0,x4,x1,x5,x2,x6,x3,x7), the order the code pairs come out in
+                uint4 o;
+                o.x = (v.x & 0xffffu) | (v.z << 16);
+                o.y = (v.x >> 16) | (v.z & 0xffff0000u);
+                o.z = (v.y & 0xffffu) | (v.w << 16);
+                o.w = (v.y >> 16) | (v.w & 0xffff0000u);
+                v = o;
+            }
+            *(uint4 *)(xs_lds + r * pitch + pc * 16) = v;
+        }
+    }
+    __syncthreads();
+    if (FACTORED) {
+        for (int idx = tid; idx < n_steps * kSkinnyTileM; idx += kSkinnyWaves * 64) {
+            const int step = idx / kSkinnyTileM, r = idx % kSkinnyTileM;
+            const uint32_t *px = (const uint32_t *)(xs_lds + r * pitch + step * KSTEP * 2);
+            float sum = 0.0f;
+#pragma unroll 8
+            for (int i = 0; i < KSTEP / 2; ++i) sum += bf16_bits_to_f32(px[i] & 0xffffu) + bf16_bits_to_f32(px[i] >> 16);
+            gs_lds[step * kSkinnyTileM + r] = sum;
+        }
+        __syncthreads();
+    }
+    if (!wave_on) return;
+
+    // A-operand source of this lane: tile row ln (zero beyond the tile), reduction half h
+    const bool x_on = ln < kSkinnyTileM;
+    const uint8_t *xlane = xs_lds + (x_on ? ln : 0) * pitch + h * KV * 2;
+
+    f32x16_t acc[NM];
+#pragma unroll
+    for (int mi = 0; mi < NM; ++mi)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[mi][r] = 0.0f;
+    float facc[NM][4];
+#pragma unroll
+    for (int mi = 0; mi < NM; ++mi)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) facc[mi][r] = 0.0f;
+
+    auto consume = [&](int step, const SkinnyStage<NM> &s) {
+        bf16x8_t xf[NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            uint4 q = make_uint4(0, 0, 0, 0);
+            if (x_on) q = *(const uint4 *)(xlane + (size_t)step * KSTEP * 2 + j * 16);
+            xf[j] = __builtin_bit_cast(bf16x8_t, q);
+        }
+        float4 gsum = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (FACTORED) gsum = *(const float4 *)(gs_lds + step * kSkinnyTileM + 4 * h);
+#pragma unroll
+        for (int mi = 0; mi < NM; ++mi) {
+            const Meta meta = CS::meta(s.sb[mi]);
+            uint32_t wp[KV / 2];
+            if (FACTORED) {
+                const uint32_t mask = vgpr_const32(0x000f000fu), magic = vgpr_const32(0x43004300u);
+                codes_to_bf16(s.raw[mi].x, mask, magic, wp);
+                codes_to_bf16(s.raw[mi].y, mask, magic, wp + 4);
+                codes_to_bf16(s.raw[mi].z, mask, magic, wp + 8);
+                codes_to_bf16(s.raw[mi].w, mask, magic, wp + 12);
+                f32x16_t p;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) p[r] = 0.0f;
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    uint4 q = make_uint4(wp[4 * j], wp[4 * j + 1], wp[4 * j + 2], wp[4 * j + 3]);
+                    p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[j], __builtin_bit_cast(bf16x8_t, q), p, 0, 0, 0);
+                }
+                const float boff = fmaf(-128.0f, meta.s, meta.b);
+                facc[mi][0] = fmaf(meta.s, p[0], fmaf(boff, gsum.x, facc[mi][0]));
+                facc[mi][1] = fmaf(meta.s, p[1], fmaf(boff, gsum.y, facc[mi][1]));
+                facc[mi][2] = fmaf(meta.s, p[2], fmaf(boff, gsum.z, facc[mi][2]));
+                facc[mi][3] = fmaf(meta.s, p[3], fmaf(boff, gsum.w, facc[mi][3]));
+            } else {
+                Fmt::decode_fast(s.raw[mi], meta, wp);
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    uint4 q = make_uint4(wp[4 * j], wp[4 * j + 1], wp[4 * j + 2], wp[4 * j + 3]);
+                    acc[mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[j], __builtin_bit_cast(bf16x8_t, q), acc[mi], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+#pragma unroll 1
+    for (int s0 = 0; s0 < n_steps; s0 += kSkinnyStages) {
+#pragma unroll
+        for (int j = 0; j < kSkinnyStages; ++j) {
+            const int step = s0 + j;
+            if (step + kSkinnyStages - 1 < n_steps) load_stage(step + kSkinnyStages - 1, ring[(j + kSkinnyStages - 1) % kSkinnyStages]);
+            if (step < n_steps) consume(step, ring[j]);
+        }
+    }
+
+    // ---- epilogue: this lane holds rows 4h..4h+3 of the tile for weight row n --------------------------
+    if (col0 + ln >= n_out) return;
+    float rs[NM];
+#pragma unroll
+    for (int mi = 0; mi < NM; ++mi) {
+        const QView &q = mi == 0 ? g.b0 : g.b1;
+        rs[mi] = Fmt::kRowScale ? *(const float *)(q.scales + e * q.s_mat + (size_t)n * q.s_row) : 1.0f;
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int i = 4 * h + r;
+        if (i >= (int)t.nrows) continue;
+        float v[NM];
+#pragma unroll
+        for (int mi = 0; mi < NM; ++mi) v[mi] = (FACTORED ? facc[mi][r] : acc[mi][r]) * rs[mi];
+        const uint32_t p = t.row0 + (uint32_t)i;
+        float val = GATE_UP ? limited_swiglu(v[0], v[NM - 1], g.swiglu_limit) : v[0];
+        if (g.row_scale) val *= g.row_scale[g.row_scale_idx ? g.row_scale_idx[p] : p];
+        const size_t dst = g.out_rows ? g.out_rows[p] : p;
+        g.out[dst * (size_t)g.ldo + n] = f32_to_bf16_bits(val);
+    }
+}
+
+static int skinny_vals(const QView &b) {
+    return (b.mode == DMOE_QUANT_AFFINE && b.bits == 4) || b.mode == DMOE_QUANT_MXFP4 ? 32 : 16;
+}
+static size_t skinny_lds_bytes(const QView &b) {
+    size_t x = (size_t)kSkinnyTileM * ((size_t)b.cols * 2 + 16);
+    size_t sums = (size_t)(b.cols / (2 * skinny_vals(b))) * kSkinnyTileM * sizeof(float);
+    return x + sums;
+}
+
+bool qgemm_skinny_supports(const QView &b) {
+    return b.cols % (2 * skinny_vals(b)) == 0 && skinny_lds_bytes(b) <= 150 * 1024;
+}
+
+struct SkinnyLaunch {
+    const GemmArgs &g;
+    hipStream_t st;
+    template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED>
+    int go() {
+        auto kern = qgemm_skinny_kernel<Fmt, GATE_UP, FACTORED, PACKED>;
+        const size_t lds = skinny_lds_bytes(g.b0);
+        static thread_local size_t allowed = 0; // per instantiation: raise the dynamic LDS limit once
+        if (lds > allowed) {
+            DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(150 * 1024)));
+            allowed = 150 * 1024;
+        }
+        dim3 grid((unsigned)ceil_div(g.b0.rows, kSkinnyWaves * 32), (unsigned)g.max_tiles), block(kSkinnyWaves * 64);
+        hipLaunchKernelGGL(kern, grid, block, lds, st, g);
+        DMOE_LAUNCH_CHECK();
+        return DMOE_OK;
+    }
+    template <typename Fmt>
+    int operator()() {
+        // the scale can be factored out of the matrix product when both halves of a step share a group
+        constexpr bool can_factor = std::is_same<Fmt, FmtAffine4>::value;
+        const bool factor = can_factor && g.b0.group >= 64;
+        if (g.b0.packed) {
+            if (factor) return g.gate_up ? go<Fmt, true, can_factor, true>() : go<Fmt, false, can_factor, true>();
+            return g.gate_up ? go<Fmt, true, false, true>() : go<Fmt, false, false, true>();
+        }
+        if (factor) return g.gate_up ? go<Fmt, true, can_factor, false>() : go<Fmt, false, can_factor, false>();
+        return g.gate_up ? go<Fmt, true, false, false>() : go<Fmt, false, false, false>();
+    }
+};
+
+int launch_qgemm_skinny(const GemmArgs &g, hipStream_t st) {
+    DMOE_REQUIRE(qgemm_skinny_supports(g.b0), "skinny GEMM: unsupported weight shape (cols=%d)", g.b0.cols);
+    DMOE_REQUIRE(g.max_tiles >= 0 && g.max_tiles <= 65535, "skinny GEMM: %d tiles exceed the grid limit", g.max_tiles);
+    DMOE_REQUIRE(g.a && g.out && g.ldo > 0 && ((uintptr_t)g.a % 16) == 0, "skinny GEMM: bad pointer");
+    if (g.gate_up)
+        DMOE_REQUIRE(g.b1.rows == g.b0.rows && g.b1.cols == g.b0.cols && g.b1.mode == g.b0.mode &&
+                         g.b1.bits == g.b0.bits && g.b1.group == g.b0.group && g.b1.packed == g.b0.packed,
+                     "skinny GEMM: gate and up projections differ in shape or format");
+    if (g.max_tiles == 0) return DMOE_OK;
+    return dispatch_format(g.b0, SkinnyLaunch{g, st});
+}
+
+} // namespace dmoe
