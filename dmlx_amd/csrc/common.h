@@ -52,7 +52,11 @@ struct Workspace {
     size_t bytes = 0;
     int device = 0;
     StageTimer timer;
+    // side stream (default priority) + fork/join events for work that overlaps the main stream
+    hipStream_t side = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr;
 };
+int side_stream_ready(Workspace *w); // creates the side stream and its events on first use
 
 // stage timing helpers (no-ops unless enabled on the workspace)
 int stage_begin(Workspace *w, int stage, hipStream_t st);

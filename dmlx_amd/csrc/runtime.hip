@@ -38,6 +38,14 @@ int workspace_reserve(dmoe_workspace ws, size_t bytes, Workspace **out) {
     return DMOE_OK;
 }
 
+int side_stream_ready(Workspace *w) {
+    if (w->side) return DMOE_OK;
+    DMOE_HIP(hipStreamCreateWithFlags(&w->side, hipStreamNonBlocking));
+    DMOE_HIP(hipEventCreateWithFlags(&w->fork, hipEventDisableTiming));
+    DMOE_HIP(hipEventCreateWithFlags(&w->join, hipEventDisableTiming));
+    return DMOE_OK;
+}
+
 int stage_flush(Workspace *w) {
     StageTimer &t = w->timer;
     for (int i = 0; i < DMOE_STAGE_COUNT; ++i) {
@@ -216,6 +224,10 @@ int dmoe_workspace_destroy(dmoe_workspace ws) {
         if (w->timer.start[i]) (void)hipEventDestroy(w->timer.start[i]);
         if (w->timer.stop[i]) (void)hipEventDestroy(w->timer.stop[i]);
     }
+    if (w->side) (void)hipStreamSynchronize(w->side);
+    if (w->fork) (void)hipEventDestroy(w->fork);
+    if (w->join) (void)hipEventDestroy(w->join);
+    if (w->side) (void)hipStreamDestroy(w->side);
     hipError_t e = w->base ? hipFree(w->base) : hipSuccess;
     delete w;
     if (e != hipSuccess) return hip_fail(e, "hipFree(workspace)");

@@ -1,0 +1,427 @@
+// Host-side layer over the C ABI (include/dmoe.h), mirroring the call surface of the reference's Zig
+// modules for this path so that a caller of dmlx finds the same names, argument meaning and error
+// behaviour:
+//
+//   src/moe_router.zig            MoERouterConfig, RouteResult, MoERouter{init, topkRoute, expandTokens,
+//                                 reduceExperts}
+//   src/models/deepseek_v4.zig    DSV4Gate.forward (from the scores on), DSV4SwitchGLU.{forward,
+//                                 forwardNoScores}, DSV4MoE.forward
+//   src/models/expert_provider.zig  ExpertProvider{forward, getCacheBias, deinit}
+//   src/models/deepseek_v4_loader.zig  SmeltConfig.buildMask, expert_remap construction
+//   src/batch_builder.zig         build (token concatenation and positions; the attention mask is not
+//                                 part of this path)
+//
+// The reference is Zig over mlx-c; this header is the same layer in C++ because no Zig toolchain is
+// available where this is built (dmlx_amd/zig/dmoe.zig is the @cImport binding a Zig caller would use).
+// Arrays are device buffers owned by the caller-visible handle (as mlx arrays are refcounted handles in
+// the reference); every failing C call throws dmoe::Error carrying dmoe_last_error(), the way the
+// reference turns a non-zero mlx-c return code into error.MlxError.
+#pragma once
+
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "dmoe.h"
+
+namespace dmoe {
+
+struct Error : std::runtime_error {
+    int code;
+    Error(int c, const std::string &m) : std::runtime_error(m), code(c) {}
+};
+
+inline void check(int rc) {
+    if (rc != DMOE_OK) throw Error(rc, dmoe_last_error());
+}
+
+// Execution context: the stream every op is enqueued on plus the scratch workspace (EagerContext of the
+// reference carries the mlx stream).
+class Context {
+  public:
+    explicit Context(int device = 0) {
+        check(dmoe_init(device));
+        check(dmoe_stream_create(&stream_));
+        check(dmoe_workspace_create(&ws_, 0));
+    }
+    ~Context() {
+        dmoe_stream_synchronize(stream_);
+        dmoe_workspace_destroy(ws_);
+        dmoe_stream_destroy(stream_);
+    }
+    Context(const Context &) = delete;
+    Context &operator=(const Context &) = delete;
+    dmoe_stream stream() const { return stream_; }
+    dmoe_workspace workspace() const { return ws_; }
+    void synchronize() const { check(dmoe_stream_synchronize(stream_)); } // Array.eval()
+
+  private:
+    dmoe_stream stream_{};
+    dmoe_workspace ws_{};
+};
+
+enum class DType { float32, bfloat16, uint32, int32, uint8 };
+inline size_t dtype_size(DType t) {
+    switch (t) {
+    case DType::bfloat16: return 2;
+    case DType::uint8: return 1;
+    default: return 4;
+    }
+}
+
+// A dense row-major device array (the path only needs 1-D..3-D). Copying shares the buffer, like the
+// reference's refcounted mlx_array handles; deinit() is implicit.
+class Array {
+  public:
+    Array() = default;
+    Array(const Context &ctx, DType dtype, std::vector<int> shape) : ctx_(&ctx), dtype_(dtype), shape_(std::move(shape)) {
+        void *p = nullptr;
+        check(dmoe_malloc(&p, nbytes()));
+        buf_ = std::shared_ptr<void>(p, [](void *q) { dmoe_free(q); });
+    }
+    // Array.fromData: copies host data to the device
+    template <typename T>
+    static Array fromData(const Context &ctx, const T *data, std::vector<int> shape, DType dtype) {
+        Array a(ctx, dtype, std::move(shape));
+        if (sizeof(T) != dtype_size(dtype)) throw Error(DMOE_ERR_INVALID, "fromData: element size does not match dtype");
+        check(dmoe_copy_to_device(a.data(), data, a.nbytes(), ctx.stream()));
+        return a;
+    }
+    // dataSlice: reads the array back (waits for the stream)
+    template <typename T>
+    std::vector<T> dataSlice() const {
+        if (sizeof(T) != dtype_size(dtype_)) throw Error(DMOE_ERR_INVALID, "dataSlice: element size does not match dtype");
+        std::vector<T> out(size());
+        check(dmoe_copy_to_host(out.data(), data(), nbytes(), ctx_->stream()));
+        return out;
+    }
+    size_t size() const {
+        size_t n = 1;
+        for (int d : shape_) n *= (size_t)d;
+        return n;
+    }
+    size_t nbytes() const { return size() * dtype_size(dtype_); }
+    const std::vector<int> &shape() const { return shape_; }
+    DType dtype() const { return dtype_; }
+    void *data() const { return buf_.get(); }
+    bool valid() const { return (bool)buf_ || size() == 0; }
+    Array reshaped(std::vector<int> shape) const {
+        Array a = *this;
+        a.shape_ = std::move(shape);
+        if (a.size() != size()) throw Error(DMOE_ERR_INVALID, "reshape: element count differs");
+        return a;
+    }
+
+  private:
+    const Context *ctx_ = nullptr;
+    DType dtype_ = DType::float32;
+    std::vector<int> shape_;
+    std::shared_ptr<void> buf_;
+};
+
+// ---- moe_router.zig ----------------------------------------------------------------------------------
+
+struct RouteResult {      // moe_router.zig:21-33
+    Array indices;        // [num_tokens, k] u32
+    Array weights;        // [num_tokens, k] f32
+    size_t k = 0;
+};
+
+struct MoERouterConfig {  // moe_router.zig:36-41
+    size_t num_experts = 0;
+    size_t top_k = 0;
+    bool normalize_weights = true;
+};
+
+class MoERouter {         // moe_router.zig:44-165
+  public:
+    MoERouterConfig config;
+    static MoERouter init(MoERouterConfig c) { return MoERouter{c}; }
+
+    // scores [num_tokens, num_experts] f32 -> indices / weights [num_tokens, k] (columns in ascending score order)
+    RouteResult topkRoute(const Context &ctx, const Array &scores) const {
+        const int T = scores.shape().at(0), E = scores.shape().at(1), K = (int)config.top_k;
+        if ((size_t)E != config.num_experts) throw Error(DMOE_ERR_INVALID, "topkRoute: scores do not have num_experts columns");
+        RouteResult r{Array(ctx, DType::uint32, {T, K}), Array(ctx, DType::float32, {T, K}), config.top_k};
+        check(dmoe_topk_route((uint32_t *)r.indices.data(), (float *)r.weights.data(), (const float *)scores.data(), T, E, K,
+                              config.normalize_weights ? 1 : 0, ctx.stream()));
+        return r;
+    }
+    // x [num_tokens, hidden] -> [num_tokens * k, hidden]
+    static Array expandTokens(const Context &ctx, const Array &x, const RouteResult &route) {
+        const int T = x.shape().at(0), D = x.shape().at(1), K = (int)route.k;
+        Array out(ctx, x.dtype(), {T * K, D});
+        check(dmoe_expand_tokens(out.data(), x.data(), T, D, K, (int)dtype_size(x.dtype()), ctx.stream()));
+        return out;
+    }
+    // expert_outs [num_tokens * k, hidden] -> [num_tokens, hidden] f32, weighted by route.weights
+    static Array reduceExperts(const Context &ctx, const Array &expert_outs, const RouteResult &route) {
+        const int T = route.weights.shape().at(0), K = (int)route.k, D = expert_outs.shape().at(1);
+        Array out(ctx, DType::float32, {T, D});
+        check(dmoe_reduce_experts((float *)out.data(), expert_outs.data(), expert_outs.dtype() == DType::bfloat16 ? 1 : 0,
+                                  (const float *)route.weights.data(), T, K, D, ctx.stream()));
+        return out;
+    }
+};
+
+// ---- deepseek_v4_loader.zig: SmeltConfig -------------------------------------------------------------------
+
+struct SmeltConfig {      // deepseek_v4_loader.zig:250-294
+    enum class Strategy { uniform = 0, first = 1 };
+    bool enabled = false;
+    float load_fraction = 1.0f;
+    Strategy strategy = Strategy::uniform;
+
+    std::vector<uint8_t> buildMask(size_t n_experts) const {
+        std::vector<uint8_t> mask(n_experts);
+        int n = 0;
+        check(dmoe_smelt_build_mask(mask.data(), &n, (int)n_experts, load_fraction, (int)strategy, enabled ? 1 : 0));
+        return mask;
+    }
+    // expert_remap of DSV4MoE (deepseek_v4_loader.zig:2151-2168)
+    static std::vector<int32_t> buildRemap(const std::vector<uint8_t> &mask) {
+        std::vector<int32_t> remap(mask.size());
+        check(dmoe_build_remap(remap.data(), mask.data(), (int)mask.size()));
+        return remap;
+    }
+};
+
+// ---- deepseek_v4.zig: gate epilogue, SwitchGLU, MoE ----------------------------------------------------------
+
+enum class ScoringFunc { softmax, sigmoid, sqrtsoftplus }; // deepseek_v4.zig:82-86
+
+// DSV4Gate from the scores on (deepseek_v4.zig:589-678). The router GEMM and the scoring function run
+// upstream of this path; `forward` takes their result.
+struct DSV4Gate {
+    size_t topk = 0, n_routed_experts = 0;
+    float route_scale = 1.0f;
+    ScoringFunc scoring_func = ScoringFunc::sqrtsoftplus;
+    Array bias;        // optional [n_routed_experts] f32 selection bias
+    Array smelt_mask;  // optional [n_routed_experts] u8 residency mask
+
+    // returns (weights [T, topk] f32, indices [T, topk] u32) like the reference's tuple
+    std::pair<Array, Array> forward(const Context &ctx, const Array &scores) const {
+        const int T = scores.shape().at(0), E = scores.shape().at(1), K = (int)topk;
+        Array idx(ctx, DType::uint32, {T, K}), w(ctx, DType::float32, {T, K});
+        check(dmoe_gate_route((uint32_t *)idx.data(), (float *)w.data(), (const float *)scores.data(),
+                              bias.data() ? (const float *)bias.data() : nullptr,
+                              smelt_mask.data() ? (const uint8_t *)smelt_mask.data() : nullptr, T, E, K,
+                              scoring_func != ScoringFunc::softmax ? 1 : 0, route_scale, ctx.stream()));
+        return {w, idx};
+    }
+};
+
+// Quantized stack description on the host side (QuantizedWeight + QuantConfig of mlx-zig)
+struct QuantizedWeight {
+    const void *data = nullptr, *scales = nullptr, *biases = nullptr; // host or device memory, see weight_source
+    int n_mats = 1, rows = 0, cols = 0;
+    int group_size = 64, bits = 4;
+    std::string mode = "affine"; // "affine" | "mxfp4" | "fp8"
+    dmoe_qweight c() const {
+        dmoe_qweight q{};
+        q.w = data;
+        q.scales = scales;
+        q.biases = biases;
+        q.n_mats = n_mats;
+        q.rows = rows;
+        q.cols = cols;
+        q.mode = dmoe_quant_mode_from_string(mode.c_str());
+        q.bits = bits;
+        q.group_size = group_size;
+        if (q.mode < 0) throw Error(DMOE_ERR_INVALID, "unknown quantization mode " + mode);
+        return q;
+    }
+};
+
+// One MoE layer's resident experts: DSV4SwitchGLU (routed, deepseek_v4.zig:687-980) + the shared
+// DSV4Expert (:442-518) + expert_remap (:991-993). Owns a dmoe_layer.
+class DSV4SwitchGLU {
+  public:
+    struct Options {
+        float swiglu_limit = 0.0f;
+        bool score_before_down = false; // true: DSV4SwitchGLU.forward (:796-806); false: provider paths
+        const QuantizedWeight *shared_gate = nullptr, *shared_up = nullptr, *shared_down = nullptr;
+        float shared_swiglu_limit = 0.0f;
+        std::vector<int32_t> remap;     // router id -> slot; empty = identity
+        dmoe_weight_source source = DMOE_WEIGHTS_COPY_FROM_HOST;
+    };
+    DSV4SwitchGLU(const Context &ctx, int hidden, int ffn, int top_k, const QuantizedWeight &gate, const QuantizedWeight &up,
+                  const QuantizedWeight &down, const Options &opt)
+        : hidden_(hidden), ffn_(ffn), top_k_(top_k) {
+        dmoe_layer_desc d{};
+        d.hidden = hidden;
+        d.ffn = ffn;
+        d.top_k = top_k;
+        d.gate = gate.c();
+        d.up = up.c();
+        d.down = down.c();
+        d.swiglu_limit = opt.swiglu_limit;
+        d.score_before_down = opt.score_before_down ? 1 : 0;
+        if (opt.shared_gate) {
+            d.has_shared = 1;
+            d.shared_gate = opt.shared_gate->c();
+            d.shared_up = opt.shared_up->c();
+            d.shared_down = opt.shared_down->c();
+            d.shared_swiglu_limit = opt.shared_swiglu_limit;
+        }
+        if (!opt.remap.empty()) {
+            d.remap = opt.remap.data();
+            d.n_experts_total = (int)opt.remap.size();
+        }
+        d.weight_source = opt.source;
+        check(dmoe_layer_create(&layer_, &d, ctx.stream()));
+    }
+    ~DSV4SwitchGLU() { dmoe_layer_destroy(layer_); } // deinit()
+    DSV4SwitchGLU(const DSV4SwitchGLU &) = delete;
+    DSV4SwitchGLU &operator=(const DSV4SwitchGLU &) = delete;
+
+    // x [N, hidden] bf16, indices [N, topk] u32 (router ids), scores [N, topk] f32 -> [N, hidden] bf16
+    // (routed experts, weighted sum over k, plus the shared expert when the layer has one)
+    Array forward(const Context &ctx, const Array &x, const Array &indices, const Array &scores) const {
+        const int T = x.shape().at(0);
+        Array out(ctx, DType::bfloat16, {T, hidden_});
+        check(dmoe_moe_forward((uint16_t *)out.data(), layer_, (const uint16_t *)x.data(), (const uint32_t *)indices.data(),
+                               (const float *)scores.data(), T, ctx.workspace(), ctx.stream()));
+        return out;
+    }
+    // expert outputs without scores, [N, topk, hidden] bf16 (deepseek_v4.zig:855-945); indices are slot ids
+    Array forwardNoScores(const Context &ctx, const Array &x, const Array &slot_indices) const {
+        const int T = x.shape().at(0);
+        Array out(ctx, DType::bfloat16, {T, top_k_, hidden_});
+        check(dmoe_switch_glu_forward_no_scores((uint16_t *)out.data(), layer_, (const uint16_t *)x.data(),
+                                                (const uint32_t *)slot_indices.data(), T, ctx.workspace(), ctx.stream()));
+        return out;
+    }
+    dmoe_layer handle() const { return layer_; }
+    int hidden() const { return hidden_; }
+    int top_k() const { return top_k_; }
+
+  private:
+    dmoe_layer layer_{};
+    int hidden_, ffn_, top_k_;
+};
+
+// ---- expert_provider.zig --------------------------------------------------------------------------------------
+
+// ExpertProvider.VTable (expert_provider.zig:12-48) as an abstract class.
+class ExpertProvider {
+  public:
+    virtual ~ExpertProvider() = default;                                   // deinit
+    virtual Array forward(const Context &ctx, size_t layer_idx, const Array &flat_x, const Array &indices,
+                          const Array &scores) = 0;
+    virtual bool getCacheBias(size_t /*layer_idx*/, std::vector<float> * /*out*/) { return false; } // optional
+};
+
+// Experts resident in HBM: what replaces ExpertStreamProvider / ExpertPreloadProvider (no SSD, no cache).
+class ResidentExpertProvider : public ExpertProvider {
+  public:
+    void addLayer(std::unique_ptr<DSV4SwitchGLU> layer, std::vector<float> cache_bias = {}) {
+        layers_.push_back(std::move(layer));
+        cache_bias_.push_back(std::move(cache_bias));
+    }
+    Array forward(const Context &ctx, size_t layer_idx, const Array &flat_x, const Array &indices, const Array &scores) override {
+        if (layer_idx >= layers_.size()) throw Error(DMOE_ERR_INVALID, "PreloadProviderNotInitialized: no such layer");
+        return layers_[layer_idx]->forward(ctx, flat_x, indices, scores);
+    }
+    bool getCacheBias(size_t layer_idx, std::vector<float> *out) override {
+        if (layer_idx >= cache_bias_.size() || cache_bias_[layer_idx].empty()) return false;
+        *out = cache_bias_[layer_idx];
+        return true;
+    }
+    // expert_preload.zig:141-160: remap + cache bias (0 loaded, -1000 not loaded) for a list of loaded ids
+    static std::pair<std::vector<int32_t>, std::vector<float>> preloadRemap(const std::vector<uint32_t> &ids, size_t n_total) {
+        std::vector<int32_t> remap(n_total);
+        std::vector<float> bias(n_total);
+        check(dmoe_preload_remap(remap.data(), bias.data(), ids.data(), (int)ids.size(), (int)n_total));
+        return {remap, bias};
+    }
+
+  private:
+    std::vector<std::unique_ptr<DSV4SwitchGLU>> layers_;
+    std::vector<std::vector<float>> cache_bias_;
+};
+
+// DSV4MoE.forward from the gate scores on (deepseek_v4.zig:1010-1056): hidden [B, S, D] -> [B, S, D].
+struct DSV4MoE {
+    DSV4Gate gate;
+    ExpertProvider *stream_provider = nullptr; // owned by the model, as in the reference
+    size_t layer_idx = 0;
+
+    Array forward(const Context &ctx, const Array &hidden_states, const Array &scores) const {
+        const auto &sh = hidden_states.shape();
+        const int B = sh.at(0), S = sh.at(1), D = sh.at(2);
+        Array flat = hidden_states.reshaped({B * S, D});
+        auto routed = gate.forward(ctx, scores);
+        if (!stream_provider) throw Error(DMOE_ERR_INVALID, "PreloadProviderNotInitialized");
+        Array y = stream_provider->forward(ctx, layer_idx, flat, routed.second, routed.first);
+        return y.reshaped({B, S, D});
+    }
+};
+
+// ---- batch_builder.zig ----------------------------------------------------------------------------------------
+
+struct Request {                     // the fields of scheduler.zig's Request that build() reads
+    enum class State { waiting, prefilling, decoding, done } state = State::waiting;
+    std::vector<uint32_t> prompt_tokens, generated_tokens;
+    size_t prefill_offset = 0;
+    size_t seqLen() const { return prompt_tokens.size() + generated_tokens.size(); }
+};
+
+struct BatchResult {                 // batch_builder.zig:24-43 without the [T,T] mask
+    std::vector<uint32_t> batched_tokens;
+    std::vector<int32_t> position_ids;
+    std::vector<int32_t> request_offsets; // start of each request in the flat batch, plus the total
+    size_t total_tokens = 0, num_requests = 0;
+};
+
+namespace batch_builder {
+// getRequestTokens (batch_builder.zig:47-83)
+inline std::vector<uint32_t> getRequestTokens(const Request &r) {
+    switch (r.state) {
+    case Request::State::prefilling:
+    case Request::State::waiting:
+        if (r.prefill_offset >= r.prompt_tokens.size()) {
+            if (!r.prompt_tokens.empty()) return {r.prompt_tokens.back()};
+            return {};
+        }
+        return std::vector<uint32_t>(r.prompt_tokens.begin() + (long)r.prefill_offset, r.prompt_tokens.end());
+    case Request::State::decoding:
+        if (!r.generated_tokens.empty()) return {r.generated_tokens.back()};
+        if (!r.prompt_tokens.empty()) return {r.prompt_tokens.back()};
+        return {};
+    default: return {};
+    }
+}
+// build (batch_builder.zig:90-214): prefill requests first, then decode requests
+inline BatchResult build(const std::vector<const Request *> &prefill_requests, const std::vector<const Request *> &decode_requests) {
+    BatchResult out;
+    std::vector<const Request *> all(prefill_requests);
+    all.insert(all.end(), decode_requests.begin(), decode_requests.end());
+    out.num_requests = all.size();
+    for (const Request *r : all) {
+        std::vector<uint32_t> toks = getRequestTokens(*r);
+        size_t base = 0;
+        switch (r->state) {
+        case Request::State::prefilling:
+        case Request::State::waiting: base = r->prefill_offset; break;
+        case Request::State::decoding: base = r->seqLen() > 0 ? r->seqLen() - toks.size() : 0; break;
+        default: base = 0;
+        }
+        out.request_offsets.push_back((int32_t)out.batched_tokens.size());
+        for (size_t j = 0; j < toks.size(); ++j) {
+            out.batched_tokens.push_back(toks[j]);
+            out.position_ids.push_back((int32_t)(base + j));
+        }
+    }
+    out.total_tokens = out.batched_tokens.size();
+    out.request_offsets.push_back((int32_t)out.total_tokens);
+    return out;
+}
+} // namespace batch_builder
+
+} // namespace dmoe

@@ -1,0 +1,178 @@
+//! Zig binding of libdmoe (include/dmoe.h) with the call surface of dmlx's own modules, so that
+//! `src/moe_router.zig` and the provider arm of `DSV4MoE.forward` can switch from mlx-c to this library
+//! without touching their callers. It is imported the way dmlx imports mlx-c:
+//!
+//!     const c = @cImport({ @cInclude("dmoe.h"); });
+//!
+//! NOTE: written against Zig 0.16 (the version dmlx pins) but NOT compiled in this repository: the build
+//! environment has no Zig toolchain. The C++ twin of this file (dmlx_amd/host/moe.hpp) is compiled and
+//! tested; the two are kept line-for-line parallel. build.zig additions:
+//!     exe.addIncludePath(.{ .cwd_relative = "<repo>/include" });
+//!     exe.addLibraryPath(.{ .cwd_relative = "<repo>/dmlx_amd/lib" });
+//!     exe.linkSystemLibrary("dmoe");
+const std = @import("std");
+pub const c = @cImport({
+    @cInclude("dmoe.h");
+});
+
+pub const Error = error{DmoeError};
+
+/// Same contract as mlx-zig's `c.check`: a non-zero return code becomes one Zig error after the
+/// library's message has been logged.
+pub fn check(rc: c_int) Error!void {
+    if (rc != 0) {
+        std.log.err("dmoe: {s}", .{std.mem.span(c.dmoe_last_error())});
+        return Error.DmoeError;
+    }
+}
+
+/// Stream + scratch workspace (what `EagerContext` carries in dmlx).
+pub const Context = struct {
+    stream: c.dmoe_stream,
+    ws: c.dmoe_workspace,
+
+    pub fn init(device: c_int) Error!Context {
+        try check(c.dmoe_init(device));
+        var s: c.dmoe_stream = undefined;
+        try check(c.dmoe_stream_create(&s));
+        var w: c.dmoe_workspace = undefined;
+        try check(c.dmoe_workspace_create(&w, 0));
+        return .{ .stream = s, .ws = w };
+    }
+    pub fn deinit(self: Context) void {
+        _ = c.dmoe_stream_synchronize(self.stream);
+        _ = c.dmoe_workspace_destroy(self.ws);
+        _ = c.dmoe_stream_destroy(self.stream);
+    }
+    /// Array.eval(): the host-visible synchronisation point
+    pub fn eval(self: Context) Error!void {
+        try check(c.dmoe_stream_synchronize(self.stream));
+    }
+};
+
+/// Dense row-major device array; `deinit` frees it (handles are owned, as `Array.fromHandle` results are).
+pub fn DeviceArray(comptime T: type) type {
+    return struct {
+        ptr: ?*anyopaque,
+        len: usize,
+        const Self = @This();
+        pub fn alloc(len: usize) Error!Self {
+            var p: ?*anyopaque = null;
+            try check(c.dmoe_malloc(&p, len * @sizeOf(T)));
+            return .{ .ptr = p, .len = len };
+        }
+        pub fn fromData(ctx: Context, data: []const T) Error!Self {
+            const a = try alloc(data.len);
+            try check(c.dmoe_copy_to_device(a.ptr, data.ptr, data.len * @sizeOf(T), ctx.stream));
+            return a;
+        }
+        pub fn dataSlice(self: Self, ctx: Context, out: []T) Error!void {
+            try check(c.dmoe_copy_to_host(out.ptr, self.ptr, self.len * @sizeOf(T), ctx.stream));
+        }
+        pub fn deinit(self: Self) void {
+            _ = c.dmoe_free(self.ptr);
+        }
+    };
+}
+
+// ---- src/moe_router.zig ------------------------------------------------------------------------------
+
+pub const RouteResult = struct {
+    indices: DeviceArray(u32), // [num_tokens, k]
+    weights: DeviceArray(f32), // [num_tokens, k]
+    k: usize,
+    num_tokens: usize,
+    pub fn deinit(self: RouteResult) void {
+        self.indices.deinit();
+        self.weights.deinit();
+    }
+};
+
+pub const MoERouterConfig = struct {
+    num_experts: usize,
+    top_k: usize,
+    normalize_weights: bool = true,
+};
+
+pub const MoERouter = struct {
+    config: MoERouterConfig,
+
+    pub fn init(config: MoERouterConfig) MoERouter {
+        return .{ .config = config };
+    }
+
+    /// scores: [num_tokens, num_experts] f32 on the device
+    pub fn topkRoute(self: *const MoERouter, ctx: Context, scores: DeviceArray(f32), num_tokens: usize) Error!RouteResult {
+        const k = self.config.top_k;
+        const idx = try DeviceArray(u32).alloc(num_tokens * k);
+        errdefer idx.deinit();
+        const w = try DeviceArray(f32).alloc(num_tokens * k);
+        errdefer w.deinit();
+        try check(c.dmoe_topk_route(@ptrCast(@alignCast(idx.ptr)), @ptrCast(@alignCast(w.ptr)), @ptrCast(@alignCast(scores.ptr)), @intCast(num_tokens), @intCast(self.config.num_experts), @intCast(k), @intFromBool(self.config.normalize_weights), ctx.stream));
+        return .{ .indices = idx, .weights = w, .k = k, .num_tokens = num_tokens };
+    }
+
+    /// x: [num_tokens, hidden] -> [num_tokens * k, hidden]
+    pub fn expandTokens(ctx: Context, comptime T: type, x: DeviceArray(T), hidden: usize, route: RouteResult) Error!DeviceArray(T) {
+        const out = try DeviceArray(T).alloc(route.num_tokens * route.k * hidden);
+        errdefer out.deinit();
+        try check(c.dmoe_expand_tokens(out.ptr, x.ptr, @intCast(route.num_tokens), @intCast(hidden), @intCast(route.k), @sizeOf(T), ctx.stream));
+        return out;
+    }
+
+    /// expert_outs: [num_tokens * k, hidden] f32 -> [num_tokens, hidden] f32
+    pub fn reduceExperts(ctx: Context, expert_outs: DeviceArray(f32), hidden: usize, route: RouteResult) Error!DeviceArray(f32) {
+        const out = try DeviceArray(f32).alloc(route.num_tokens * hidden);
+        errdefer out.deinit();
+        try check(c.dmoe_reduce_experts(@ptrCast(@alignCast(out.ptr)), expert_outs.ptr, 0, @ptrCast(@alignCast(route.weights.ptr)), @intCast(route.num_tokens), @intCast(route.k), @intCast(hidden), ctx.stream));
+        return out;
+    }
+};
+
+// ---- src/models/deepseek_v4.zig: gate epilogue and the provider arm of DSV4MoE.forward ----------------------
+
+/// DSV4Gate.forward from the scores on (deepseek_v4.zig:589-678)
+pub fn gateRoute(ctx: Context, scores: DeviceArray(f32), bias: ?DeviceArray(f32), smelt_mask: ?DeviceArray(u8), num_tokens: usize, n_experts: usize, topk: usize, renorm: bool, route_scale: f32) Error!RouteResult {
+    const idx = try DeviceArray(u32).alloc(num_tokens * topk);
+    errdefer idx.deinit();
+    const w = try DeviceArray(f32).alloc(num_tokens * topk);
+    errdefer w.deinit();
+    try check(c.dmoe_gate_route(@ptrCast(@alignCast(idx.ptr)), @ptrCast(@alignCast(w.ptr)), @ptrCast(@alignCast(scores.ptr)), if (bias) |b| @ptrCast(@alignCast(b.ptr)) else null, if (smelt_mask) |m| @ptrCast(@alignCast(m.ptr)) else null, @intCast(num_tokens), @intCast(n_experts), @intCast(topk), @intFromBool(renorm), route_scale, ctx.stream));
+    return .{ .indices = idx, .weights = w, .k = topk, .num_tokens = num_tokens };
+}
+
+/// ExpertProvider over HBM-resident experts: `forward(layer_idx, flat_x, indices, scores)` as in
+/// src/models/expert_provider.zig:21; replaces ExpertStreamProvider.streamForward (expert_stream.zig:245-261).
+pub const ResidentExpertProvider = struct {
+    layers: []c.dmoe_layer,
+    hidden: usize,
+
+    pub fn forward(self: *ResidentExpertProvider, ctx: Context, layer_idx: usize, flat_x: DeviceArray(u16), indices: DeviceArray(u32), scores: DeviceArray(f32), num_tokens: usize) Error!DeviceArray(u16) {
+        if (layer_idx >= self.layers.len) return Error.DmoeError; // error.PreloadProviderNotInitialized in dmlx
+        const out = try DeviceArray(u16).alloc(num_tokens * self.hidden);
+        errdefer out.deinit();
+        try check(c.dmoe_moe_forward(@ptrCast(@alignCast(out.ptr)), self.layers[layer_idx], @ptrCast(@alignCast(flat_x.ptr)), @ptrCast(@alignCast(indices.ptr)), @ptrCast(@alignCast(scores.ptr)), @intCast(num_tokens), ctx.ws, ctx.stream));
+        return out;
+    }
+
+    pub fn deinit(self: *ResidentExpertProvider) void {
+        for (self.layers) |l| _ = c.dmoe_layer_destroy(l);
+    }
+};
+
+/// SmeltConfig.buildMask (deepseek_v4_loader.zig:272-293)
+pub fn smeltBuildMask(allocator: std.mem.Allocator, n_experts: usize, load_fraction: f32, first: bool, enabled: bool) ![]u8 {
+    const mask = try allocator.alloc(u8, n_experts);
+    errdefer allocator.free(mask);
+    var n: c_int = 0;
+    try check(c.dmoe_smelt_build_mask(mask.ptr, &n, @intCast(n_experts), load_fraction, @intFromBool(first), @intFromBool(enabled)));
+    return mask;
+}
+
+/// expert_remap (deepseek_v4_loader.zig:2151-2168)
+pub fn buildRemap(allocator: std.mem.Allocator, mask: []const u8) ![]i32 {
+    const remap = try allocator.alloc(i32, mask.len);
+    errdefer allocator.free(remap);
+    try check(c.dmoe_build_remap(remap.ptr, mask.ptr, @intCast(mask.len)));
+    return remap;
+}

@@ -1,0 +1,250 @@
+// Runs the reference's own router / remap / batch-builder test vectors (src/moe_router.zig:169-439,
+// src/tests/expert_remap_test.zig, src/tests/batch_builder_tests.zig) through the C++ host layer
+// (dmlx_amd/host/moe.hpp) on the GPU, plus a closed-form check of the layer forward, the way the
+// reference's model smoke tests use constant weights (src/tests/deepseek_v4_tests.zig:398-610).
+// Built with g++ against libdmoe.so; prints "ALL HOST TESTS PASSED" and exits 0 on success.
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <set>
+
+#include "../../dmlx_amd/host/moe.hpp"
+
+using namespace dmoe;
+
+static int g_failed = 0;
+#define EXPECT(cond)                                                              \
+    do {                                                                          \
+        if (!(cond)) {                                                            \
+            std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);         \
+            ++g_failed;                                                           \
+        }                                                                         \
+    } while (0)
+#define NEAR(a, b, tol) EXPECT(std::fabs((double)(a) - (double)(b)) <= (tol))
+
+static uint16_t bf16(float f) {
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+static float from_bf16(uint16_t h) {
+    uint32_t u = (uint32_t)h << 16;
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
+}
+
+static void test_topk(const Context &ctx) {
+    { // "MoERouter topkRoute selects correct top-k experts"
+        auto router = MoERouter::init({4, 2, false});
+        const float s[] = {0.1f, 0.9f, 0.3f, 0.7f, 0.8f, 0.2f, 0.6f, 0.4f};
+        auto r = router.topkRoute(ctx, Array::fromData(ctx, s, {2, 4}, DType::float32));
+        EXPECT(r.k == 2 && r.indices.shape() == std::vector<int>({2, 2}) && r.weights.shape() == std::vector<int>({2, 2}));
+        auto w = r.weights.dataSlice<float>();
+        NEAR(w[0] + w[1], 1.6, 1e-5);
+        NEAR(w[2] + w[3], 1.4, 1e-5);
+    }
+    { // "MoERouter topkRoute with weight normalization"
+        auto router = MoERouter::init({3, 2, true});
+        const float s[] = {0.2f, 0.6f, 0.4f};
+        auto r = router.topkRoute(ctx, Array::fromData(ctx, s, {1, 3}, DType::float32));
+        auto w = r.weights.dataSlice<float>();
+        auto idx = r.indices.dataSlice<uint32_t>();
+        NEAR(w[0] + w[1], 1.0, 1e-5);
+        EXPECT((idx[0] == 1 && idx[1] == 2) || (idx[0] == 2 && idx[1] == 1));
+        for (int i = 0; i < 2; ++i) NEAR(w[i], s[idx[i]] / (0.6f + 0.4f), 1e-5);
+    }
+    { // "MoERouter config with different num_experts and top_k"
+        auto router = MoERouter::init({8, 3, false});
+        const float s[] = {0.1f, 0.2f, 0.8f, 0.3f, 0.9f, 0.4f, 0.7f, 0.5f};
+        auto r = router.topkRoute(ctx, Array::fromData(ctx, s, {1, 8}, DType::float32));
+        auto idx = r.indices.dataSlice<uint32_t>();
+        auto w = r.weights.dataSlice<float>();
+        std::set<uint32_t> got(idx.begin(), idx.end());
+        EXPECT(got == std::set<uint32_t>({2, 4, 6}));
+        for (int i = 0; i < 3; ++i) NEAR(w[i], s[idx[i]], 1e-5);
+    }
+}
+
+static void test_expand_reduce(const Context &ctx) {
+    const float x[] = {1, 2, 3, 4, 5, 6};
+    const uint32_t di[] = {0, 1, 2, 3};
+    const float dw[] = {0.6f, 0.4f, 0.7f, 0.3f};
+    RouteResult route{Array::fromData(ctx, di, {2, 2}, DType::uint32), Array::fromData(ctx, dw, {2, 2}, DType::float32), 2};
+    auto ex = MoERouter::expandTokens(ctx, Array::fromData(ctx, x, {2, 3}, DType::float32), route);
+    EXPECT(ex.shape() == std::vector<int>({4, 3}));
+    auto e = ex.dataSlice<float>();
+    const float want[] = {1, 2, 3, 1, 2, 3, 4, 5, 6, 4, 5, 6};
+    for (int i = 0; i < 12; ++i) NEAR(e[i], want[i], 1e-5);
+
+    const float eo[] = {1, 0, 0, 0, 1, 0, 0, 0, 1, 1, 1, 1};
+    const float rw[] = {0.7f, 0.3f, 0.4f, 0.6f};
+    RouteResult r2{Array::fromData(ctx, di, {2, 2}, DType::uint32), Array::fromData(ctx, rw, {2, 2}, DType::float32), 2};
+    auto red = MoERouter::reduceExperts(ctx, Array::fromData(ctx, eo, {4, 3}, DType::float32), r2).dataSlice<float>();
+    const float wr[] = {0.7f, 0.3f, 0.0f, 0.6f, 0.6f, 1.0f};
+    for (int i = 0; i < 6; ++i) NEAR(red[i], wr[i], 1e-5);
+
+    // "MoERouter end-to-end route-expand-reduce": identity expert + normalised weights give x back
+    auto router = MoERouter::init({4, 2, true});
+    const float s[] = {0.1f, 0.5f, 0.3f, 0.1f, 0.4f, 0.1f, 0.1f, 0.4f, 0.2f, 0.2f, 0.5f, 0.1f};
+    const float x3[] = {1, 2, 3, 4, 5, 6};
+    auto xs = Array::fromData(ctx, x3, {3, 2}, DType::float32);
+    auto r3 = router.topkRoute(ctx, Array::fromData(ctx, s, {3, 4}, DType::float32));
+    auto back = MoERouter::reduceExperts(ctx, MoERouter::expandTokens(ctx, xs, r3), r3).dataSlice<float>();
+    for (int i = 0; i < 6; ++i) NEAR(back[i], x3[i], 1e-4);
+}
+
+static void test_property_18(const Context &ctx) {
+    // moe_router.zig:455-628, 100 random configurations
+    uint64_t seed = 18;
+    auto rnd = [&](uint32_t n) {
+        seed = seed * 6364136223846793005ull + 1442695040888963407ull;
+        return (uint32_t)((seed >> 33) % n);
+    };
+    const int tok[] = {1, 2, 3, 4, 5, 8}, exps[] = {4, 6, 8, 12, 16}, ks[] = {1, 2, 3, 4};
+    for (int it = 0; it < 100; ++it) {
+        const int T = tok[rnd(6)], E = exps[rnd(5)], K = std::min(ks[rnd(4)], E);
+        const bool normalize = rnd(2);
+        std::vector<float> s((size_t)T * E);
+        for (auto &v : s) v = (float)rnd(10001) / 10000.0f;
+        auto r = MoERouter::init({(size_t)E, (size_t)K, normalize}).topkRoute(ctx, Array::fromData(ctx, s.data(), {T, E}, DType::float32));
+        auto idx = r.indices.dataSlice<uint32_t>();
+        auto w = r.weights.dataSlice<float>();
+        for (int t = 0; t < T; ++t) {
+            std::vector<float> sorted(s.begin() + (size_t)t * E, s.begin() + (size_t)(t + 1) * E);
+            std::sort(sorted.rbegin(), sorted.rend());
+            float min_sel = 2.0f, sum = 0.0f;
+            std::set<uint32_t> sel;
+            for (int k = 0; k < K; ++k) {
+                const uint32_t e = idx[(size_t)t * K + k];
+                EXPECT(e < (uint32_t)E);
+                sel.insert(e);
+                EXPECT(s[(size_t)t * E + e] >= sorted[K - 1] - 1e-5f);
+                min_sel = std::min(min_sel, s[(size_t)t * E + e]);
+                sum += w[(size_t)t * K + k];
+                if (!normalize) NEAR(w[(size_t)t * K + k], s[(size_t)t * E + e], 1e-5);
+            }
+            EXPECT((int)sel.size() == K);
+            for (int e = 0; e < E; ++e)
+                if (!sel.count((uint32_t)e)) EXPECT(s[(size_t)t * E + e] <= min_sel + 1e-5f);
+            if (normalize) NEAR(sum, 1.0, 1e-4);
+        }
+    }
+}
+
+static void test_remap_smelt_batch(const Context &ctx) {
+    // expert_remap_test.zig: remap {0->0, 22->1, 31->2, 87->3} on [87,0,31,0,22,0] -> [3,0,2,0,1,0]
+    auto rb = ResidentExpertProvider::preloadRemap({0, 22, 31, 87}, 256);
+    const uint32_t idx[] = {87, 0, 31, 0, 22, 0};
+    Array d_remap = Array::fromData(ctx, rb.first.data(), {256}, DType::int32);
+    Array d_idx = Array::fromData(ctx, idx, {1, 6}, DType::uint32);
+    Array out(ctx, DType::uint32, {1, 6});
+    check(dmoe_remap_indices((uint32_t *)out.data(), (const int32_t *)d_remap.data(), (const uint32_t *)d_idx.data(), 6, 256, ctx.stream()));
+    auto got = out.dataSlice<uint32_t>();
+    const uint32_t want[] = {3, 0, 2, 0, 1, 0};
+    for (int i = 0; i < 6; ++i) EXPECT(got[i] == want[i]);
+    EXPECT(rb.second[22] == 0.0f && rb.second[23] == -1000.0f);
+
+    SmeltConfig sc;
+    sc.enabled = true;
+    sc.load_fraction = 0.2f;
+    auto mask = sc.buildMask(256);
+    EXPECT(std::count(mask.begin(), mask.end(), 1) == 51 && mask[0] == 1 && mask[255] == 1);
+    auto remap = SmeltConfig::buildRemap(mask);
+    int slot = 0;
+    for (int e = 0; e < 256; ++e) EXPECT(remap[e] == (mask[e] ? slot++ : 0));
+
+    // batch_builder: prefill requests first, then decode; positions continue each request
+    Request a, b, c;
+    a.state = Request::State::prefilling;
+    a.prompt_tokens = {10, 11, 12, 13, 14};
+    a.prefill_offset = 2;
+    b.state = Request::State::decoding;
+    b.prompt_tokens = {20, 21, 22};
+    b.generated_tokens = {30, 31};
+    c.state = Request::State::waiting;
+    c.prompt_tokens = {40};
+    auto br = batch_builder::build({&a, &c}, {&b});
+    EXPECT(br.total_tokens == 5 && br.num_requests == 3);
+    EXPECT(br.batched_tokens == std::vector<uint32_t>({12, 13, 14, 40, 31}));
+    EXPECT(br.position_ids == std::vector<int32_t>({2, 3, 4, 0, 4}));
+    EXPECT(br.request_offsets == std::vector<int32_t>({0, 3, 4, 5}));
+}
+
+static void test_layer_closed_form(const Context &ctx) {
+    // E=2, K=2, D=256, F=64, affine-4 g64 with every code 0: each dequantized weight equals its bias.
+    // Then gate = up = bg * sum(x), h = silu(gate) * up, every down output = bd * sum_f(h), and the layer
+    // output is (w0 + w1) * that, the same for every expert.
+    const int E = 2, K = 2, D = 256, F = 64, T = 3;
+    const float bg = 0.01f, bd = 0.02f;
+    std::vector<uint32_t> wz_g((size_t)E * F * D / 8, 0u), wz_d((size_t)E * D * F / 8, 0u);
+    std::vector<uint16_t> s_g((size_t)E * F * D / 64, bf16(0.5f)), b_g((size_t)E * F * D / 64, bf16(bg));
+    std::vector<uint16_t> s_d((size_t)E * D * F / 64, bf16(0.5f)), b_d((size_t)E * D * F / 64, bf16(bd));
+    QuantizedWeight gate{wz_g.data(), s_g.data(), b_g.data(), E, F, D, 64, 4, "affine"};
+    QuantizedWeight up = gate;
+    QuantizedWeight down{wz_d.data(), s_d.data(), b_d.data(), E, D, F, 64, 4, "affine"};
+    DSV4SwitchGLU::Options opt;
+    auto layer = std::make_unique<DSV4SwitchGLU>(ctx, D, F, K, gate, up, down, opt);
+    ResidentExpertProvider provider;
+    provider.addLayer(std::move(layer));
+
+    std::vector<uint16_t> x((size_t)T * D);
+    std::vector<double> sumx(T, 0.0);
+    for (int t = 0; t < T; ++t)
+        for (int d = 0; d < D; ++d) {
+            float v = 0.05f * (float)((t * 7 + d * 3) % 11 - 5);
+            x[(size_t)t * D + d] = bf16(v);
+            sumx[t] += from_bf16(bf16(v));
+        }
+    std::vector<float> scores((size_t)T * E);
+    for (int t = 0; t < T; ++t) {
+        scores[t * 2] = 0.3f + 0.1f * t;
+        scores[t * 2 + 1] = 0.6f - 0.1f * t;
+    }
+    DSV4MoE moe;
+    moe.gate.topk = K;
+    moe.gate.n_routed_experts = E;
+    moe.gate.route_scale = 1.5f;
+    moe.gate.scoring_func = ScoringFunc::sigmoid;
+    moe.stream_provider = &provider;
+    Array hidden = Array::fromData(ctx, x.data(), {1, T, D}, DType::bfloat16);
+    Array out = moe.forward(ctx, hidden, Array::fromData(ctx, scores.data(), {T, E}, DType::float32));
+    EXPECT(out.shape() == std::vector<int>({1, T, D}));
+    auto y = out.dataSlice<uint16_t>();
+    const double bgr = from_bf16(bf16(bg)), bdr = from_bf16(bf16(bd));
+    for (int t = 0; t < T; ++t) {
+        const double g = bgr * sumx[t], h = g / (1.0 + std::exp(-g)) * g;
+        const double want = 1.5 * bdr * F * h; // renormalised weights sum to 1, times route_scale
+        for (int d = 0; d < D; d += 37) NEAR(from_bf16(y[(size_t)t * D + d]), want, std::fabs(want) * 2e-2 + 1e-6);
+    }
+    // error path: an unknown layer index is reported, not ignored
+    bool threw = false;
+    try {
+        provider.forward(ctx, 5, hidden.reshaped({T, D}), Array(ctx, DType::uint32, {T, K}), Array(ctx, DType::float32, {T, K}));
+    } catch (const Error &) {
+        threw = true;
+    }
+    EXPECT(threw);
+}
+
+int main() {
+    try {
+        Context ctx(0);
+        test_topk(ctx);
+        test_expand_reduce(ctx);
+        test_property_18(ctx);
+        test_remap_smelt_batch(ctx);
+        test_layer_closed_form(ctx);
+        ctx.synchronize();
+    } catch (const Error &e) {
+        std::printf("dmoe::Error %d: %s\n", e.code, e.what());
+        return 2;
+    }
+    if (g_failed) {
+        std::printf("%d check(s) failed\n", g_failed);
+        return 1;
+    }
+    std::printf("ALL HOST TESTS PASSED\n");
+    return 0;
+}
