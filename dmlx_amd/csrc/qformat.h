@@ -53,7 +53,7 @@ __device__ __forceinline__ float e4m3_to_f32(uint32_t v) {
 // Fmt::kRowScale                      true: an f32 per-row scale is applied to the finished dot product
 // Fmt::load_meta(q, row_s, row_b, k0) scale/bias of the chunk starting at column k0 (MLX layout)
 // Fmt::load_meta_raw / meta_from_raw  the same in two steps: raw words while a load is in flight, f32 at use
-// Fmt::load_meta_packed / meta_from_packed   raw word(s) from the packed layout
+// Fmt::packed_meta_base/_lane/_step, load_meta_at, meta_from_packed   raw word(s) from the packed layout
 // Fmt::decode(raw, meta, out)         kVals/2 packed bf16 pairs, natural order, exact per-format arithmetic
 // Fmt::decode_fast                    same values through the gfx950 packed conversion instructions
 
@@ -71,11 +71,20 @@ struct FmtAffine4 {
         sb[0] = ((const uint16_t *)row_s)[g];
         sb[1] = row_b ? ((const uint16_t *)row_b)[g] : 0u;
     }
-    __device__ static __forceinline__ void load_meta_packed(const QView &q, size_t mat, int nb, int step, int h,
-                                                            int ln, uint32_t *sb) {
-        const int g = (step * 2 + h) * kVals / q.group, n_groups = q.cols / q.group;
-        sb[0] = *(const uint32_t *)(q.meta + mat * q.m_mat + (((size_t)nb * n_groups + g) * 32 + ln) * 4);
+    // Packed meta addressing, split into a part that is uniform over the wavefront (scalar arithmetic) and a
+    // per-lane constant: word ((nb * n_groups + g) * 32 + ln) with g = (step * 2 + h) * kVals / group. Group sizes
+    // are powers of two, and either a multiple of a step (g does not depend on h) or a divisor of a chunk, so g
+    // splits exactly into a step term and an h term.
+    __device__ static __forceinline__ size_t packed_meta_base(const QView &q, size_t mat, int nb) {
+        return mat * q.m_mat + (size_t)nb * (size_t)(q.cols >> __builtin_ctz(q.group)) * 128;
     }
+    __device__ static __forceinline__ uint32_t packed_meta_lane(const QView &q, int h, int ln) {
+        return (uint32_t)((((h * kVals) >> __builtin_ctz(q.group)) * 32 + ln) * 4);
+    }
+    __device__ static __forceinline__ uint32_t packed_meta_step(const QView &q, int step) {
+        return (uint32_t)(((step * 2 * kVals) >> __builtin_ctz(q.group)) * 128);
+    }
+    __device__ static __forceinline__ void load_meta_at(const uint8_t *p, uint32_t *sb) { sb[0] = *(const uint32_t *)p; }
     __device__ static __forceinline__ Meta meta_from_raw(const uint32_t *sb) {
         Meta m;
         m.s = bf16_bits_to_f32(sb[0]);
@@ -108,6 +117,19 @@ struct FmtAffine4 {
         decode_word(raw.w, m, out + 12);
     }
     __device__ static __forceinline__ void decode_fast(const uint4 &raw, Meta m, uint32_t *out) { decode(raw, m, out); }
+    // values (2q, 2q+1) of the chunk only, for callers that spread the decode between other instructions; q must
+    // run upwards through a chunk, `st` carries the two nibble planes of the current word between calls. The planes
+    // are made opaque so that the byte picks compile to v_cvt_f32_ubyteN instead of a bit-field extract each.
+    __device__ static __forceinline__ void decode_pair(const uint4 &raw, Meta m, int q, uint32_t *out, uint32_t *st) {
+        if (q % 4 == 0) {
+            const uint32_t w = (q / 4) == 0 ? raw.x : (q / 4) == 1 ? raw.y : (q / 4) == 2 ? raw.z : raw.w;
+            st[0] = w & 0x0f0f0f0fu;
+            st[1] = (w >> 4) & 0x0f0f0f0fu;
+            asm("" : "+v"(st[0]), "+v"(st[1]));
+        }
+        const uint32_t lo = (st[0] >> (8 * (q % 4))) & 0xffu, hi = (st[1] >> (8 * (q % 4))) & 0xffu;
+        out[q] = pack_bf16x2(fmaf((float)lo, m.s, m.b), fmaf((float)hi, m.s, m.b));
+    }
 };
 
 struct FmtAffine8 {
@@ -118,11 +140,20 @@ struct FmtAffine8 {
                                                          int k0, uint32_t *sb) {
         FmtAffine4::load_meta_raw(q, row_s, row_b, k0, sb);
     }
-    __device__ static __forceinline__ void load_meta_packed(const QView &q, size_t mat, int nb, int step, int h,
-                                                            int ln, uint32_t *sb) {
-        const int g = (step * 2 + h) * kVals / q.group, n_groups = q.cols / q.group;
-        sb[0] = *(const uint32_t *)(q.meta + mat * q.m_mat + (((size_t)nb * n_groups + g) * 32 + ln) * 4);
+    // Packed meta addressing, split into a part that is uniform over the wavefront (scalar arithmetic) and a
+    // per-lane constant: word ((nb * n_groups + g) * 32 + ln) with g = (step * 2 + h) * kVals / group. Group sizes
+    // are powers of two, and either a multiple of a step (g does not depend on h) or a divisor of a chunk, so g
+    // splits exactly into a step term and an h term.
+    __device__ static __forceinline__ size_t packed_meta_base(const QView &q, size_t mat, int nb) {
+        return mat * q.m_mat + (size_t)nb * (size_t)(q.cols >> __builtin_ctz(q.group)) * 128;
     }
+    __device__ static __forceinline__ uint32_t packed_meta_lane(const QView &q, int h, int ln) {
+        return (uint32_t)((((h * kVals) >> __builtin_ctz(q.group)) * 32 + ln) * 4);
+    }
+    __device__ static __forceinline__ uint32_t packed_meta_step(const QView &q, int step) {
+        return (uint32_t)(((step * 2 * kVals) >> __builtin_ctz(q.group)) * 128);
+    }
+    __device__ static __forceinline__ void load_meta_at(const uint8_t *p, uint32_t *sb) { sb[0] = *(const uint32_t *)p; }
     __device__ static __forceinline__ Meta meta_from_raw(const uint32_t *sb) { return FmtAffine4::meta_from_raw(sb); }
     __device__ static __forceinline__ Meta meta_from_packed(const uint32_t *sb) { return FmtAffine4::meta_from_packed(sb); }
     __device__ static __forceinline__ Meta load_meta(const QView &q, const uint8_t *row_s, const uint8_t *row_b,
@@ -140,6 +171,11 @@ struct FmtAffine8 {
         decode_word(raw.w, m, out + 6);
     }
     __device__ static __forceinline__ void decode_fast(const uint4 &raw, Meta m, uint32_t *out) { decode(raw, m, out); }
+    __device__ static __forceinline__ void decode_pair(const uint4 &raw, Meta m, int q, uint32_t *out, uint32_t *) {
+        const uint32_t w = (q / 2) == 0 ? raw.x : (q / 2) == 1 ? raw.y : (q / 2) == 2 ? raw.z : raw.w;
+        const uint32_t v = w >> (16 * (q % 2));
+        out[q] = pack_bf16x2(fmaf((float)(v & 0xffu), m.s, m.b), fmaf((float)((v >> 8) & 0xffu), m.s, m.b));
+    }
 };
 
 struct FmtMxfp4 {
@@ -151,11 +187,13 @@ struct FmtMxfp4 {
         sb[0] = row_s[k0 >> 5];
         sb[1] = 0u;
     }
-    __device__ static __forceinline__ void load_meta_packed(const QView &q, size_t mat, int nb, int step, int h,
-                                                            int ln, uint32_t *sb) {
-        const int n_steps = q.cols / (2 * kVals);
-        sb[0] = q.meta[mat * q.m_mat + (((size_t)nb * n_steps + step) * 2 + h) * 32 + ln];
+    // packed meta: byte ((nb * n_steps + step) * 2 + h) * 32 + ln
+    __device__ static __forceinline__ size_t packed_meta_base(const QView &q, size_t mat, int nb) {
+        return mat * q.m_mat + (size_t)nb * (size_t)(q.cols / (2 * kVals)) * 64;
     }
+    __device__ static __forceinline__ uint32_t packed_meta_lane(const QView &, int h, int ln) { return (uint32_t)(h * 32 + ln); }
+    __device__ static __forceinline__ uint32_t packed_meta_step(const QView &, int step) { return (uint32_t)step * 64u; }
+    __device__ static __forceinline__ void load_meta_at(const uint8_t *p, uint32_t *sb) { sb[0] = *p; }
     __device__ static __forceinline__ Meta meta_from_raw(const uint32_t *sb) {
         Meta m;
         m.s = e8m0_to_f32(sb[0]);
@@ -196,6 +234,15 @@ struct FmtMxfp4 {
         fast_word(raw.z, m.s, out + 8);
         fast_word(raw.w, m.s, out + 12);
     }
+    __device__ static __forceinline__ void decode_pair(const uint4 &raw, Meta m, int q, uint32_t *out, uint32_t *) {
+        const uint32_t w = (q / 4) == 0 ? raw.x : (q / 4) == 1 ? raw.y : (q / 4) == 2 ? raw.z : raw.w;
+        switch (q % 4) { // the byte selector is an immediate
+        case 0: out[q] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, m.s, 0)); break;
+        case 1: out[q] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, m.s, 1)); break;
+        case 2: out[q] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, m.s, 2)); break;
+        default: out[q] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, m.s, 3)); break;
+        }
+    }
 };
 
 struct FmtFp8Row {
@@ -207,9 +254,10 @@ struct FmtFp8Row {
         sb[0] = 0u;
         sb[1] = 0u;
     }
-    __device__ static __forceinline__ void load_meta_packed(const QView &, size_t, int, int, int, int, uint32_t *sb) {
-        sb[0] = 0u;
-    }
+    __device__ static __forceinline__ size_t packed_meta_base(const QView &, size_t, int) { return 0; }
+    __device__ static __forceinline__ uint32_t packed_meta_lane(const QView &, int, int) { return 0u; }
+    __device__ static __forceinline__ uint32_t packed_meta_step(const QView &, int) { return 0u; }
+    __device__ static __forceinline__ void load_meta_at(const uint8_t *, uint32_t *sb) { sb[0] = 0u; }
     __device__ static __forceinline__ Meta meta_from_raw(const uint32_t *) {
         Meta m;
         m.s = 1.0f;
@@ -240,6 +288,11 @@ struct FmtFp8Row {
         fast_word(raw.z, out + 4);
         fast_word(raw.w, out + 6);
     }
+    __device__ static __forceinline__ void decode_pair(const uint4 &raw, Meta, int q, uint32_t *out, uint32_t *) {
+        const uint32_t w = (q / 2) == 0 ? raw.x : (q / 2) == 1 ? raw.y : (q / 2) == 2 ? raw.z : raw.w;
+        if (q % 2 == 0) out[q] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false));
+        else out[q] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true));
+    }
 };
 
 // dispatch a callable templated on the format: f.template operator()<Fmt>()
@@ -256,33 +309,37 @@ inline int dispatch_format(const QView &q, F &&f) {
 // ---- addressing of one lane's chunk stream (lane = (ln = row within the 32-row block, h = step half)) ----
 template <typename Fmt, bool PACKED>
 struct ChunkStream {
-    const uint8_t *w;     // first chunk of this lane
-    const uint8_t *srow;  // MLX layout: this row's scales / biases
+    // packed layout: w / mbase are uniform over the wavefront, the lane's share is a 32-bit offset (so the loads can
+    // take a scalar base); MLX layout: w is this lane's first chunk, srow / brow its row's scales / biases
+    const uint8_t *w;
+    const uint8_t *mbase;
+    const uint8_t *srow;
     const uint8_t *brow;
-    size_t mat;
-    int nb, h, ln;
-    size_t stride;        // bytes between consecutive steps
+    uint32_t wlane, mlane;
+    int h;
 
-    __device__ __forceinline__ void init(const QView &q, size_t mat_, int row_block, int ln_, int h_, int n_clamped) {
-        mat = mat_;
-        nb = row_block;
+    __device__ __forceinline__ void init(const QView &q, size_t mat, int row_block, int ln, int h_, int n_clamped) {
         h = h_;
-        ln = ln_;
         if (PACKED) {
             const int n_steps = q.cols / (2 * Fmt::kVals);
-            w = q.w + mat * q.w_mat + ((size_t)nb * n_steps * 2 + h) * 512 + (size_t)ln * 16;
-            stride = 1024;
+            w = q.w + mat * q.w_mat + (size_t)row_block * n_steps * 1024;
+            wlane = (uint32_t)(h * 32 + ln) * 16u;
+            mbase = q.meta + Fmt::packed_meta_base(q, mat, row_block);
+            mlane = Fmt::packed_meta_lane(q, h, ln);
             srow = brow = nullptr;
         } else {
             w = q.w + mat * q.w_mat + (size_t)n_clamped * q.w_row + (size_t)h * 16;
-            stride = 32;
+            wlane = mlane = 0;
+            mbase = nullptr;
             srow = q.scales + mat * q.s_mat + (size_t)n_clamped * q.s_row;
             brow = q.biases ? q.biases + mat * q.s_mat + (size_t)n_clamped * q.s_row : nullptr;
         }
     }
-    __device__ __forceinline__ uint4 load_chunk(int step) const { return *(const uint4 *)(w + (size_t)step * stride); }
+    __device__ __forceinline__ uint4 load_chunk(int step) const {
+        return *(const uint4 *)(w + (size_t)step * (PACKED ? 1024 : 32) + wlane);
+    }
     __device__ __forceinline__ void load_meta(const QView &q, int step, uint32_t *sb) const {
-        if (PACKED) Fmt::load_meta_packed(q, mat, nb, step, h, ln, sb);
+        if (PACKED) Fmt::load_meta_at(mbase + Fmt::packed_meta_step(q, step) + mlane, sb);
         else Fmt::load_meta_raw(q, srow, brow, (step * 2 + h) * Fmt::kVals, sb);
     }
     __device__ static __forceinline__ Meta meta(const uint32_t *sb) {

@@ -6,13 +6,16 @@
 // v_mfma_f32_32x32x16_bf16: lane (n = lane % 32, h = lane / 32) loads the 16-byte chunk h of weight row
 // n for a reduction step, i.e. exactly the values its MFMA operand slots need. Those loads run through a
 // register ring kMfmaRing steps deep. The activations of the tile's rows are shared by all wavefronts
-// through LDS (double-buffered blocks of two steps, padded rows, one barrier per block) and feed the B
-// operand, so the accumulators hold out^T: lane = token row, registers = 16 output columns in runs of
-// four, which lets the epilogue store 8 bytes at a time.
+// through LDS (double-buffered blocks of kMfmaRing steps, padded rows, one barrier per block) and feed
+// the B operand, so the accumulators hold out^T: lane = token row, registers = 16 output columns in runs
+// of four, which lets the epilogue store 8 bytes at a time.
 //
-// The loop is software-pipelined by hand: while the matrix core works through the 32 MFMAs of step s
-// with the weights decoded during step s-1, the vector ALU decodes the weights of step s+1, so the two
-// pipes overlap inside a single wavefront (the register budget leaves one wavefront per SIMD).
+// The loop is software-pipelined by hand: while the matrix core works through the MFMAs of step s with
+// the weights decoded during step s-1, the vector ALU decodes the weights of step s+1. A wavefront
+// issues in order, so the two pipes only overlap if the instruction stream alternates between them:
+// the step is written as units of [one MFMA | one slice of the decode] separated by scheduling barriers.
+// Measured on MI355X a unit costs max(34, 13 + 4 * vector instructions) cycles, which is why the decode
+// is kept under six instructions per MFMA.
 //
 // A reduction step covers 2 chunks (64 values for 4-bit formats, 32 for 8-bit ones). The order of the
 // products inside a step is permuted identically for both operands, which a sum does not see.
@@ -24,37 +27,32 @@
 namespace dmoe {
 
 constexpr int kMfmaWaves = 4;
-constexpr int kMfmaRing = 4;          // weight steps held in registers (kMfmaRing - 1 in flight)
-constexpr int kStepsPerBlock = 2;     // reduction steps per LDS activation block
+constexpr int kMfmaRing = 4; // weight steps held in registers = reduction steps per LDS activation block
 
 template <typename Fmt>
 struct MfmaGeom {
     static constexpr int KV = Fmt::kVals;          // values per 16-byte chunk
     static constexpr int KSTEP = 2 * KV;           // reduction elements per step
     static constexpr int NJ = KV / 8;              // MFMAs (K = 16) per step and tile
-    static constexpr int KB = kStepsPerBlock * KSTEP; // reduction elements per activation block
+    static constexpr int KB = kMfmaRing * KSTEP;   // reduction elements per activation block
     static constexpr int LDA = KB + 8;             // LDS row pitch in bf16 elements (+16 bytes: conflict-free b128 reads)
-    static constexpr int CH = KB / 8;              // 16-byte pieces per activation row and block
-    static constexpr int RP = 256 / CH;            // rows staged per pass
-    static constexpr int PASSES = kMfmaTileM / RP;
-    static constexpr size_t kLdsBytes = 2ull * kMfmaTileM * LDA * 2;
+    static constexpr int NI = KB / 64;             // 128-byte granules per activation row and block
+    static constexpr size_t kBufBytes = (size_t)kMfmaTileM * LDA * 2;
+    static constexpr size_t kLdsBytes = 2 * kBufBytes;
+    static_assert(NJ % 2 == 0 && NI % 2 == 0, "fragment ping-pong and half-block staging need even counts");
 };
 
-// One tile with MT 32-row MFMA tiles (MT is a template parameter so that the reduction loop is straight-line
-// code: the scheduler can then interleave the decode arithmetic with the matrix instructions).
+// One tile with MT 32-row MFMA tiles (MT is a template parameter so that the reduction loop is straight-line code).
 template <typename Fmt, bool GATE_UP, bool PACKED, int MT>
-__device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint16_t *mfma_lds) {
+__device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint8_t *lds) {
     using CS = ChunkStream<Fmt, PACKED>;
     using G = MfmaGeom<Fmt>;
-    constexpr int KV = G::KV, KSTEP = G::KSTEP, NJ = G::NJ, KB = G::KB, LDA = G::LDA, CH = G::CH, RP = G::RP,
-                  PASSES = G::PASSES;
+    constexpr int KV = G::KV, KSTEP = G::KSTEP, NJ = G::NJ, KB = G::KB, LDA = G::LDA, NI = G::NI;
     constexpr int NT = 2; // 32-column MFMA tiles per wavefront
-    constexpr int n_mt = MT;
     const int tid = (int)threadIdx.x, lane = tid & 63, ln = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int cols = g.b0.cols, n_out = g.b0.rows;
     const int n_steps = cols / KSTEP;
-    const int n_blk = (n_steps + kStepsPerBlock - 1) / kStepsPerBlock;
     const size_t e = t.expert;
 
     // ---- this wavefront's weight rows -------------------------------------------------------------------
@@ -81,39 +79,45 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
             cs[nt].load_meta(b, step, ring_sb[slot_][nt]);
         }
     };
-    // weight loads depend on the tile only: start them first
+    // weight loads depend on the tile only: start them first (steps past the end are clamped, their data unused)
 #pragma unroll
-    for (int j = 0; j < kMfmaRing; ++j)
-        if (j < n_steps) load_b(j, j);
+    for (int j = 0; j < kMfmaRing; ++j) load_b(j < n_steps ? j : n_steps - 1, j);
 
-    // ---- activation staging: thread -> (row within pass, 16-byte piece) ------------------------------
-    const int a_piece = tid % CH, a_row = tid / CH;
-    constexpr int rows_used = n_mt * 32;
-    const uint16_t *a_src[PASSES];
+    // ---- activation staging ------------------------------------------------------------------------------
+    // thread -> (row a_row + 32 * p, 16-byte piece a_piece of each 128-byte granule): eight lanes cover one full
+    // cache line of a row. A block is staged in two halves (granules [0, NI/2) and [NI/2, NI)) so that only half of
+    // it sits in registers at a time. Rows past the segment end alias the tile's first row; they are never stored.
+    constexpr int rows_used = MT * 32;
+    const int a_piece = tid & 7, a_row = tid >> 3;
+    const uint16_t *a_ptr[4];
 #pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-        const int r = a_row + p * RP;
-        a_src[p] = nullptr;
-        if (r < (int)t.nrows) {
-            const uint32_t pr = t.row0 + (uint32_t)r;
-            const size_t src = g.a_rows ? g.a_rows[pr] : pr;
-            a_src[p] = g.a + src * (size_t)cols + a_piece * 8;
-        }
+    for (int p = 0; p < 4; ++p) {
+        const int r = a_row + 32 * p;
+        const uint32_t pr = t.row0 + (uint32_t)(r < (int)t.nrows ? r : 0);
+        const size_t src = g.a_rows ? g.a_rows[pr] : pr;
+        a_ptr[p] = g.a + src * (size_t)cols + a_piece * 8;
     }
-    uint4 a_reg[PASSES];
-    auto load_a = [&](int blk) {
+    uint4 a_reg[4][NI / 2];
+    auto load_a = [&](int blk, int half) {
 #pragma unroll
-        for (int p = 0; p < PASSES; ++p) {
-            a_reg[p] = make_uint4(0, 0, 0, 0);
-            // the last block may be half a block wide (n_steps odd): pieces past the row end stay zero
-            if (a_src[p] && blk * KB + a_piece * 8 < cols) a_reg[p] = *(const uint4 *)(a_src[p] + (size_t)blk * KB);
+        for (int ii = 0; ii < NI / 2; ++ii) {
+            const int k0 = blk * KB + (half * (NI / 2) + ii) * 64; // uniform
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                if (p * 32 >= rows_used) continue;
+                a_reg[p][ii] = make_uint4(0, 0, 0, 0); // past the row end (the surplus steps of the last trip): zeros
+                if (k0 < cols) a_reg[p][ii] = *(const uint4 *)(a_ptr[p] + k0); // rows are whole granules long
+            }
         }
     };
-    auto store_a = [&](int buf) {
+    uint8_t *const a_wr = lds + ((size_t)a_row * LDA + a_piece * 8) * 2;
+    auto store_a = [&](uint32_t buf_off, int half) {
 #pragma unroll
-        for (int p = 0; p < PASSES; ++p)
-            if (p * RP < rows_used) // rows of MFMA tiles that are not computed are never read
-                *(uint4 *)&mfma_lds[((size_t)buf * kMfmaTileM + a_row + p * RP) * LDA + a_piece * 8] = a_reg[p];
+        for (int ii = 0; ii < NI / 2; ++ii)
+#pragma unroll
+            for (int p = 0; p < 4; ++p)
+                if (p * 32 < rows_used) // rows of MFMA tiles that are not computed are never read
+                    *(uint4 *)(a_wr + buf_off + ((size_t)p * 32 * LDA + (half * (NI / 2) + ii) * 64) * 2) = a_reg[p][ii];
     };
 
     f32x16_t acc[MT][NT];
@@ -125,88 +129,105 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
             for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0.0f;
 
     uint32_t wp[2][NT][KV / 2]; // decoded weights of the current / next step
-    auto decode = [&](int slot_, int which) {
+    bf16x8_t xf[2][MT];         // activation fragments of the current / next MFMA group
+    const uint8_t *const x_rd = lds + ((size_t)ln * LDA + h * KV) * 2;
+    auto read_x = [&](uint32_t buf_off, int sb, int j, int pp) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) Fmt::decode_fast(ring_raw[slot_][nt], CS::meta(ring_sb[slot_][nt]), wp[which][nt]);
+        for (int mt = 0; mt < MT; ++mt) {
+            uint4 q = *(const uint4 *)(x_rd + buf_off + ((size_t)mt * 32 * LDA + sb * KSTEP + 8 * j) * 2);
+            xf[pp][mt] = __builtin_bit_cast(bf16x8_t, q);
+        }
     };
-    // One reduction step: the MT*NT*NJ matrix instructions of step s (weights wp[which], decoded one step
-    // earlier) with the vector-ALU decode of step s+1 spread between them. Activation fragments are read
-    // from LDS one MFMA group ahead. The scheduling-group barriers at the end pin that interleaving; left to
-    // itself the compiler emits the whole decode first and the matrix instructions after it.
-    auto step_body = [&](int slot_next, int which, int buf, int sb) {
-        bf16x8_t xf[2][MT];
-        auto read_x = [&](int j, int pp) {
+    // One reduction step: MT*NT*NJ units of [one MFMA of step s | the decode of a slice of step s+1's weights], with
+    // a scheduling barrier after every unit (left to itself the compiler emits the whole decode first and the
+    // MFMAs after it, which serialises the two pipes). Activation fragments are read from LDS one MFMA group
+    // (MT*NT units) ahead of their use; the first group of the next step of the same block is fetched during the
+    // last group of this one.
+    auto step_body = [&](int slot_next, int which, uint32_t buf_off, int sb) {
+        constexpr int NU = NJ * MT * NT; // units
+        constexpr int NP = NT * (KV / 2); // packed pairs to decode for the next step
+        Meta meta_next[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) meta_next[nt] = CS::meta(ring_sb[slot_next][nt]);
+        uint32_t dstate[2] = {0, 0};
+        if (sb == 0) {
+            read_x(buf_off, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-                uint4 q = *(const uint4 *)&mfma_lds[((size_t)buf * kMfmaTileM + mt * 32 + ln) * LDA + sb * KSTEP + h * KV + 8 * j];
-                xf[pp][mt] = __builtin_bit_cast(bf16x8_t, q);
-            }
-        };
-        read_x(0, 0);
-        decode(slot_next, which ^ 1);
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            if (j + 1 < NJ) read_x(j + 1, (j + 1) & 1);
-            bf16x8_t wf[NT];
+                for (int nt = 0; nt < NT; ++nt) {
+                    const int u = (j * MT + mt) * NT + nt;
+                    if (mt == 0 && nt == 0) {
+                        if (j + 1 < NJ) read_x(buf_off, sb, j + 1, (j + 1) & 1);
+                        else if (sb + 1 < kMfmaRing) read_x(buf_off, sb + 1, 0, 0);
+                    }
+                    uint4 q = make_uint4(wp[which][nt][4 * j], wp[which][nt][4 * j + 1], wp[which][nt][4 * j + 2],
+                                         wp[which][nt][4 * j + 3]);
+                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, q), xf[j & 1][mt],
+                                                                          acc[mt][nt], 0, 0, 0);
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                uint4 q = make_uint4(wp[which][nt][4 * j], wp[which][nt][4 * j + 1], wp[which][nt][4 * j + 2],
-                                     wp[which][nt][4 * j + 3]);
-                wf[nt] = __builtin_bit_cast(bf16x8_t, q);
-            }
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[nt], xf[j & 1][mt], acc[mt][nt], 0, 0, 0);
-        }
-        constexpr int kMfmas = NJ * MT * NT;
-        constexpr int kValuPerMfma = (Fmt::kDecodeOps * NT + kMfmas - 1) / kMfmas;
-        __builtin_amdgcn_sched_group_barrier(0x100, MT, 0); // LDS reads of the first group
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            if (j + 1 < NJ) __builtin_amdgcn_sched_group_barrier(0x100, MT, 0);
-#pragma unroll
-            for (int k = 0; k < MT * NT; ++k) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            // one matrix instruction
-                __builtin_amdgcn_sched_group_barrier(0x002, kValuPerMfma, 0); // its share of the decode
-            }
-        }
-    };
-
-    load_a(0);
-    store_a(0);
-    __syncthreads();
-    decode(0, 0);
-
-    // kMfmaRing steps per trip so that ring slots, LDS buffers and the wp pair are compile-time indices. Full trips
-    // run without any guard (loads past the end are clamped onto valid memory and their data is never used), so a
-    // trip is straight-line code between barriers; a trailing partial trip runs the guarded copy.
-    static_assert(kMfmaRing % (2 * kStepsPerBlock) == 0, "ring must cover whole pairs of activation blocks");
-    auto trip = [&](int s0, auto guard) {
-        constexpr bool GUARD = decltype(guard)::value;
-#pragma unroll
-        for (int j = 0; j < kMfmaRing; ++j) {
-            const int s = s0 + j;
-            if (!GUARD || s < n_steps) {
-                const int blk = s / kStepsPerBlock;
-                const int sb = j % kStepsPerBlock, buf = (j / kStepsPerBlock) & 1;
-                const int s_ahead = s + kMfmaRing < n_steps ? s + kMfmaRing : n_steps - 1;
-                load_b(s_ahead, j); // slot j was decoded one step ago
-                if (sb == 0) load_a(blk + 1 < n_blk ? blk + 1 : n_blk - 1);
-                step_body((j + 1) % kMfmaRing, j & 1, buf, sb);
-                if (sb == kStepsPerBlock - 1 || (GUARD && s + 1 == n_steps)) {
-                    store_a(buf ^ 1);
-                    __syncthreads();
+                    for (int p = u * NP / NU; p < (u + 1) * NP / NU; ++p) {
+                        Fmt::decode_pair(ring_raw[slot_next][p / (KV / 2)], meta_next[p / (KV / 2)], p % (KV / 2),
+                                         wp[which ^ 1][p / (KV / 2)], dstate);
+                        // pin the slice here: without it the optimiser sinks the decode of a trip's last step
+                        // into the head of the next trip, where nothing overlaps it
+                        asm volatile("" : "+v"(wp[which ^ 1][p / (KV / 2)][p % (KV / 2)]));
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
         }
     };
-    int s0 = 0;
-#pragma unroll 1
-    for (; s0 + kMfmaRing <= n_steps; s0 += kMfmaRing) trip(s0, std::false_type{});
-    if (s0 < n_steps) trip(s0, std::true_type{});
 
+    load_a(0, 0);
+    store_a(0, 0);
+    load_a(0, 1);
+    store_a(0, 1);
+    __syncthreads();
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) Fmt::decode_fast(ring_raw[0][nt], CS::meta(ring_sb[0][nt]), wp[0][nt]);
+
+    // The loop always runs whole trips of kMfmaRing steps (one activation block): past the end of the reduction the
+    // activation blocks are zero-filled and the weight loads are clamped onto the last valid step, so the surplus
+    // steps add 0 * w and the loop body is one straight line with no guarded copy. While a trip computes from one
+    // LDS buffer, the next block is staged into the other in two halves; one barrier per trip publishes it.
+    const int n_trips = (n_steps + kMfmaRing - 1) / kMfmaRing;
+    static_assert(kMfmaRing == 4, "the staging schedule below is written for four steps per trip");
+#ifdef DMOE_MFMA_CLOCK // debug aid: cycles per reduction step of a few workgroups
+    const long long exp_t0 = clock64();
+#endif
+#pragma unroll 1
+    for (int trip = 0; trip < n_trips; ++trip) {
+        const int s0 = trip * kMfmaRing;
+        const uint32_t rd_off = (trip & 1) ? (uint32_t)G::kBufBytes : 0u, wr_off = (uint32_t)G::kBufBytes - rd_off;
+        const bool more = trip + 1 < n_trips; // uniform
+#pragma unroll
+        for (int j = 0; j < kMfmaRing; ++j) {
+            const int s = s0 + j;
+            const int s_ahead = s + kMfmaRing < n_steps ? s + kMfmaRing : n_steps - 1;
+            load_b(s_ahead, j); // slot j was decoded one step ago
+            if (j == 0 && more) load_a(trip + 1, 0);
+            step_body((j + 1) % kMfmaRing, j & 1, rd_off, j);
+            if (j == 1 && more) {
+                store_a(wr_off, 0);
+                load_a(trip + 1, 1);
+            }
+            if (j == 3) {
+                if (more) store_a(wr_off, 1);
+                __syncthreads();
+            }
+        }
+    }
+
+#ifdef DMOE_MFMA_CLOCK // debug aid: cycles per reduction step of a few workgroups
+    if (blockIdx.x == 3 && (blockIdx.y % 97) == 5 && tid == 0)
+        printf("MT %d gate_up %d slot %d steps %d clk/step %lld\n", MT, (int)GATE_UP, (int)blockIdx.y, n_steps,
+               (clock64() - exp_t0) / n_steps);
+#endif
     // ---- epilogue: lane = token row (ln), registers r -> output column 8*(r/4) + 4*h + r%4 -------------
     if (!wave_on) return;
 #pragma unroll
@@ -259,7 +280,7 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
 
 template <typename Fmt, bool GATE_UP, bool PACKED>
 __global__ __launch_bounds__(kMfmaWaves * 64) void qgemm_mfma_kernel(GemmArgs g) {
-    extern __shared__ __attribute__((aligned(16))) uint16_t mfma_lds[]; // As[2][kMfmaTileM][LDA]
+    extern __shared__ __attribute__((aligned(16))) uint8_t mfma_lds[]; // bf16 As[2][kMfmaTileM][LDA]
     Tile t;
     const uint32_t slot = blockIdx.y;
     if (g.tiles) {
@@ -273,7 +294,8 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void qgemm_mfma_kernel(GemmArgs g)
         uint32_t left = (uint32_t)g.dense_rows - t.row0;
         t.nrows = left < (uint32_t)kMfmaTileM ? left : (uint32_t)kMfmaTileM;
     }
-    switch ((t.nrows + 31u) >> 5) { // uniform over the workgroup
+    // the tile is the same for the whole workgroup; saying so keeps the four variants apart as scalar branches
+    switch (__builtin_amdgcn_readfirstlane((int)((t.nrows + 31u) >> 5))) {
     case 1: mfma_tile<Fmt, GATE_UP, PACKED, 1>(g, t, mfma_lds); break;
     case 2: mfma_tile<Fmt, GATE_UP, PACKED, 2>(g, t, mfma_lds); break;
     case 3: mfma_tile<Fmt, GATE_UP, PACKED, 3>(g, t, mfma_lds); break;
@@ -284,7 +306,7 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void qgemm_mfma_kernel(GemmArgs g)
 
 bool qgemm_mfma_supports(const QView &b) {
     int vals = (b.mode == DMOE_QUANT_AFFINE && b.bits == 4) || b.mode == DMOE_QUANT_MXFP4 ? 32 : 16;
-    return b.cols % (2 * vals) == 0 && b.rows % 4 == 0;
+    return b.cols % (2 * vals) == 0 && b.cols % 64 == 0 && b.rows % 4 == 0; // activation rows are staged in 128-byte granules
 }
 
 struct MfmaLaunch {
