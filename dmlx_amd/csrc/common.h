@@ -198,7 +198,7 @@ __device__ __forceinline__ float limited_swiglu(float g, float u, float limit) {
         g = fminf(g, limit);
         u = fminf(fmaxf(u, -limit), limit);
     }
-    float silu = g / (1.0f + __expf(-g));
+    float silu = g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)); // 1-ulp reciprocal; the result is rounded to bf16
     return silu * u;
 }
 

@@ -87,7 +87,6 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
     // thread -> (row a_row + 32 * p, 16-byte piece a_piece of each 128-byte granule): eight lanes cover one full
     // cache line of a row. A block is staged in two halves (granules [0, NI/2) and [NI/2, NI)) so that only half of
     // it sits in registers at a time. Rows past the segment end alias the tile's first row; they are never stored.
-    constexpr int rows_used = MT * 32;
     const int a_piece = tid & 7, a_row = tid >> 3;
     const uint16_t *a_ptr[4];
 #pragma unroll
@@ -97,27 +96,36 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
         const size_t src = g.a_rows ? g.a_rows[pr] : pr;
         a_ptr[p] = g.a + src * (size_t)cols + a_piece * 8;
     }
-    uint4 a_reg[4][NI / 2];
-    auto load_a = [&](int blk, int half) {
-#pragma unroll
-        for (int ii = 0; ii < NI / 2; ++ii) {
-            const int k0 = blk * KB + (half * (NI / 2) + ii) * 64; // uniform
-#pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                if (p * 32 >= rows_used) continue;
-                a_reg[p][ii] = make_uint4(0, 0, 0, 0); // past the row end (the surplus steps of the last trip): zeros
-                if (k0 < cols) a_reg[p][ii] = *(const uint4 *)(a_ptr[p] + k0); // rows are whole granules long
-            }
-        }
+    // One staging operation = one 16-byte load (or LDS store) per thread: piece ii of half `half` for the rows of
+    // pass p. Both halves of a block have registers of their own, so that every load has two reduction steps to
+    // arrive before its store, and the operations are issued one at a time between the MFMAs (a burst of them
+    // stalls the wavefront's in-order issue while the memory pipes drain: ~50 cycles per LDS store).
+    constexpr int kOpsPerHalf = MT * (NI / 2);
+    typedef uint32_t u32x4_t __attribute__((ext_vector_type(4))); // a first-class value, unlike HIP's uint4 struct
+    u32x4_t a_reg[2 * MT * (NI / 2)];
+    auto load_a_op = [&](int blk, int half, int op) {
+        const int p = op % MT, ii = op / MT;
+        // uniform, clamped into the row: granules past the row end (the surplus steps of the last trip, or the
+        // block after the last one) re-read the last granule and are zeroed in LDS by zero_tail
+        int k0 = blk * KB + (half * (NI / 2) + ii) * 64;
+        k0 = k0 < cols - 64 ? k0 : cols - 64;
+        a_reg[(half * MT + p) * (NI / 2) + ii] = *(const u32x4_t *)(a_ptr[p] + k0);
     };
     uint8_t *const a_wr = lds + ((size_t)a_row * LDA + a_piece * 8) * 2;
-    auto store_a = [&](uint32_t buf_off, int half) {
+    auto store_a_op = [&](uint32_t buf_off, int half, int op) {
+        const int p = op % MT, ii = op / MT;
+        *(u32x4_t *)(a_wr + buf_off + ((size_t)p * 32 * LDA + (half * (NI / 2) + ii) * 64) * 2) =
+            a_reg[(half * MT + p) * (NI / 2) + ii];
+    };
+    // zero the granules of block blk that lie past the row end (only the last block of a reduction whose step count
+    // is not a multiple of the trip length has any); runs after this thread's own stores to the same addresses
+    auto zero_tail = [&](uint32_t buf_off, int blk) {
 #pragma unroll
-        for (int ii = 0; ii < NI / 2; ++ii)
+        for (int i = 0; i < NI; ++i)
+            if (blk * KB + i * 64 >= cols)
 #pragma unroll
-            for (int p = 0; p < 4; ++p)
-                if (p * 32 < rows_used) // rows of MFMA tiles that are not computed are never read
-                    *(uint4 *)(a_wr + buf_off + ((size_t)p * 32 * LDA + (half * (NI / 2) + ii) * 64) * 2) = a_reg[p][ii];
+                for (int p = 0; p < MT; ++p)
+                    *(uint4 *)(a_wr + buf_off + ((size_t)p * 32 * LDA + i * 64) * 2) = make_uint4(0, 0, 0, 0);
     };
 
     f32x16_t acc[MT][NT];
@@ -131,19 +139,16 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
     uint32_t wp[2][NT][KV / 2]; // decoded weights of the current / next step
     bf16x8_t xf[2][MT];         // activation fragments of the current / next MFMA group
     const uint8_t *const x_rd = lds + ((size_t)ln * LDA + h * KV) * 2;
-    auto read_x = [&](uint32_t buf_off, int sb, int j, int pp) {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            uint4 q = *(const uint4 *)(x_rd + buf_off + ((size_t)mt * 32 * LDA + sb * KSTEP + 8 * j) * 2);
-            xf[pp][mt] = __builtin_bit_cast(bf16x8_t, q);
-        }
+    auto read_x = [&](uint32_t buf_off, int sb, int j, int mt, int pp) {
+        uint4 q = *(const uint4 *)(x_rd + buf_off + ((size_t)mt * 32 * LDA + sb * KSTEP + 8 * j) * 2);
+        xf[pp][mt] = __builtin_bit_cast(bf16x8_t, q);
     };
     // One reduction step: MT*NT*NJ units of [one MFMA of step s | the decode of a slice of step s+1's weights], with
     // a scheduling barrier after every unit (left to itself the compiler emits the whole decode first and the
     // MFMAs after it, which serialises the two pipes). Activation fragments are read from LDS one MFMA group
     // (MT*NT units) ahead of their use; the first group of the next step of the same block is fetched during the
     // last group of this one.
-    auto step_body = [&](int slot_next, int which, uint32_t buf_off, int sb) {
+    auto step_body = [&](int slot_next, int which, uint32_t buf_off, int sb, auto side) {
         constexpr int NU = NJ * MT * NT; // units
         constexpr int NP = NT * (KV / 2); // packed pairs to decode for the next step
         Meta meta_next[NT];
@@ -151,7 +156,8 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
         for (int nt = 0; nt < NT; ++nt) meta_next[nt] = CS::meta(ring_sb[slot_next][nt]);
         uint32_t dstate[2] = {0, 0};
         if (sb == 0) {
-            read_x(buf_off, 0, 0, 0);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) read_x(buf_off, 0, 0, mt, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
@@ -161,10 +167,11 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
                     const int u = (j * MT + mt) * NT + nt;
-                    if (mt == 0 && nt == 0) {
-                        if (j + 1 < NJ) read_x(buf_off, sb, j + 1, (j + 1) & 1);
-                        else if (sb + 1 < kMfmaRing) read_x(buf_off, sb + 1, 0, 0);
+                    if (nt == 0) { // one fragment per unit pair, a whole MFMA group ahead of its use
+                        if (j + 1 < NJ) read_x(buf_off, sb, j + 1, mt, (j + 1) & 1);
+                        else if (sb + 1 < kMfmaRing) read_x(buf_off, sb + 1, 0, mt, 0);
                     }
+                    side(u);
                     uint4 q = make_uint4(wp[which][nt][4 * j], wp[which][nt][4 * j + 1], wp[which][nt][4 * j + 2],
                                          wp[which][nt][4 * j + 3]);
                     acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, q), xf[j & 1][mt],
@@ -183,10 +190,17 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
         }
     };
 
-    load_a(0, 0);
-    store_a(0, 0);
-    load_a(0, 1);
-    store_a(0, 1);
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int op = 0; op < kOpsPerHalf; ++op) load_a_op(0, half, op);
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int op = 0; op < kOpsPerHalf; ++op) store_a_op(0, half, op);
+    const int n_trips = (n_steps + kMfmaRing - 1) / kMfmaRing;
+    const bool ragged = n_steps % kMfmaRing != 0; // uniform, rare
+    if (ragged && n_trips == 1) zero_tail(0, 0);
     __syncthreads();
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) Fmt::decode_fast(ring_raw[0][nt], CS::meta(ring_sb[0][nt]), wp[0][nt]);
@@ -194,8 +208,7 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
     // The loop always runs whole trips of kMfmaRing steps (one activation block): past the end of the reduction the
     // activation blocks are zero-filled and the weight loads are clamped onto the last valid step, so the surplus
     // steps add 0 * w and the loop body is one straight line with no guarded copy. While a trip computes from one
-    // LDS buffer, the next block is staged into the other in two halves; one barrier per trip publishes it.
-    const int n_trips = (n_steps + kMfmaRing - 1) / kMfmaRing;
+    // LDS buffer, the next block is staged into the other; one barrier per trip publishes it.
     static_assert(kMfmaRing == 4, "the staging schedule below is written for four steps per trip");
 #ifdef DMOE_MFMA_CLOCK // debug aid: cycles per reduction step of a few workgroups
     const long long exp_t0 = clock64();
@@ -204,20 +217,21 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
     for (int trip = 0; trip < n_trips; ++trip) {
         const int s0 = trip * kMfmaRing;
         const uint32_t rd_off = (trip & 1) ? (uint32_t)G::kBufBytes : 0u, wr_off = (uint32_t)G::kBufBytes - rd_off;
-        const bool more = trip + 1 < n_trips; // uniform
 #pragma unroll
         for (int j = 0; j < kMfmaRing; ++j) {
             const int s = s0 + j;
             const int s_ahead = s + kMfmaRing < n_steps ? s + kMfmaRing : n_steps - 1;
             load_b(s_ahead, j); // slot j was decoded one step ago
-            if (j == 0 && more) load_a(trip + 1, 0);
-            step_body((j + 1) % kMfmaRing, j & 1, rd_off, j);
-            if (j == 1 && more) {
-                store_a(wr_off, 0);
-                load_a(trip + 1, 1);
-            }
+            // steps 0, 1: fetch the two halves of the next block; steps 2, 3: store them into the other buffer
+            step_body((j + 1) % kMfmaRing, j & 1, rd_off, j, [&](int u) {
+                constexpr int NU = NJ * MT * NT, every = NU / kOpsPerHalf;
+                static_assert(NU % kOpsPerHalf == 0, "staging operations must spread evenly over the units");
+                if (u % every != 0) return;
+                if (j < 2) load_a_op(trip + 1, j, u / every);
+                else store_a_op(wr_off, j - 2, u / every);
+            });
             if (j == 3) {
-                if (more) store_a(wr_off, 1);
+                if (ragged && trip + 2 == n_trips) zero_tail(wr_off, trip + 1);
                 __syncthreads();
             }
         }
