@@ -145,16 +145,22 @@ struct GemmArgs {
     const Tile *tiles = nullptr;  // nullable: dense mode (one segment, expert 0, `dense_rows` rows)
     const uint32_t *n_tiles = nullptr;
     int max_tiles = 0;
+    int tile_m = 0;               // rows per tile the tile list (or the dense split) was built with
     int dense_rows = 0;
     float swiglu_limit = 0.0f;
 };
 // tile_m the kernels were built for
 constexpr int kSkinnyTileM = 8;
 constexpr int kMfmaTileM = 128;
+constexpr int kMfmaWideTileM = 256;
 int launch_qgemm_skinny(const GemmArgs &g, hipStream_t st);
-int launch_qgemm_mfma(const GemmArgs &g, hipStream_t st);
+int launch_qgemm_mfma(const GemmArgs &g, hipStream_t st); // picks the wide kernel when the format allows it
+int launch_qgemm_wide(const GemmArgs &g, hipStream_t st);
 bool qgemm_skinny_supports(const QView &b);
 bool qgemm_mfma_supports(const QView &b);
+bool qgemm_wide_supports(const QView &b);
+// tile size to build tile lists with for the MFMA path of this weight matrix
+inline int qgemm_mfma_tile_m(const QView &b) { return qgemm_wide_supports(b) ? kMfmaWideTileM : kMfmaTileM; }
 
 } // namespace dmoe
 

@@ -3,6 +3,7 @@
 // Also dmoe_gather_qmm, the leaf operator, built from the same pack + grouped-GEMM kernels.
 #include <string.h>
 
+#include <algorithm>
 #include <new>
 
 #include "common.h"
@@ -165,7 +166,8 @@ static FwdLayout forward_layout(const Layer *L, int T) {
     Bump b;
     size_t n = (size_t)T * L->K;
     f.small = use_small_path(n, L->E, L->gate.view) && qgemm_skinny_supports(L->down.view);
-    f.tile_m = f.small ? kSkinnyTileM : kMfmaTileM;
+    // one tile list serves both GEMMs: the smaller of their tile sizes
+    f.tile_m = f.small ? kSkinnyTileM : std::min(qgemm_mfma_tile_m(L->gate.view), qgemm_mfma_tile_m(L->down.view));
     f.max_tiles = pack_max_tiles(n, L->E, f.tile_m);
     f.slot_idx = b.take(n * 4);
     f.order = b.take(n * 4);
@@ -220,6 +222,7 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     gu.tiles = po.tiles;
     gu.n_tiles = po.n_tiles;
     gu.max_tiles = f.max_tiles;
+    gu.tile_m = f.tile_m;
     gu.swiglu_limit = L->swiglu_limit;
     if (L->score_before_down && d_scores) {
         gu.row_scale = d_scores;
@@ -238,6 +241,7 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     dn.tiles = po.tiles;
     dn.n_tiles = po.n_tiles;
     dn.max_tiles = f.max_tiles;
+    dn.tile_m = f.tile_m;
     DMOE_TRY(stage_begin(w, DMOE_STAGE_DOWN, st));
     DMOE_TRY(run_gemm(dn, f.small, st));
     DMOE_TRY(stage_end(w, DMOE_STAGE_DOWN, st));
@@ -249,7 +253,7 @@ static int shared_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     // up to 64 rows the dense expert is streamed by the skinny kernel in 8-row tiles (many workgroups per
     // block of weight rows); above that the big-tile kernel amortises the dequantization
     const bool small = T <= kSharedSkinnyRows && qgemm_skinny_supports(L->sgate.view) && qgemm_skinny_supports(L->sdown.view);
-    const int tile_m = small ? kSkinnyTileM : kMfmaTileM;
+    const int tile_m = small ? kSkinnyTileM : std::min(qgemm_mfma_tile_m(L->sgate.view), qgemm_mfma_tile_m(L->sdown.view));
     GemmArgs gu;
     gu.b0 = L->sgate.view;
     gu.b1 = L->sup.view;
@@ -259,6 +263,7 @@ static int shared_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     gu.ldo = L->Fs;
     gu.dense_rows = T;
     gu.max_tiles = ceil_div(T, tile_m);
+    gu.tile_m = tile_m;
     gu.swiglu_limit = L->shared_swiglu_limit;
     DMOE_TRY(run_gemm(gu, small, st));
     GemmArgs dn;
@@ -268,6 +273,7 @@ static int shared_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     dn.ldo = L->D;
     dn.dense_rows = T;
     dn.max_tiles = ceil_div(T, tile_m);
+    dn.tile_m = tile_m;
     DMOE_TRY(run_gemm(dn, small, st));
     return DMOE_OK;
 }
@@ -466,7 +472,7 @@ int dmoe_gather_qmm(uint16_t *d_out, const uint16_t *d_x, const dmoe_qweight *qw
     hipStream_t st = to_hip(s);
     const bool small = use_small_path((size_t)R, v.n_mats, v);
     DMOE_REQUIRE(small || qgemm_mfma_supports(v), "gather_qmm: unsupported weight shape rows=%d cols=%d", v.rows, v.cols);
-    const int tile_m = small ? kSkinnyTileM : kMfmaTileM;
+    const int tile_m = small ? kSkinnyTileM : qgemm_mfma_tile_m(v);
     const int max_tiles = pack_max_tiles((size_t)R, v.n_mats, tile_m);
     Bump b;
     size_t o_order = b.take((size_t)R * 4), o_arows = b.take((size_t)R * 4);
@@ -497,6 +503,7 @@ int dmoe_gather_qmm(uint16_t *d_out, const uint16_t *d_x, const dmoe_qweight *qw
     g.tiles = po.tiles;
     g.n_tiles = po.n_tiles;
     g.max_tiles = max_tiles;
+    g.tile_m = tile_m;
     return run_gemm(g, small, st);
 }
 

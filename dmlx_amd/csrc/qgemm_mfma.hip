@@ -303,10 +303,10 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void qgemm_mfma_kernel(GemmArgs g)
         if (slot >= n_tiles) return;
     } else {
         t.expert = 0;
-        t.row0 = slot * (uint32_t)kMfmaTileM;
+        t.row0 = slot * (uint32_t)g.tile_m;
         if ((int)t.row0 >= g.dense_rows) return;
         uint32_t left = (uint32_t)g.dense_rows - t.row0;
-        t.nrows = left < (uint32_t)kMfmaTileM ? left : (uint32_t)kMfmaTileM;
+        t.nrows = left < (uint32_t)g.tile_m ? left : (uint32_t)g.tile_m;
     }
     // the tile is the same for the whole workgroup; saying so keeps the four variants apart as scalar branches
     switch (__builtin_amdgcn_readfirstlane((int)((t.nrows + 31u) >> 5))) {
@@ -349,6 +349,8 @@ struct MfmaLaunch {
 };
 
 int launch_qgemm_mfma(const GemmArgs &g, hipStream_t st) {
+    if (qgemm_wide_supports(g.b0)) return launch_qgemm_wide(g, st);
+    DMOE_REQUIRE(g.tile_m > 0 && g.tile_m <= kMfmaTileM && g.tile_m % 32 == 0, "MFMA GEMM: bad tile size %d", g.tile_m);
     DMOE_REQUIRE(qgemm_mfma_supports(g.b0), "MFMA GEMM: unsupported weight shape (rows=%d cols=%d)", g.b0.rows,
                  g.b0.cols);
     DMOE_REQUIRE(g.max_tiles >= 0 && g.max_tiles <= 65535, "MFMA GEMM: %d tiles exceed the grid limit", g.max_tiles);

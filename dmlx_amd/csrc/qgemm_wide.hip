@@ -1,0 +1,337 @@
+// Grouped quantized GEMM, wide MFMA path (prefill, 4-bit formats in the packed resident layout).
+//
+// Same decomposition as the 128-row MFMA kernel (one workgroup = one tile of ONE expert segment against a strip
+// of output columns, each wavefront dequantizes its own 64 weight rows straight into the A operand of
+// v_mfma_f32_32x32x16_bf16), but with tiles of up to 256 rows: every decoded weight fragment then feeds eight
+// matrix instructions instead of four, which halves the decode arithmetic per MFMA -- the vector ALU, not the
+// matrix core, is what bounds the 128-row kernel. 256 rows x 64 columns of f32 accumulators fill all 256
+// accumulation registers of a wavefront, so everything else has to be lean:
+//
+//  * Activations go from global memory into LDS without passing through registers (global_load_lds_dwordx4).
+//    One such instruction moves 1 KiB: 8 rows x 128 bytes (one reduction step of 64 bf16). Inside that KiB the
+//    16-byte pieces of row r are stored at position piece ^ r, so that the MFMA operand reads (32 rows at the
+//    same reduction offset) hit 32 different banks; the swizzle costs nothing because each lane picks its
+//    global source address freely.
+//  * Four LDS buffers of one reduction step each (4 x 32 KiB): while step s computes, the loads of step s+2
+//    are in flight. The compiler does not know about these loads (they are issued from inline assembly), so
+//    their completion is tracked by hand: VMEM operations return in order, hence "at most MT operations
+//    outstanding" three quarters into step s implies that everything issued before this step's own MT loads
+//    -- in particular the loads of step s+1 -- has landed. One s_barrier per step then publishes the buffer.
+//  * Activation fragments are single-buffered (except for tiles of at most 64 rows): the fragment of row tile mt
+//    is reloaded for the next MFMA group right after its last use in this one, 2*MT-1 units before it is needed
+//    again.
+//
+// The reduction loop is software-pipelined exactly like the 128-row kernel: units of [one MFMA | a slice of the
+// decode of the next step's weights] separated by scheduling barriers.
+#include <type_traits>
+
+#include "common.h"
+#include "qformat.h"
+
+namespace dmoe {
+
+constexpr int kWideWaves = 4;
+constexpr int kWideRing = 4;                              // weight steps in registers = LDS activation buffers
+constexpr int kWideBufBytes = kMfmaWideTileM * 128;       // one reduction step (64 bf16) of every row of the tile
+constexpr size_t kWideLdsBytes = (size_t)kWideRing * kWideBufBytes;
+
+// s_waitcnt immediates (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14])
+constexpr int wait_vmcnt(int n) { return 0x0f70 | (n & 15) | ((n >> 4) << 14); }
+constexpr int wait_vmcnt_lgkm0(int n) { return 0x0070 | (n & 15) | ((n >> 4) << 14); }
+constexpr int kWaitLgkm0 = 0xc07f;
+
+template <typename Fmt, bool GATE_UP, int MT>
+__device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint8_t *lds) {
+    using CS = ChunkStream<Fmt, true>;
+    static_assert(Fmt::kVals == 32, "one reduction step must be 64 elements = one 128-byte activation granule");
+    constexpr int KV = 32, KSTEP = 64, NJ = 4, NT = 2;
+    constexpr int NU = NJ * MT * NT;  // units (MFMAs) per step
+    constexpr int NP = NT * (KV / 2); // packed pairs to decode per step
+    const int tid = (int)threadIdx.x, lane = tid & 63, ln = lane & 31, h = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int cols = g.b0.cols, n_out = g.b0.rows;
+    const int n_steps = cols / KSTEP;
+    const int n_trips = (n_steps + kWideRing - 1) / kWideRing;
+    const size_t e = t.expert;
+
+    // ---- this wavefront's weight rows (gate_up: tile 0 = gate, tile 1 = up rows of the same 32 columns) ----
+    const int col_base = ((int)blockIdx.x * kWideWaves + wave) * (GATE_UP ? 32 : 64);
+    const bool wave_on = col_base < n_out;
+    CS cs[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const QView &b = (GATE_UP && nt == 1) ? g.b1 : g.b0;
+        const int base = GATE_UP ? col_base : col_base + 32 * nt;
+        const bool on = wave_on && base < n_out;
+        int n = base + ln;
+        if (n >= n_out) n = n_out - 1;
+        cs[nt].init(b, e, (on ? base : 0) >> 5, ln, h, n); // a switched-off tile aliases valid memory, never stored
+    }
+    uint4 ring_raw[kWideRing][NT];
+    uint32_t ring_sb[kWideRing][NT][2];
+    auto load_b = [&](int step, int slot_) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const QView &b = (GATE_UP && nt == 1) ? g.b1 : g.b0;
+            ring_raw[slot_][nt] = cs[nt].load_chunk(step);
+            cs[nt].load_meta(b, step, ring_sb[slot_][nt]);
+        }
+    };
+#pragma unroll
+    for (int j = 0; j < kWideRing; ++j) load_b(j < n_steps ? j : n_steps - 1, j);
+
+    // ---- activation staging -------------------------------------------------------------------------------
+    // operation i of this wavefront moves rows (wave + 4 i) * 8 .. + 7; lane = (row r8 of the eight, position c),
+    // and fetches piece c ^ r8 of its row. Rows past the segment end alias the tile's first row (never stored).
+    const int r8 = lane >> 3, c = lane & 7;
+    const uint8_t *a_src[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int r = (wave + 4 * i) * 8 + r8;
+        const uint32_t pr = t.row0 + (uint32_t)(r < (int)t.nrows ? r : 0);
+        const size_t src = g.a_rows ? g.a_rows[pr] : pr;
+        a_src[i] = (const uint8_t *)(g.a + src * (size_t)cols) + ((c ^ r8) * 16);
+    }
+    const uint32_t lds_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+    auto stage_op = [&](int blk, int buf, int i) {
+        const uint8_t *gp = a_src[i] + (size_t)blk * 128;
+        const uint32_t la = lds_addr + (uint32_t)(buf * kWideBufBytes + (wave + 4 * i) * 1024); // uniform
+        asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gp), "s"(la) : "memory"); // nothing else in this kernel uses M0
+    };
+    // surplus steps of the last trip (n_steps not a multiple of the ring) must multiply zeros
+    auto zero_block = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+            *(uint4 *)(lds + buf * kWideBufBytes + (wave + 4 * i) * 1024 + lane * 16) = make_uint4(0, 0, 0, 0);
+        __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
+    };
+
+    f32x16_t acc[MT][NT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0.0f;
+
+    uint32_t wp[2][NT][KV / 2]; // decoded weights of the current / next step
+    // activation fragment of each row tile for the current MFMA group; small tiles have registers to spare and too
+    // few units per group to hide an LDS round trip, so they keep a second set and fetch a whole group ahead
+    constexpr int XB = MT <= 2 ? 2 : 1;
+    // blocks in flight ahead of the one being computed. A short step (small tile) does not cover a memory round
+    // trip, so small tiles run three blocks ahead; that reuses the buffer read during the previous step, which is
+    // only safe because those tiles also wait for their own LDS reads before each barrier (see below).
+    constexpr int AHEAD = MT <= 2 ? 3 : 2;
+    bf16x8_t xf[XB][MT];
+    // fragment (mt, j) of a step: row mt * 32 + ln, piece h * 4 + j, stored at piece ^ (row & 7)
+    const uint8_t *x_rd[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) x_rd[j] = lds + (ln >> 3) * 1024 + (ln & 7) * 128 + (((h * 4 + j) ^ (ln & 7)) * 16);
+    auto read_x = [&](int buf, int j, int mt) {
+        uint4 q = *(const uint4 *)(x_rd[j] + buf * kWideBufBytes + mt * 4096);
+        xf[j % XB][mt] = __builtin_bit_cast(bf16x8_t, q);
+    };
+
+    // ---- prologue: the first AHEAD blocks, first decode ----------------------------------------------------------
+#pragma unroll
+    for (int b = 0; b < AHEAD; ++b) {
+        if (b < n_steps) {
+#pragma unroll
+            for (int i = 0; i < MT; ++i) stage_op(b, b, i);
+        } else {
+            zero_block(b);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) Fmt::decode_fast(ring_raw[0][nt], CS::meta(ring_sb[0][nt]), wp[0][nt]);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) read_x(0, 0, mt);
+
+#ifdef DMOE_MFMA_CLOCK // debug aid: cycles per reduction step of a few workgroups
+    const long long exp_t0 = clock64();
+#endif
+    // The loop always runs whole trips of kWideRing steps: surplus steps multiply zeroed activations with weights
+    // clamped onto the last valid step. Step j of a trip computes from buffer j, requests block s + AHEAD into buffer
+    // (j + AHEAD) % 4 during its first three MFMA groups, and at the start of the fourth waits for block s + 1 and
+    // synchronises, so that the first fragments of the next step can be fetched during that last group.
+#pragma unroll 1
+    for (int trip = 0; trip < n_trips; ++trip) {
+        const int s0 = trip * kWideRing;
+#pragma unroll
+        for (int j = 0; j < kWideRing; ++j) {
+            const int s = s0 + j;
+            const int s_ahead = s + kWideRing < n_steps ? s + kWideRing : n_steps - 1;
+            load_b(s_ahead, j); // slot j was decoded one step ago
+            const int slot_next = (j + 1) % kWideRing, which = j & 1, buf_next = (j + 1) % kWideRing;
+            const bool stage = s + AHEAD < n_steps; // uniform
+            Meta meta_next[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) meta_next[nt] = CS::meta(ring_sb[slot_next][nt]);
+            uint32_t dstate[2] = {0, 0};
+#pragma unroll
+            for (int jj = 0; jj < NJ; ++jj) {
+                if (jj == NJ - 1) {
+                    // block s + 1 must have landed; the AHEAD - 1 younger requests of MT operations each may still
+                    // fly (fewer near the end of the reduction, when nothing is requested any more)
+                    if (AHEAD == 2) {
+                        if (stage) __builtin_amdgcn_s_waitcnt(wait_vmcnt(MT));
+                        else __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));
+                    } else {
+                        // also drain this wavefront's LDS reads: the next step's requests overwrite the buffer
+                        // that the reads issued during the previous MFMA group came from
+                        if (stage) __builtin_amdgcn_s_waitcnt(wait_vmcnt_lgkm0(2 * MT));
+                        else if (s + AHEAD - 1 < n_steps) __builtin_amdgcn_s_waitcnt(wait_vmcnt_lgkm0(MT));
+                        else __builtin_amdgcn_s_waitcnt(wait_vmcnt_lgkm0(0));
+                    }
+                    asm volatile("" ::: "memory");
+                    __builtin_amdgcn_s_barrier();
+                    asm volatile("" ::: "memory");
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        const int u = (jj * MT + mt) * NT + nt;
+                        uint4 q = make_uint4(wp[which][nt][4 * jj], wp[which][nt][4 * jj + 1], wp[which][nt][4 * jj + 2],
+                                             wp[which][nt][4 * jj + 3]);
+                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, q),
+                                                                              xf[jj % XB][mt], acc[mt][nt], 0, 0, 0);
+                        // fetch the fragment of the next group: after the last use of this one (one register set),
+                        // or at the first (two sets)
+                        if (nt == (XB == 1 ? NT - 1 : 0)) {
+                            if (jj + 1 < NJ) read_x(j, jj + 1, mt);
+                            else read_x(buf_next, 0, mt);
+                        }
+                        if (u % 6 == 0 && u / 6 < MT) { // the staging requests all fall into the first three groups
+                            if (stage) stage_op(s + AHEAD, (j + AHEAD) % kWideRing, u / 6);
+                        }
+#pragma unroll
+                        for (int p = u * NP / NU; p < (u + 1) * NP / NU; ++p) {
+                            Fmt::decode_pair(ring_raw[slot_next][p / (KV / 2)], meta_next[p / (KV / 2)], p % (KV / 2),
+                                             wp[which ^ 1][p / (KV / 2)], dstate);
+                            // pin the slice here (the optimiser would sink a trip's last decode into the next trip)
+                            asm volatile("" : "+v"(wp[which ^ 1][p / (KV / 2)][p % (KV / 2)]));
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+            if (!stage && s + AHEAD < n_trips * kWideRing) zero_block((j + AHEAD) % kWideRing); // a surplus step: zeros
+        }
+    }
+#ifdef DMOE_MFMA_CLOCK
+    if (blockIdx.x == 3 && (blockIdx.y % 97) == 5 && tid == 0)
+        printf("MT %d gate_up %d slot %d steps %d clk/step %lld\n", MT, (int)GATE_UP, (int)blockIdx.y, n_steps,
+               (clock64() - exp_t0) / n_steps);
+#endif
+
+    // ---- epilogue: lane = token row (ln), registers r -> output column 8*(r/4) + 4*h + r%4 -------------
+    if (!wave_on) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int rl = mt * 32 + ln;
+        if (rl >= (int)t.nrows) continue;
+        const uint32_t p = t.row0 + (uint32_t)rl;
+        const size_t dst = g.out_rows ? g.out_rows[p] : p;
+        float rscale = 1.0f;
+        if (g.row_scale) rscale = g.row_scale[g.row_scale_idx ? g.row_scale_idx[p] : p];
+        uint16_t *orow = g.out + dst * (size_t)g.ldo;
+        if (GATE_UP) {
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) {
+                const int n0 = col_base + 8 * rg + 4 * h;
+                if (n0 >= n_out) continue;
+                float v[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    v[i] = limited_swiglu(acc[mt][0][4 * rg + i], acc[mt][1][4 * rg + i], g.swiglu_limit) * rscale;
+                *(uint2 *)(orow + n0) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+            }
+        } else {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                for (int rg = 0; rg < 4; ++rg) {
+                    const int n0 = col_base + 32 * nt + 8 * rg + 4 * h;
+                    if (n0 >= n_out) continue;
+                    float v[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v[i] = acc[mt][nt][4 * rg + i] * rscale;
+                    *(uint2 *)(orow + n0) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+                }
+            }
+        }
+    }
+}
+
+template <typename Fmt, bool GATE_UP>
+__global__ __launch_bounds__(kWideWaves * 64) void qgemm_wide_kernel(GemmArgs g) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t wide_lds[]; // [kWideRing][256 rows][128 bytes], swizzled
+    Tile t;
+    const uint32_t slot = blockIdx.y;
+    if (g.tiles) {
+        const uint32_t n_tiles = *g.n_tiles;
+        t = g.tiles[slot];
+        if (slot >= n_tiles) return;
+    } else {
+        t.expert = 0;
+        t.row0 = slot * (uint32_t)g.tile_m;
+        if ((int)t.row0 >= g.dense_rows) return;
+        uint32_t left = (uint32_t)g.dense_rows - t.row0;
+        t.nrows = left < (uint32_t)g.tile_m ? left : (uint32_t)g.tile_m;
+    }
+    // the tile is the same for the whole workgroup; saying so keeps the variants apart as scalar branches
+    const int mt = __builtin_amdgcn_readfirstlane((int)((t.nrows + 31u) >> 5));
+    if (mt <= 1) wide_tile<Fmt, GATE_UP, 1>(g, t, wide_lds);
+    else if (mt == 2) wide_tile<Fmt, GATE_UP, 2>(g, t, wide_lds);
+    else if (mt == 3) wide_tile<Fmt, GATE_UP, 3>(g, t, wide_lds);
+    else if (mt == 4) wide_tile<Fmt, GATE_UP, 4>(g, t, wide_lds);
+    else if (mt <= 6) wide_tile<Fmt, GATE_UP, 6>(g, t, wide_lds);
+    else wide_tile<Fmt, GATE_UP, 8>(g, t, wide_lds);
+}
+
+bool qgemm_wide_supports(const QView &b) {
+    const bool four_bit = (b.mode == DMOE_QUANT_AFFINE && b.bits == 4) || b.mode == DMOE_QUANT_MXFP4;
+    return four_bit && b.packed && b.cols % 64 == 0 && b.rows % 4 == 0;
+}
+
+template <typename Fmt, bool GATE_UP>
+static int launch_wide(const GemmArgs &g, hipStream_t st) {
+    auto kern = qgemm_wide_kernel<Fmt, GATE_UP>;
+    static thread_local bool raised = false; // per instantiation: allow more than 64 KiB of dynamic LDS once
+    if (!raised) {
+        DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsBytes));
+        raised = true;
+    }
+    const int cols_per_block = kWideWaves * (GATE_UP ? 32 : 64);
+    dim3 grid((unsigned)ceil_div(g.b0.rows, cols_per_block), (unsigned)g.max_tiles), block(kWideWaves * 64);
+    hipLaunchKernelGGL(kern, grid, block, kWideLdsBytes, st, g);
+    DMOE_LAUNCH_CHECK();
+    return DMOE_OK;
+}
+
+int launch_qgemm_wide(const GemmArgs &g, hipStream_t st) {
+    DMOE_REQUIRE(qgemm_wide_supports(g.b0), "wide MFMA GEMM: unsupported weight format or shape (rows=%d cols=%d)",
+                 g.b0.rows, g.b0.cols);
+    DMOE_REQUIRE(g.tile_m > 0 && g.tile_m <= kMfmaWideTileM && g.tile_m % 32 == 0, "wide MFMA GEMM: bad tile size %d",
+                 g.tile_m);
+    DMOE_REQUIRE(g.max_tiles >= 0 && g.max_tiles <= 65535, "wide MFMA GEMM: %d tiles exceed the grid limit", g.max_tiles);
+    DMOE_REQUIRE(g.a && g.out && g.ldo > 0 && g.ldo % 4 == 0 && ((uintptr_t)g.out % 8) == 0 &&
+                     ((uintptr_t)g.a % 16) == 0,
+                 "wide MFMA GEMM: bad output / activation pointer or pitch");
+    if (g.gate_up)
+        DMOE_REQUIRE(g.b1.rows == g.b0.rows && g.b1.cols == g.b0.cols && g.b1.mode == g.b0.mode &&
+                         g.b1.bits == g.b0.bits && g.b1.group == g.b0.group && g.b1.packed == g.b0.packed,
+                     "wide MFMA GEMM: gate and up projections differ in shape or format");
+    if (g.max_tiles == 0) return DMOE_OK;
+    if (g.b0.mode == DMOE_QUANT_MXFP4)
+        return g.gate_up ? launch_wide<FmtMxfp4, true>(g, st) : launch_wide<FmtMxfp4, false>(g, st);
+    return g.gate_up ? launch_wide<FmtAffine4, true>(g, st) : launch_wide<FmtAffine4, false>(g, st);
+}
+
+} // namespace dmoe

@@ -60,7 +60,9 @@ def test_dequantize_bit_exact(dmoe, orc, fmt):
 @pytest.mark.parametrize("fmt", FORMATS)
 @pytest.mark.parametrize("R,n_mats,rows,cols", [(24, 8, 256, 1024),     # small-M path (<= 4 rows per expert on average)
                                                 (700, 4, 256, 512),     # MFMA path, ragged segments
-                                                (130, 1, 128, 2048)])   # single expert, MFMA, partial tile
+                                                (130, 1, 128, 2048),    # single expert, MFMA, partial tile
+                                                (700, 4, 256, 384),     # reduction not a multiple of the pipeline depth
+                                                (1200, 2, 192, 640)])   # 256-row tiles, idle wavefronts in the last strip
 def test_gather_qmm_matches_oracle(dmoe, orc, ws, fmt, R, n_mats, rows, cols):
     qw = _stack(fmt, n_mats, rows, cols, 2)
     g = torch.Generator(device="cuda").manual_seed(3)
