@@ -79,8 +79,10 @@ __device__ uint32_t emit_segments(uint32_t count, int e, int E, size_t n, int ti
         if (e == 0 && o.n_live) *o.n_live = lt;
     }
     if (tile_m > 0 && o.tiles) {
-        uint32_t nt = (count + (uint32_t)tile_m - 1) / (uint32_t)tile_m, tt;
-        uint32_t tb = block_excl_scan(nt, &tt, sm);
+        // tiles stay grouped by expert: tiles of one expert that run together share its weights through L2
+        // (emitting the full tiles of all experts first, to shorten the tail of the GEMM launches, measured slower)
+        uint32_t nt = (count + (uint32_t)tile_m - 1) / (uint32_t)tile_m, tf;
+        uint32_t tb = block_excl_scan(nt, &tf, sm);
         for (uint32_t j = 0; j < nt; ++j) {
             Tile t;
             t.expert = (uint32_t)e;
@@ -90,7 +92,7 @@ __device__ uint32_t emit_segments(uint32_t count, int e, int E, size_t n, int ti
             t.pad = 0;
             o.tiles[tb + j] = t;
         }
-        if (e == 0 && o.n_tiles) *o.n_tiles = tt;
+        if (e == 0 && o.n_tiles) *o.n_tiles = tf;
     }
     return off;
 }

@@ -85,7 +85,7 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArg
     auto load_stage = [&](int step, SkinnyStage<NM> &s) {
 #pragma unroll
         for (int mi = 0; mi < NM; ++mi) {
-            s.raw[mi] = cs[mi].load_chunk(step);
+            s.raw[mi] = cs[mi].load_chunk_stream(step);
             cs[mi].load_meta(mi == 0 ? g.b0 : g.b1, step, s.sb[mi]);
         }
     };
@@ -98,20 +98,21 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArg
             if (j < n_steps) load_stage(j, ring[j]);
     }
 
-    // ---- activations of the tile -> LDS (rows past the tile are zero) -----------------------------------
+    // ---- activations of the tile -> LDS ---------------------------------------------------------------
+    // Only the rows the tile has are staged (most decode tiles hold one to three): row m of the A operand only
+    // reaches accumulator row m, and accumulator rows past the tile are never stored, so whatever the lanes of the
+    // missing rows feed the matrix core does not matter (they feed zeros, see x_on below).
     const int pitch = cols * 2 + 16; // bytes per LDS row; +16 keeps the 8 rows on different banks
+    const int nrows = (int)t.nrows;
     uint8_t *xs_lds = skinny_lds;
     float *gs_lds = (float *)(skinny_lds + kSkinnyTileM * pitch); // [n_steps][8]: per-step sums of x (factored)
     {
         const int pieces = cols / 8; // 16-byte pieces per row
-        for (int idx = tid; idx < kSkinnyTileM * pieces; idx += kSkinnyWaves * 64) {
+        for (int idx = tid; idx < nrows * pieces; idx += kSkinnyWaves * 64) {
             const int r = idx / pieces, pc = idx - r * pieces;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (r < (int)t.nrows) {
-                const uint32_t p = t.row0 + (uint32_t)r;
-                const size_t src = g.a_rows ? g.a_rows[p] : p;
-                v = *(const uint4 *)(g.a + src * (size_t)cols + pc * 8);
-            }
+            const uint32_t p = t.row0 + (uint32_t)r;
+            const size_t src = g.a_rows ? g.a_rows[p] : p;
+            uint4 v = *(const uint4 *)(g.a + src * (size_t)cols + pc * 8);
             if (FACTORED) { // (x0..x7) -> (x0,x4,x1,x5,x2,x6,x3,x7), the order the code pairs come out in
                 uint4 o;
                 o.x = (v.x & 0xffffu) | (v.z << 16);
@@ -125,8 +126,8 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArg
     }
     __syncthreads();
     if (FACTORED) {
-        for (int idx = tid; idx < n_steps * kSkinnyTileM; idx += kSkinnyWaves * 64) {
-            const int step = idx / kSkinnyTileM, r = idx % kSkinnyTileM;
+        for (int idx = tid; idx < n_steps * nrows; idx += kSkinnyWaves * 64) {
+            const int step = idx / nrows, r = idx - step * nrows;
             const uint32_t *px = (const uint32_t *)(xs_lds + r * pitch + step * KSTEP * 2);
             float sum = 0.0f;
 #pragma unroll 8
@@ -137,8 +138,8 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArg
     }
     if (!wave_on) return;
 
-    // A-operand source of this lane: tile row ln (zero beyond the tile), reduction half h
-    const bool x_on = ln < kSkinnyTileM;
+    // A-operand source of this lane: tile row ln (zeros beyond the tile), reduction half h
+    const bool x_on = ln < nrows;
     const uint8_t *xlane = xs_lds + (x_on ? ln : 0) * pitch + h * KV * 2;
 
     f32x16_t acc[NM];
