@@ -23,6 +23,12 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+COPY_PROBE_BYTES = 256 << 20  # --copy-probe: bytes read (and written) by each calibration copy
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
+# (scaled by the same counters' reading for the --copy-probe copies; profiles/hbm_traffic_gemm_kernels.txt).
+# A counter cannot be read from inside the timed run, so these are the recorded values for the default workloads.
+MEASURED_TRAFFIC = {(1, "gate_up"): 1052284000, (1, "down"): 529434000,
+                    (3, "gate_up"): 5182157000, (3, "down"): 2804555000}
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 
@@ -69,6 +75,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", type=int, default=1, choices=[0, 1, 2, 3, 4])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run three plain 256 MiB device copies first: the known-size kernel that scales the "
+                         "FETCH_SIZE / WRITE_SIZE counters when this command runs under rocprofv3 --pmc")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures the one-GPU path only: this build has no multi-GPU path (run with --gpus 1)",
@@ -89,6 +98,14 @@ def main():
 
     def step():
         return layer.layer_forward(wl.x, wl.scores, wl.bias, wl.resident_mask, wl.renorm, wl.route_scale, ws)
+
+    if args.copy_probe:
+        src = torch.ones(COPY_PROBE_BYTES // 4, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         out = step()
@@ -136,6 +153,7 @@ def main():
         achieved = k_flops / (k_ms * 1e-3) / 1e12
         roof = {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None}
+    roof["traffic"] = MEASURED_TRAFFIC.get((args.config, kern))
     roof.update({"kernel": f"grouped {kern} GEMM ({'small-M' if decode else 'MFMA'} path)", "kernel_ms": k_ms,
                  "algorithmic_bytes": k_bytes, "algorithmic_flops": k_flops, "live_experts": U})
 
