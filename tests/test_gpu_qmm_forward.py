@@ -151,6 +151,18 @@ def test_score_position_variants(dmoe, orc, ws, before):
     _check_layer(dmoe, orc, ws, wl)
 
 
+@pytest.mark.parametrize("config,T", [(1, 300), (2, 700)])
+def test_prefill_sized_batch_with_4bit_shared_expert(dmoe, orc, ws, config, T):
+    """A prefill-sized batch on the decode configurations: routed experts AND the dense shared expert (4-bit) on the
+    256-row matrix-core kernel, the latter in its dense mode (no tile list); 300 and 700 rows leave a partial tile."""
+    wl = workloads.make(config, scale=0.125)
+    g = torch.Generator(device="cuda").manual_seed(11)
+    wl.T = T
+    wl.x = torch.randn((T, wl.D), generator=g, device="cuda").to(torch.bfloat16)
+    wl.scores = torch.sigmoid(torch.randn((T, wl.E_total), generator=g, device="cuda"))
+    _check_layer(dmoe, orc, ws, wl)
+
+
 def test_c1_decode_full_size(dmoe, orc, ws):
     """BASELINE config 1 at full size (64 x 1 tokens, D=4096, 256 experts top-6 + shared, F=2048, affine-4)."""
     wl = workloads.make(1)
