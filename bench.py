@@ -68,6 +68,29 @@ def cpu_baseline(wl, max_tokens, min_seconds=10.0, max_runs=5):
                       f"workload, median {med:.3f} s (CPU restatement of the dmlx/MLX op sequence, OpenMP)"}
 
 
+def measured_peaks(torch):
+    """What simple library kernels reach on this GPU, reported next to the published peaks: a device-to-device copy
+    (read + written bytes per second) and a square bf16 GEMM through torch (hipBLASLt)."""
+    out = {}
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    a = torch.randn((8192, 8192), device="cuda", dtype=torch.bfloat16)
+    b = torch.randn((8192, 8192), device="cuda", dtype=torch.bfloat16)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for name, fn, work in (("d2d_copy_GBs", lambda: dst.copy_(src), 2.0 * n / 1e9),
+                           ("bf16_gemm_TFLOPs", lambda: torch.matmul(a, b), 2.0 * 8192 ** 3 / 1e12)):
+        for _ in range(3):
+            fn()
+        e0.record()
+        for _ in range(10):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        out[name] = work / (e0.elapsed_time(e1) / 10 * 1e-3)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -154,6 +177,7 @@ def main():
         roof = {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None}
     roof["traffic"] = MEASURED_TRAFFIC.get((args.config, kern))
+    roof["measured_peaks"] = measured_peaks(torch)
     roof.update({"kernel": f"grouped {kern} GEMM ({'small-M' if decode else 'MFMA'} path)", "kernel_ms": k_ms,
                  "algorithmic_bytes": k_bytes, "algorithmic_flops": k_flops, "live_experts": U})
 

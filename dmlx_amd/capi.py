@@ -41,6 +41,15 @@ class LayerDescC(C.Structure):
                 ("weight_source", C.c_int)]
 
 
+class GateDescC(C.Structure):
+    _fields_ = [("weight", C.c_void_p), ("bias", C.c_void_p), ("resident_mask", C.c_void_p),
+                ("n_experts", C.c_int), ("dim", C.c_int), ("top_k", C.c_int),
+                ("scoring_func", C.c_int), ("route_scale", C.c_float), ("is_hash", C.c_int),
+                ("weight_source", C.c_int)]
+
+
+SCORE_SOFTMAX, SCORE_SIGMOID, SCORE_SQRTSOFTPLUS = 0, 1, 2
+
 # every symbol include/dmoe.h declares
 EXPORTS = [
     "dmoe_quant_mode_from_string", "dmoe_version", "dmoe_last_error", "dmoe_init",
@@ -53,6 +62,7 @@ EXPORTS = [
     "dmoe_pack", "dmoe_dequantize", "dmoe_gather_qmm",
     "dmoe_layer_create", "dmoe_layer_destroy", "dmoe_moe_forward",
     "dmoe_switch_glu_forward_no_scores", "dmoe_moe_layer_forward", "dmoe_debug_last_activations",
+    "dmoe_gate_create", "dmoe_gate_destroy", "dmoe_gate_forward",
 ]
 
 _lib = None
@@ -243,6 +253,42 @@ def gather_qmm(x, qw, rhs_indices, ws, lhs_indices=None, sorted_indices=False):
     check(lib().dmoe_gather_qmm(_ptr(out), _ptr(x), C.byref(c), _ptr(lhs_indices), _ptr(rhs_indices), R,
                                 int(sorted_indices), ws.h, _stream()))
     return out
+
+
+class Gate:
+    """Resident router (dmoe_gate): DSV4Gate.forward from the hidden states on."""
+
+    def __init__(self, weight, top_k, scoring_func, route_scale=1.0, bias=None, resident_mask=None):
+        assert weight.dtype == torch.bfloat16 and weight.dim() == 2
+        d = GateDescC()
+        d.weight, d.bias, d.resident_mask = _ptr(weight), _ptr(bias), _ptr(resident_mask)
+        d.n_experts, d.dim, d.top_k = weight.shape[0], weight.shape[1], top_k
+        d.scoring_func, d.route_scale, d.is_hash = scoring_func, route_scale, 0
+        d.weight_source = WEIGHTS_COPY_FROM_DEVICE if weight.is_cuda else WEIGHTS_COPY_FROM_HOST
+        for t in (bias, resident_mask):
+            assert t is None or t.is_cuda == weight.is_cuda, "gate tensors must live on the same side"
+        self.n_experts, self.top_k = weight.shape[0], top_k
+        self.h = _Handle()
+        check(lib().dmoe_gate_create(C.byref(self.h), C.byref(d), _stream()))
+
+    def forward(self, x, ws, want_scores=False):
+        T = x.shape[0]
+        idx = torch.empty((T, self.top_k), dtype=torch.int32, device=x.device)
+        w = torch.empty((T, self.top_k), dtype=torch.float32, device=x.device)
+        scores = torch.empty((T, self.n_experts), dtype=torch.float32, device=x.device) if want_scores else None
+        check(lib().dmoe_gate_forward(_ptr(idx), _ptr(w), _ptr(scores), self.h, _ptr(x), T, ws.h, _stream()))
+        return (idx, w, scores) if want_scores else (idx, w)
+
+    def close(self):
+        if self.h.ctx:
+            check(lib().dmoe_gate_destroy(self.h))
+            self.h = _Handle()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 class Layer:

@@ -195,14 +195,43 @@ struct SmeltConfig {      // deepseek_v4_loader.zig:250-294
 
 enum class ScoringFunc { softmax, sigmoid, sqrtsoftplus }; // deepseek_v4.zig:82-86
 
-// DSV4Gate from the scores on (deepseek_v4.zig:589-678). The router GEMM and the scoring function run
-// upstream of this path; `forward` takes their result.
+// DSV4Gate (deepseek_v4.zig:521-681). `forward(ctx, scores)` takes the result of the scoring function (the
+// gate epilogue, :589-678); once `load` has uploaded the router weight, `forwardHidden` serves the whole
+// DSV4Gate.forward(hidden_states, null, stream): matmul, scoring function, selection.
 struct DSV4Gate {
     size_t topk = 0, n_routed_experts = 0;
     float route_scale = 1.0f;
     ScoringFunc scoring_func = ScoringFunc::sqrtsoftplus;
+    bool is_hash = false;
     Array bias;        // optional [n_routed_experts] f32 selection bias
     Array smelt_mask;  // optional [n_routed_experts] u8 residency mask
+
+    DSV4Gate() = default;
+    DSV4Gate(const DSV4Gate &) = delete;
+    DSV4Gate &operator=(const DSV4Gate &) = delete;
+    ~DSV4Gate() { deinit(); }
+    void deinit() {
+        if (handle_.ctx) dmoe_gate_destroy(handle_);
+        handle_.ctx = nullptr;
+    }
+
+    // uploads `weight` (HOST bf16 [n_routed_experts, dim]) together with the bias / mask given as host vectors
+    void load(const Context &ctx, const uint16_t *weight, int dim, const float *host_bias = nullptr,
+              const uint8_t *host_mask = nullptr) {
+        deinit();
+        dmoe_gate_desc d{};
+        d.weight = weight;
+        d.bias = host_bias;
+        d.resident_mask = host_mask;
+        d.n_experts = (int)n_routed_experts;
+        d.dim = dim;
+        d.top_k = (int)topk;
+        d.scoring_func = (int)scoring_func;
+        d.route_scale = route_scale;
+        d.is_hash = is_hash ? 1 : 0;
+        d.weight_source = DMOE_WEIGHTS_COPY_FROM_HOST;
+        check(dmoe_gate_create(&handle_, &d, ctx.stream()));
+    }
 
     // returns (weights [T, topk] f32, indices [T, topk] u32) like the reference's tuple
     std::pair<Array, Array> forward(const Context &ctx, const Array &scores) const {
@@ -214,6 +243,22 @@ struct DSV4Gate {
                               scoring_func != ScoringFunc::softmax ? 1 : 0, route_scale, ctx.stream()));
         return {w, idx};
     }
+
+    // hidden_states bf16 [T, dim] (or [B, S, dim]) -> (weights, indices); needs load()
+    std::pair<Array, Array> forwardHidden(const Context &ctx, const Array &hidden_states) const {
+        if (!handle_.ctx) throw Error(DMOE_ERR_INVALID, "DSV4Gate.forwardHidden: no router weight loaded");
+        const auto &sh = hidden_states.shape();
+        int T = 1;
+        for (size_t i = 0; i + 1 < sh.size(); ++i) T *= sh[i];
+        const int K = (int)topk;
+        Array idx(ctx, DType::uint32, {T, K}), w(ctx, DType::float32, {T, K});
+        check(dmoe_gate_forward((uint32_t *)idx.data(), (float *)w.data(), nullptr, handle_,
+                                (const uint16_t *)hidden_states.data(), T, ctx.workspace(), ctx.stream()));
+        return {w, idx};
+    }
+
+  private:
+    dmoe_gate handle_{};
 };
 
 // Quantized stack description on the host side (QuantizedWeight + QuantConfig of mlx-zig)

@@ -141,6 +141,43 @@ pub fn gateRoute(ctx: Context, scores: DeviceArray(f32), bias: ?DeviceArray(f32)
     return .{ .indices = idx, .weights = w, .k = topk, .num_tokens = num_tokens };
 }
 
+/// DSV4Gate (deepseek_v4.zig:521-681) with the router weight resident on the device: `forward` is the whole
+/// DSV4Gate.forward(hidden_states, null, stream) -- matmul, scoring function, selection.
+pub const ResidentGate = struct {
+    handle: c.dmoe_gate,
+    topk: usize,
+
+    /// weight: host bf16 bits [n_experts * dim]; bias / mask: host slices or null
+    pub fn init(ctx: Context, weight: []const u16, bias: ?[]const f32, smelt_mask: ?[]const u8, n_experts: usize, dim: usize, topk: usize, scoring_func: c_int, route_scale: f32) Error!ResidentGate {
+        var d = std.mem.zeroes(c.dmoe_gate_desc);
+        d.weight = weight.ptr;
+        d.bias = if (bias) |b| b.ptr else null;
+        d.resident_mask = if (smelt_mask) |m| m.ptr else null;
+        d.n_experts = @intCast(n_experts);
+        d.dim = @intCast(dim);
+        d.top_k = @intCast(topk);
+        d.scoring_func = scoring_func;
+        d.route_scale = route_scale;
+        d.weight_source = c.DMOE_WEIGHTS_COPY_FROM_HOST;
+        var h: c.dmoe_gate = undefined;
+        try check(c.dmoe_gate_create(&h, &d, ctx.stream));
+        return .{ .handle = h, .topk = topk };
+    }
+
+    pub fn deinit(self: *ResidentGate) void {
+        _ = c.dmoe_gate_destroy(self.handle);
+    }
+
+    pub fn forward(self: *ResidentGate, ctx: Context, hidden_states: DeviceArray(u16), num_tokens: usize) Error!RouteResult {
+        const idx = try DeviceArray(u32).alloc(num_tokens * self.topk);
+        errdefer idx.deinit();
+        const w = try DeviceArray(f32).alloc(num_tokens * self.topk);
+        errdefer w.deinit();
+        try check(c.dmoe_gate_forward(@ptrCast(@alignCast(idx.ptr)), @ptrCast(@alignCast(w.ptr)), null, self.handle, @ptrCast(@alignCast(hidden_states.ptr)), @intCast(num_tokens), ctx.ws, ctx.stream));
+        return .{ .indices = idx, .weights = w, .k = self.topk, .num_tokens = num_tokens };
+    }
+};
+
 /// ExpertProvider over HBM-resident experts: `forward(layer_idx, flat_x, indices, scores)` as in
 /// src/models/expert_provider.zig:21; replaces ExpertStreamProvider.streamForward (expert_stream.zig:245-261).
 pub const ResidentExpertProvider = struct {

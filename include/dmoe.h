@@ -51,6 +51,7 @@ typedef enum {
 typedef struct dmoe_stream_ { void *ctx; } dmoe_stream;           /* ctx = hipStream_t */
 typedef struct dmoe_workspace_ { void *ctx; } dmoe_workspace;     /* grow-only device scratch */
 typedef struct dmoe_layer_ { void *ctx; } dmoe_layer;             /* resident expert weights of one MoE layer */
+typedef struct dmoe_gate_ { void *ctx; } dmoe_gate;               /* resident router of one MoE layer */
 
 /* "affine" -> DMOE_QUANT_AFFINE, "mxfp4" -> DMOE_QUANT_MXFP4, "fp8" -> DMOE_QUANT_FP8_ROW; -1 if unknown */
 int dmoe_quant_mode_from_string(const char *name);
@@ -238,6 +239,42 @@ int dmoe_moe_layer_forward(uint16_t *d_out, uint32_t *d_out_indices, float *d_ou
                            const uint16_t *d_x, const float *d_scores, const float *d_bias,
                            const uint8_t *d_resident_mask, int T, int E_total, int renorm, float route_scale,
                            dmoe_workspace ws, dmoe_stream s);
+
+/* ---- router (gate) from the hidden states on ------------------------------------------------ */
+
+/* DSV4Config.ScoringFunc (deepseek_v4.zig:82-86) */
+typedef enum {
+    DMOE_SCORE_SOFTMAX = 0,
+    DMOE_SCORE_SIGMOID = 1,
+    DMOE_SCORE_SQRTSOFTPLUS = 2 /* sqrt(log(1 + exp(x))), the reference's default (:48) */
+} dmoe_scoring_func;
+
+/* DSV4Gate fields (deepseek_v4.zig:521-535). Pointers are host or device memory as `weight_source` says
+ * (DMOE_WEIGHTS_COPY_FROM_HOST / _FROM_DEVICE; the weight is re-ordered, so it is always copied). */
+typedef struct {
+    const void *weight;           /* bf16 [n_experts, dim] (:523)                                  */
+    const float *bias;            /* nullable f32 [n_experts]: selection bias (:524, :593-599)     */
+    const uint8_t *resident_mask; /* nullable u8 [n_experts]: Smelt mask, 1 = resident (:531-535)  */
+    int n_experts, dim, top_k;
+    int scoring_func;             /* dmoe_scoring_func */
+    float route_scale;            /* :528 */
+    int is_hash;                  /* hash routing through tid2eid (:525, :619-636): must be 0, not supported */
+    int weight_source;            /* dmoe_weight_source */
+} dmoe_gate_desc;
+
+int dmoe_gate_create(dmoe_gate *out, const dmoe_gate_desc *desc, dmoe_stream s);
+int dmoe_gate_destroy(dmoe_gate gate);
+
+/* DSV4Gate.forward(hidden_states, input_ids = null) (deepseek_v4.zig:546-681): logits = (x @ W^T) in bf16
+ * widened to f32, scoring function, then dmoe_gate_route with the gate's bias, mask, top_k and route scale
+ * (renormalised unless the scoring function is softmax). Returns (weights, indices) like the reference.
+ *   d_out_indices u32 [T,K]; d_out_weights f32 [T,K]; d_out_scores nullable f32 [T,n_experts]: the
+ *   unbiased scores, for inspection; d_x bf16 [T,dim], 16-byte aligned.
+ * The order of the f32 additions in the matmul and the evaluation of exp / log are fixed by this library
+ * (segments of 128 reduction elements summed left to right; polynomial exp / log), so the selected experts
+ * do not depend on tile shapes or library versions; MLX's own choices are not observable from the reference. */
+int dmoe_gate_forward(uint32_t *d_out_indices, float *d_out_weights, float *d_out_scores, dmoe_gate gate,
+                      const uint16_t *d_x, int T, dmoe_workspace ws, dmoe_stream s);
 
 /* Inspection of the last dmoe_moe_forward / dmoe_switch_glu_forward_no_scores on this workspace:
  * the SwiGLU activations in flat (t*K+k) row order, bf16 [T*K, F]. For parity tests. */

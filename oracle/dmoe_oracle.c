@@ -136,6 +136,117 @@ void orc_gate_scores(const float *logits, int T, int E, int func, float *out) {
     }
 }
 
+/* ---- router matmul and scoring with a fixed arithmetic (u7) ---------------------------------- */
+
+/* deepseek_v4.zig:556-565. Products of two bf16 numbers are exact in f32; what is not
+ * fixed by the reference is the order of the f32 additions. The order used here: the
+ * reduction dimension is cut into segments of 128 elements, each segment is summed
+ * left to right starting from 0, and the segment sums are added left to right. The
+ * result is rounded to bf16 (the matmul's output dtype) and widened to f32 (:563). */
+#define ORC_GATE_SEG 128
+void orc_gate_logits(const uint16_t *x, const uint16_t *wg, int T, int D, int E, float *out) {
+#pragma omp parallel for schedule(static)
+    for (int t = 0; t < T; t++) {
+        const uint16_t *xr = x + (size_t)t * D;
+        for (int e = 0; e < E; e++) {
+            const uint16_t *wr = wg + (size_t)e * D;
+            float total = 0.0f;
+            for (int k0 = 0; k0 < D; k0 += ORC_GATE_SEG) {
+                int k1 = k0 + ORC_GATE_SEG < D ? k0 + ORC_GATE_SEG : D;
+                float part = 0.0f;
+                for (int k = k0; k < k1; k++) part = fmaf(orc_bf16_to_f32(xr[k]), orc_bf16_to_f32(wr[k]), part);
+                total = total + part;
+            }
+            out[(size_t)t * E + e] = orc_bf16_to_f32(orc_f32_to_bf16(total));
+        }
+    }
+}
+
+static float bits_to_f32(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+static uint32_t f32_to_bits(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+
+/* exp(x) in f32 from IEEE operations only (Cody-Waite reduction by ln 2 in two parts, the
+ * degree-5 polynomial of the Cephes expf, scaling by two exact powers of two). Inputs below
+ * -87 give 0 (no denormal results), above 88.72 give +inf; NaN passes through. */
+float orc_det_expf(float x) {
+    if (x != x) return x;
+    if (x > 88.72283935546875f) return bits_to_f32(0x7f800000u);
+    if (x < -87.0f) return 0.0f;
+    float n = rintf(x * 1.44269504088896341f);
+    float r = fmaf(n, -0.693359375f, x);
+    r = fmaf(n, 2.12194440e-4f, r);
+    float p = 1.9875691500E-4f;
+    p = fmaf(p, r, 1.3981999507E-3f);
+    p = fmaf(p, r, 8.3334519073E-3f);
+    p = fmaf(p, r, 4.1665795894E-2f);
+    p = fmaf(p, r, 1.6666665459E-1f);
+    p = fmaf(p, r, 5.0000001201E-1f);
+    float y = fmaf(p, r * r, r) + 1.0f;
+    int ni = (int)n, k1 = ni / 2, k2 = ni - k1;
+    y = y * bits_to_f32((uint32_t)(k1 + 127) << 23);
+    return y * bits_to_f32((uint32_t)(k2 + 127) << 23);
+}
+
+/* log(x) in f32 for normal x > 0 (the Cephes logf: mantissa in [sqrt(1/2), sqrt(2)), degree-8
+ * polynomial, exponent added back in two parts); +inf -> +inf, 0 -> -inf, negative or NaN -> NaN. */
+float orc_det_logf(float x) {
+    if (x != x || x < 0.0f) return bits_to_f32(0x7fc00000u);
+    if (x == 0.0f) return bits_to_f32(0xff800000u);
+    uint32_t u = f32_to_bits(x);
+    if (u == 0x7f800000u) return x;
+    int e = (int)((u >> 23) & 0xffu) - 126;
+    float m = bits_to_f32((u & 0x007fffffu) | 0x3f000000u); /* [0.5, 1) */
+    if (m < 0.707106781186547524f) {
+        e -= 1;
+        m = (m + m) - 1.0f;
+    } else {
+        m = m - 1.0f;
+    }
+    float z = m * m;
+    float y = 7.0376836292E-2f;
+    y = fmaf(y, m, -1.1514610310E-1f);
+    y = fmaf(y, m, 1.1676998740E-1f);
+    y = fmaf(y, m, -1.2420140846E-1f);
+    y = fmaf(y, m, 1.4249322787E-1f);
+    y = fmaf(y, m, -1.6668057665E-1f);
+    y = fmaf(y, m, 2.0000714765E-1f);
+    y = fmaf(y, m, -2.4999993993E-1f);
+    y = fmaf(y, m, 3.3333331174E-1f);
+    y = (y * m) * z;
+    float fe = (float)e;
+    y = fmaf(fe, -2.12194440e-4f, y);
+    y = fmaf(-0.5f, z, y);
+    float r = m + y;
+    return fmaf(fe, 0.693359375f, r);
+}
+
+/* deepseek_v4.zig:567-585, op by op, with orc_det_expf / orc_det_logf in place of MLX's exp / log.
+ * softmax (:569): exp(x - max) / sum, the sum taken as 64 strided partial sums (element e goes to
+ * partial e mod 64, in increasing e) that are then folded by halves (p[i] += p[i + 32], 16, .. 1). */
+void orc_gate_scores_det(const float *logits, int T, int E, int func, float *out) {
+    for (int t = 0; t < T; t++) {
+        const float *x = logits + (size_t)t * E;
+        float *o = out + (size_t)t * E;
+        if (func == ORC_SCORE_SOFTMAX) {
+            float mx = x[0];
+            for (int e = 1; e < E; e++) mx = x[e] > mx ? x[e] : mx;
+            float part[64];
+            for (int i = 0; i < 64; i++) part[i] = 0.0f;
+            for (int e = 0; e < E; e++) {
+                o[e] = orc_det_expf(x[e] - mx);
+                part[e & 63] = part[e & 63] + o[e];
+            }
+            for (int off = 32; off >= 1; off >>= 1)
+                for (int i = 0; i < off; i++) part[i] = part[i] + part[i + off];
+            for (int e = 0; e < E; e++) o[e] = o[e] / part[0];
+        } else if (func == ORC_SCORE_SIGMOID) {
+            for (int e = 0; e < E; e++) o[e] = 1.0f / (1.0f + orc_det_expf(-x[e]));
+        } else {
+            for (int e = 0; e < E; e++) o[e] = sqrtf(orc_det_logf(1.0f + orc_det_expf(x[e])));
+        }
+    }
+}
+
 /* deepseek_v4.zig:589-678. choice = scores + bias[E] (:593-599), then
  * + (resident ? 0 : -1e9) (:601-615); indices = last K of the ascending argsort of
  * choice (:654 -> :383-396); weights gathered from the UNBIASED scores (:589,:658);

@@ -20,6 +20,12 @@
  *   (u4) gather_qmm / quantized_matmul accumulate in f32; output dtype = x dtype.
  *   (u5) bf16 (activations) x f32 (scores) promotes to f32.
  *   (u6) FP8 is OCP E4M3FN (no infinities, 0x7f/0xff are NaN).
+ *   (u7) the router matmul (bf16 x bf16 -> bf16) accumulates in f32 and rounds once;
+ *        the accumulation ORDER and the rounding of exp / log inside the scoring
+ *        function are MLX's and unknown. orc_gate_logits / orc_gate_scores_det fix
+ *        one order and one explicit polynomial exp / log (stated at their
+ *        definitions) so that a GPU implementation of the same arithmetic can be
+ *        compared bit for bit; against libm they agree to a few ulp (tests).
  * Functions whose results depend on one of (u1), (u3)..(u6) are marked
  * "parity unpinned vs MLX" at their definition.
  *
@@ -58,6 +64,13 @@ void orc_topk_route(const float *scores, int T, int E, int K, int normalize,
                     uint32_t *idx_out, float *w_out);
 /* deepseek_v4.zig:567-585 */
 void orc_gate_scores(const float *logits, int T, int E, int func, float *scores_out);
+/* deepseek_v4.zig:556-565: logits = (x @ Wg^T) in bf16, then astype(f32).
+ * x bf16 [T,D], wg bf16 [E,D] -> logits f32 [T,E] (every value representable in bf16). */
+void orc_gate_logits(const uint16_t *x, const uint16_t *wg, int T, int D, int E, float *logits_out);
+/* deepseek_v4.zig:567-585 with exp / log evaluated by explicit f32 polynomials (u7) */
+void orc_gate_scores_det(const float *logits, int T, int E, int func, float *scores_out);
+float orc_det_expf(float x);
+float orc_det_logf(float x);
 /* deepseek_v4.zig:589-678 (selection on biased/masked scores, weights from the
  * unbiased ones, renorm when not softmax, * route_scale) */
 void orc_gate_route(const float *scores, const float *bias, const uint8_t *resident,

@@ -122,6 +122,37 @@ def gate_scores(logits, func):
     return out
 
 
+def gate_logits(x_bf16, wg_bf16):
+    """x, wg: uint16 arrays of bf16 bits, [T,D] and [E,D] -> f32 [T,E] (bf16-valued)"""
+    x = _c(x_bf16, np.uint16)
+    w = _c(wg_bf16, np.uint16)
+    T, D = x.shape
+    E = w.shape[0]
+    out = np.empty((T, E), np.float32)
+    lib().orc_gate_logits(_p(x), _p(w), T, D, E, _p(out))
+    return out
+
+
+def gate_scores_det(logits, func):
+    x = _c(logits, np.float32)
+    T, E = x.shape
+    out = np.empty_like(x)
+    lib().orc_gate_scores_det(_p(x), T, E, func, _p(out))
+    return out
+
+
+def det_expf(x):
+    f = lib().orc_det_expf
+    f.restype = C.c_float
+    return np.array([f(C.c_float(float(v))) for v in np.asarray(x, np.float32).ravel()], np.float32)
+
+
+def det_logf(x):
+    f = lib().orc_det_logf
+    f.restype = C.c_float
+    return np.array([f(C.c_float(float(v))) for v in np.asarray(x, np.float32).ravel()], np.float32)
+
+
 def gate_route(scores, bias, resident, K, renorm, route_scale):
     s = _c(scores, np.float32)
     T, E = s.shape

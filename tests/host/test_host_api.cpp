@@ -228,6 +228,40 @@ static void test_layer_closed_form(const Context &ctx) {
     EXPECT(threw);
 }
 
+// DSV4Gate.forward from the hidden states on. x = e_0 scaled: logit of expert e = 2 * W[e][0], exactly
+// representable, so the selection and the sigmoid weights are known in closed form.
+static void test_gate_from_hidden(Context &ctx) {
+    const int T = 3, D = 64, E = 8, K = 2;
+    std::vector<uint16_t> x((size_t)T * D, bf16(0.0f)), wg((size_t)E * D, bf16(0.0f));
+    for (int t = 0; t < T; ++t) x[(size_t)t * D] = bf16(2.0f);
+    const float w0[E] = {0.5f, -1.0f, 1.5f, 0.25f, -0.5f, 1.0f, 0.0f, -2.0f}; // logits 1, -2, 3, .5, -1, 2, 0, -4
+    for (int e = 0; e < E; ++e) wg[(size_t)e * D] = bf16(w0[e]);
+    DSV4Gate gate;
+    gate.topk = K;
+    gate.n_routed_experts = E;
+    gate.route_scale = 1.0f;
+    gate.scoring_func = ScoringFunc::sigmoid;
+    gate.load(ctx, wg.data(), D);
+    auto r = gate.forwardHidden(ctx, Array::fromData(ctx, x.data(), {T, D}, DType::bfloat16));
+    auto idx = r.second.dataSlice<uint32_t>();
+    auto w = r.first.dataSlice<float>();
+    const double s3 = 1.0 / (1.0 + std::exp(-3.0)), s2 = 1.0 / (1.0 + std::exp(-2.0));
+    for (int t = 0; t < T; ++t) {
+        EXPECT(idx[t * K] == 5u && idx[t * K + 1] == 2u); // ascending score order: expert 5 (logit 2), then 2 (logit 3)
+        NEAR(w[t * K], s2 / (s2 + s3), 1e-6);
+        NEAR(w[t * K + 1], s3 / (s2 + s3), 1e-6);
+    }
+    bool threw = false;
+    try {
+        DSV4Gate empty;
+        empty.topk = K;
+        empty.forwardHidden(ctx, Array::fromData(ctx, x.data(), {T, D}, DType::bfloat16));
+    } catch (const Error &) {
+        threw = true;
+    }
+    EXPECT(threw);
+}
+
 int main() {
     try {
         Context ctx(0);
@@ -236,6 +270,7 @@ int main() {
         test_property_18(ctx);
         test_remap_smelt_batch(ctx);
         test_layer_closed_form(ctx);
+        test_gate_from_hidden(ctx);
         ctx.synchronize();
     } catch (const Error &e) {
         std::printf("dmoe::Error %d: %s\n", e.code, e.what());

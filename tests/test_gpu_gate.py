@@ -1,0 +1,74 @@
+"""GPU parity of DSV4Gate.forward from the hidden states on (router matmul -> scoring -> selection), through
+the C ABI, against the oracle. The library and the oracle fix the same accumulation order and the same
+polynomial exp / log, so scores, routing weights and indices must match bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+from tests.helpers import bf16_bits, to_np_u32
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(seed, T, D, E, with_bias, with_mask, spread):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    x = (torch.randn((T, D), generator=g, device="cuda") * spread).to(torch.bfloat16)
+    wg = (torch.randn((E, D), generator=g, device="cuda") * (1.0 / D ** 0.5)).to(torch.bfloat16)
+    bias = torch.randn(E, generator=g, device="cuda") * 0.1 if with_bias else None
+    mask = None
+    if with_mask:
+        mask = (torch.rand(E, generator=g, device="cuda") < 0.4).to(torch.uint8)
+        mask[:8] = 1  # at least K resident experts
+    return x, wg, bias, mask
+
+
+@pytest.mark.parametrize("func", [0, 1, 2])
+@pytest.mark.parametrize("T,D,E,K,with_bias,with_mask", [
+    (64, 4096, 256, 6, True, False),     # decode shape of configuration 1: one reduction segment per wavefront
+    (5, 200, 72, 3, True, True),         # short last segment, experts not a multiple of 64, Smelt mask
+    (1, 128, 8, 2, False, False),
+    (700, 1024, 64, 4, True, False),     # several segments per wavefront, sums through scratch
+    (4200, 256, 128, 6, True, False),    # many tokens: a wavefront walks all segments itself
+])
+def test_gate_forward_bit_exact(dmoe, orc, ws, func, T, D, E, K, with_bias, with_mask):
+    x, wg, bias, mask = _case(7 + func, T, D, E, with_bias, with_mask, spread=2.0)
+    gate = dmoe.Gate(wg, K, func, route_scale=1.5, bias=bias, resident_mask=mask)
+    idx, w, scores = gate.forward(x, ws, want_scores=True)
+    logits = orc.gate_logits(bf16_bits(x), bf16_bits(wg))
+    want_scores = orc.gate_scores_det(logits, func)
+    np.testing.assert_array_equal(scores.cpu().numpy().view(np.uint32), want_scores.view(np.uint32))
+    want_idx, want_w = orc.gate_route(want_scores, None if bias is None else bias.cpu().numpy(),
+                                      None if mask is None else mask.cpu().numpy(), K, func != 0, 1.5)
+    np.testing.assert_array_equal(to_np_u32(idx), want_idx)
+    np.testing.assert_array_equal(w.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
+    # without the inspection output the routing is the same
+    idx2, w2 = gate.forward(x, ws)
+    assert torch.equal(idx2, idx) and torch.equal(w2, w)
+    gate.close()
+
+
+def test_gate_extreme_logits(dmoe, orc, ws):
+    """Saturating inputs: sigmoid -> 0 / 1, softplus overflow of the reference's literal form (exp -> inf)."""
+    T, D, E = 4, 64, 64
+    x = torch.full((T, D), 8.0, device="cuda").to(torch.bfloat16)
+    wg = torch.zeros((E, D), device="cuda")
+    wg[0] = 0.25      # logit 128: exp overflows, log(inf) = inf
+    wg[1] = -0.25     # logit -128
+    wg[2] = 0.0
+    wg = wg.to(torch.bfloat16)
+    for func in (1, 2):
+        gate = dmoe.Gate(wg, 2, func)
+        _, _, scores = gate.forward(x, ws, want_scores=True)
+        want = orc.gate_scores_det(orc.gate_logits(bf16_bits(x), bf16_bits(wg)), func)
+        np.testing.assert_array_equal(scores.cpu().numpy().view(np.uint32), want.view(np.uint32))
+        gate.close()
+
+
+def test_gate_rejects_bad_arguments(dmoe):
+    wg = torch.zeros((8, 64), device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(dmoe.DmoeError):
+        dmoe.Gate(wg, 9, 1)            # top_k > experts
+    with pytest.raises(dmoe.DmoeError):
+        dmoe.Gate(wg[:, :60].contiguous(), 2, 1)   # dim not a multiple of 8
+    with pytest.raises(dmoe.DmoeError):
+        dmoe.Gate(wg, 2, 7)            # unknown scoring function

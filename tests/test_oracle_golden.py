@@ -392,3 +392,47 @@ def test_batch_concat_and_mask_properties(orc):
             for c in range(T):
                 allowed = owner[r] == owner[c] and c <= r
                 assert m[r, c] == (0.0 if allowed else -np.inf)
+
+
+# ---- router matmul and scoring with fixed arithmetic (assumption u7) ----------------------------------------
+
+def test_det_exp_log_within_one_ulp_of_the_exact_value(orc):
+    """Pins the polynomial exp / log against the mathematical functions (float64 numpy), not against themselves."""
+    x = np.linspace(-87.0, 88.0, 4001).astype(np.float32)
+    got = orc.det_expf(x).astype(np.float64)
+    ref = np.exp(x.astype(np.float64))
+    assert (np.abs(got - ref) / np.spacing(ref.astype(np.float32)).astype(np.float64)).max() < 1.0
+    y = np.exp(np.linspace(np.log(1e-30), np.log(3e38), 4001)).astype(np.float32)
+    got = orc.det_logf(y).astype(np.float64)
+    ref = np.log(y.astype(np.float64))
+    assert (np.abs(got - ref) / np.spacing(np.abs(ref).astype(np.float32)).astype(np.float64)).max() < 1.0
+    # special values
+    assert orc.det_expf([0.0])[0] == 1.0 and orc.det_expf([-100.0])[0] == 0.0 and np.isinf(orc.det_expf([100.0])[0])
+    assert orc.det_logf([1.0])[0] == 0.0 and np.isinf(orc.det_logf([np.inf])[0]) and np.isnan(orc.det_logf([-1.0])[0])
+    assert np.isnan(orc.det_expf([np.nan])[0])
+
+
+def test_gate_logits_match_a_float64_matmul(orc):
+    rng = np.random.default_rng(5)
+    T, D, E = 7, 392, 24      # a short last segment (392 = 3 * 128 + 8)
+    x = orc.f32_to_bf16(rng.standard_normal((T, D)).astype(np.float32))
+    w = orc.f32_to_bf16((rng.standard_normal((E, D)) / 16).astype(np.float32))
+    got = orc.gate_logits(x, w)
+    exact = orc.bf16_to_f32(x).astype(np.float64) @ orc.bf16_to_f32(w).astype(np.float64).T
+    # every logit is a bf16 number within one bf16 rounding step of the exact dot product
+    assert np.array_equal(orc.bf16_to_f32(orc.f32_to_bf16(got)), got)
+    assert (np.abs(got - exact) <= np.abs(exact) * 2.0 ** -8 + 1e-6).all()
+    # a single product: exact
+    one = orc.gate_logits(orc.f32_to_bf16(np.array([[1.5] + [0.0] * 7], np.float32)),
+                          orc.f32_to_bf16(np.array([[-2.25] + [0.0] * 7], np.float32)))
+    assert one[0, 0] == -3.375
+
+
+def test_gate_scores_det_agree_with_libm(orc):
+    rng = np.random.default_rng(6)
+    logits = orc.bf16_to_f32(orc.f32_to_bf16((rng.standard_normal((9, 70)) * 4).astype(np.float32)))
+    for func in (0, 1, 2):
+        a, b = orc.gate_scores_det(logits, func), orc.gate_scores(logits, func)
+        np.testing.assert_allclose(a, b, rtol=2e-6, atol=1e-12)
+    sm = orc.gate_scores_det(logits, 0)
+    np.testing.assert_allclose(sm.sum(1), 1.0, rtol=1e-6)
