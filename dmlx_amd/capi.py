@@ -48,6 +48,13 @@ class GateDescC(C.Structure):
                 ("weight_source", C.c_int)]
 
 
+class SafetensorsOptsC(C.Structure):
+    _fields_ = [("top_k", C.c_int), ("mode", C.c_char_p), ("group_size", C.c_int), ("bits", C.c_int),
+                ("swiglu_limit", C.c_float), ("score_before_down", C.c_int), ("load_shared", C.c_int),
+                ("shared_mode", C.c_char_p), ("shared_group_size", C.c_int), ("shared_bits", C.c_int),
+                ("shared_swiglu_limit", C.c_float), ("resident_mask", C.c_void_p), ("n_experts_total", C.c_int)]
+
+
 SCORE_SOFTMAX, SCORE_SIGMOID, SCORE_SQRTSOFTPLUS = 0, 1, 2
 
 # every symbol include/dmoe.h declares
@@ -63,6 +70,7 @@ EXPORTS = [
     "dmoe_layer_create", "dmoe_layer_destroy", "dmoe_moe_forward",
     "dmoe_switch_glu_forward_no_scores", "dmoe_moe_layer_forward", "dmoe_debug_last_activations",
     "dmoe_gate_create", "dmoe_gate_destroy", "dmoe_gate_forward",
+    "dmoe_layer_create_from_safetensors", "dmoe_layer_dims",
 ]
 
 _lib = None
@@ -317,6 +325,29 @@ class Layer:
         self.hidden, self.ffn, self.top_k = hidden, ffn, top_k
         self.h = _Handle()
         check(lib().dmoe_layer_create(C.byref(self.h), C.byref(d), _stream()))
+
+    @classmethod
+    def from_safetensors(cls, paths, layer_idx, top_k, mode, group_size, bits, swiglu_limit=0.0,
+                         score_before_down=False, load_shared=True, shared_swiglu_limit=0.0, resident_mask=None):
+        """dmoe_layer_create_from_safetensors; `resident_mask` is a host sequence of 0/1 per expert in the file."""
+        o = SafetensorsOptsC()
+        o.top_k, o.mode, o.group_size, o.bits = top_k, mode.encode(), group_size, bits
+        o.swiglu_limit, o.score_before_down, o.load_shared = swiglu_limit, int(score_before_down), int(load_shared)
+        o.shared_mode, o.shared_group_size, o.shared_bits, o.shared_swiglu_limit = None, 0, 0, shared_swiglu_limit
+        keep = None
+        if resident_mask is not None:
+            keep = (C.c_uint8 * len(resident_mask))(*[int(v) for v in resident_mask])
+            o.resident_mask, o.n_experts_total = C.cast(keep, C.c_void_p), len(resident_mask)
+        arr = (C.c_char_p * len(paths))(*[p.encode() for p in paths])
+        self = cls.__new__(cls)
+        self._remap_host, self._keep = None, None
+        self.h = _Handle()
+        check(lib().dmoe_layer_create_from_safetensors(C.byref(self.h), arr, len(paths), layer_idx, C.byref(o),
+                                                       _stream()))
+        d, f, n, k = C.c_int(), C.c_int(), C.c_int(), C.c_int()
+        check(lib().dmoe_layer_dims(C.byref(d), C.byref(f), C.byref(n), C.byref(k), self.h))
+        self.hidden, self.ffn, self.n_slots, self.top_k = d.value, f.value, n.value, k.value
+        return self
 
     def forward(self, x, indices, scores, ws):
         T = x.shape[0]

@@ -355,6 +355,16 @@ int dmoe_layer_create(dmoe_layer *out, const dmoe_layer_desc *d, dmoe_stream s) 
     return DMOE_OK;
 }
 
+int dmoe_layer_dims(int *out_hidden, int *out_ffn, int *out_n_slots, int *out_top_k, dmoe_layer layer) {
+    const Layer *L = (const Layer *)layer.ctx;
+    DMOE_REQUIRE(L != nullptr, "layer_dims: null layer");
+    if (out_hidden) *out_hidden = L->D;
+    if (out_ffn) *out_ffn = L->F;
+    if (out_n_slots) *out_n_slots = L->E;
+    if (out_top_k) *out_top_k = L->K;
+    return DMOE_OK;
+}
+
 int dmoe_layer_destroy(dmoe_layer layer) {
     if (layer.ctx) free_layer((Layer *)layer.ctx);
     return DMOE_OK;

@@ -321,6 +321,35 @@ class DSV4SwitchGLU {
         d.weight_source = opt.source;
         check(dmoe_layer_create(&layer_, &d, ctx.stream()));
     }
+    // Resident upload from MLX-format safetensors shards (replaces TensorIndex + LayerExpertMeta + the stream
+    // provider set up in model_registry.zig:255-329). `smelt_mask` empty = every expert of the file.
+    struct FileOptions {
+        std::string mode = "mxfp4"; // the reference passes ("mxfp4", 32, 4) (:318-321)
+        int group_size = 32, bits = 4;
+        float swiglu_limit = 0.0f, shared_swiglu_limit = 0.0f;
+        bool score_before_down = false, load_shared = true;
+        std::vector<uint8_t> smelt_mask;
+    };
+    DSV4SwitchGLU(const Context &ctx, const std::vector<std::string> &paths, int layer_idx, int top_k,
+                  const FileOptions &opt) {
+        std::vector<const char *> p;
+        for (const auto &s : paths) p.push_back(s.c_str());
+        dmoe_safetensors_opts o{};
+        o.top_k = top_k;
+        o.mode = opt.mode.c_str();
+        o.group_size = opt.group_size;
+        o.bits = opt.bits;
+        o.swiglu_limit = opt.swiglu_limit;
+        o.score_before_down = opt.score_before_down ? 1 : 0;
+        o.load_shared = opt.load_shared ? 1 : 0;
+        o.shared_swiglu_limit = opt.shared_swiglu_limit;
+        if (!opt.smelt_mask.empty()) {
+            o.resident_mask = opt.smelt_mask.data();
+            o.n_experts_total = (int)opt.smelt_mask.size();
+        }
+        check(dmoe_layer_create_from_safetensors(&layer_, p.data(), (int)p.size(), layer_idx, &o, ctx.stream()));
+        check(dmoe_layer_dims(&hidden_, &ffn_, nullptr, &top_k_, layer_));
+    }
     ~DSV4SwitchGLU() { dmoe_layer_destroy(layer_); } // deinit()
     DSV4SwitchGLU(const DSV4SwitchGLU &) = delete;
     DSV4SwitchGLU &operator=(const DSV4SwitchGLU &) = delete;

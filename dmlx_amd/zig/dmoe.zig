@@ -178,6 +178,25 @@ pub const ResidentGate = struct {
     }
 };
 
+/// One-time resident upload of a layer's experts from MLX-format safetensors shards (what
+/// model_registry.zig:255-329 prepares for on-demand reads). `paths` are NUL-terminated.
+pub fn layerFromSafetensors(ctx: Context, paths: []const [*:0]const u8, layer_idx: usize, top_k: usize, mode: [*:0]const u8, group_size: i32, bits: i32, swiglu_limit: f32, smelt_mask: ?[]const u8) Error!c.dmoe_layer {
+    var o = std.mem.zeroes(c.dmoe_safetensors_opts);
+    o.top_k = @intCast(top_k);
+    o.mode = mode;
+    o.group_size = group_size;
+    o.bits = bits;
+    o.swiglu_limit = swiglu_limit;
+    o.load_shared = 1;
+    if (smelt_mask) |m| {
+        o.resident_mask = m.ptr;
+        o.n_experts_total = @intCast(m.len);
+    }
+    var layer: c.dmoe_layer = undefined;
+    try check(c.dmoe_layer_create_from_safetensors(&layer, @ptrCast(paths.ptr), @intCast(paths.len), @intCast(layer_idx), &o, ctx.stream));
+    return layer;
+}
+
 /// ExpertProvider over HBM-resident experts: `forward(layer_idx, flat_x, indices, scores)` as in
 /// src/models/expert_provider.zig:21; replaces ExpertStreamProvider.streamForward (expert_stream.zig:245-261).
 pub const ResidentExpertProvider = struct {

@@ -219,6 +219,35 @@ typedef struct {
 int dmoe_layer_create(dmoe_layer *out, const dmoe_layer_desc *desc, dmoe_stream s);
 int dmoe_layer_destroy(dmoe_layer layer);
 
+/* One-time resident upload of a layer's experts from MLX-format safetensors files: what
+ * model_registry.zig:255-329 prepares for on-demand reads (TensorIndex + LayerExpertMeta +
+ * ExpertStreamProvider.initWithStrategy(..., quantized, group_size, bits, mode, swiglu_limit, ...)) done once,
+ * into HBM. Tensor names as there (:264-269):
+ *   model.layers.{layer_idx}.ffn.switch_mlp.{gate,up,down}_proj.{weight,scales,biases}   U32 / BF16|U8 / BF16
+ *   model.layers.{layer_idx}.ffn.shared_experts.{gate,up,down}_proj.{...}                 (when load_shared)
+ * Shapes [E, rows, cols*bits/32] and [E, rows, cols/group]; D, F and E are read from them. */
+typedef struct {
+    int top_k;
+    const char *mode;            /* "affine" | "mxfp4" (the reference passes "mxfp4", 32, 4; :318-321) */
+    int group_size, bits;
+    float swiglu_limit;
+    int score_before_down;
+    int load_shared;             /* also load the shared expert when the files hold one */
+    const char *shared_mode;     /* NULL / 0 below: same as the routed experts */
+    int shared_group_size, shared_bits;
+    float shared_swiglu_limit;
+    const uint8_t *resident_mask;/* nullable HOST u8 [n_experts_total]: Smelt, only experts with 1 are uploaded, in
+                                    increasing id order; the router-id -> slot remap is built like
+                                    deepseek_v4_loader.zig:2151-2168 (unloaded -> 0) */
+    int n_experts_total;         /* length of resident_mask = experts in the file */
+} dmoe_safetensors_opts;
+
+int dmoe_layer_create_from_safetensors(dmoe_layer *out, const char *const *paths, int n_paths, int layer_idx,
+                                       const dmoe_safetensors_opts *opts, dmoe_stream s);
+
+/* shape of a resident layer: D, F, resident expert slots, K (any out pointer may be NULL) */
+int dmoe_layer_dims(int *out_hidden, int *out_ffn, int *out_n_slots, int *out_top_k, dmoe_layer layer);
+
 /* ExpertProvider.VTable.forward(ptr, layer_idx, flat_x, indices, scores) (expert_provider.zig:21) ==
  * ExpertStreamProvider.streamForward (expert_stream.zig:245-261) == the provider arm of DSV4MoE.forward
  * (deepseek_v4.zig:1030-1047), plus the shared expert and the final add (:1021, :1050-1052) when the layer
