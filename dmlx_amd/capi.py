@@ -45,7 +45,7 @@ class GateDescC(C.Structure):
     _fields_ = [("weight", C.c_void_p), ("bias", C.c_void_p), ("resident_mask", C.c_void_p),
                 ("n_experts", C.c_int), ("dim", C.c_int), ("top_k", C.c_int),
                 ("scoring_func", C.c_int), ("route_scale", C.c_float), ("is_hash", C.c_int),
-                ("weight_source", C.c_int)]
+                ("tid2eid", C.c_void_p), ("vocab_size", C.c_int), ("weight_source", C.c_int)]
 
 
 class SafetensorsOptsC(C.Structure):
@@ -266,25 +266,29 @@ def gather_qmm(x, qw, rhs_indices, ws, lhs_indices=None, sorted_indices=False):
 class Gate:
     """Resident router (dmoe_gate): DSV4Gate.forward from the hidden states on."""
 
-    def __init__(self, weight, top_k, scoring_func, route_scale=1.0, bias=None, resident_mask=None):
+    def __init__(self, weight, top_k, scoring_func, route_scale=1.0, bias=None, resident_mask=None, tid2eid=None):
         assert weight.dtype == torch.bfloat16 and weight.dim() == 2
         d = GateDescC()
         d.weight, d.bias, d.resident_mask = _ptr(weight), _ptr(bias), _ptr(resident_mask)
         d.n_experts, d.dim, d.top_k = weight.shape[0], weight.shape[1], top_k
-        d.scoring_func, d.route_scale, d.is_hash = scoring_func, route_scale, 0
+        d.scoring_func, d.route_scale, d.is_hash = scoring_func, route_scale, int(tid2eid is not None)
+        if tid2eid is not None:
+            assert tid2eid.dtype == torch.int32 and tid2eid.shape[1] == top_k
+            d.tid2eid, d.vocab_size = _ptr(tid2eid), tid2eid.shape[0]
         d.weight_source = WEIGHTS_COPY_FROM_DEVICE if weight.is_cuda else WEIGHTS_COPY_FROM_HOST
-        for t in (bias, resident_mask):
+        for t in (bias, resident_mask, tid2eid):
             assert t is None or t.is_cuda == weight.is_cuda, "gate tensors must live on the same side"
         self.n_experts, self.top_k = weight.shape[0], top_k
         self.h = _Handle()
         check(lib().dmoe_gate_create(C.byref(self.h), C.byref(d), _stream()))
 
-    def forward(self, x, ws, want_scores=False):
+    def forward(self, x, ws, want_scores=False, input_ids=None):
         T = x.shape[0]
         idx = torch.empty((T, self.top_k), dtype=torch.int32, device=x.device)
         w = torch.empty((T, self.top_k), dtype=torch.float32, device=x.device)
         scores = torch.empty((T, self.n_experts), dtype=torch.float32, device=x.device) if want_scores else None
-        check(lib().dmoe_gate_forward(_ptr(idx), _ptr(w), _ptr(scores), self.h, _ptr(x), T, ws.h, _stream()))
+        check(lib().dmoe_gate_forward(_ptr(idx), _ptr(w), _ptr(scores), self.h, _ptr(x), _ptr(input_ids), T, ws.h,
+                                      _stream()))
         return (idx, w, scores) if want_scores else (idx, w)
 
     def close(self):

@@ -35,6 +35,8 @@ struct Gate {
     uint16_t *wgp = nullptr; // [D/8][E][8] bf16
     float *bias = nullptr;   // [E] or null
     uint8_t *mask = nullptr; // [E] or null (1 = resident)
+    int32_t *tid2eid = nullptr; // [vocab, K] or null: hash routing table
+    int vocab = 0;
 };
 
 __global__ void gate_repack_kernel(uint4 *__restrict__ dst, const uint16_t *__restrict__ src, int E, int D) {
@@ -244,6 +246,34 @@ __global__ __launch_bounds__(kGateWaves * 64) void gate_scores_kernel(float *__r
     }
 }
 
+// Hash routing (deepseek_v4.zig:619-636, then :655-678): the experts of a token come from a table indexed by its
+// token id; the weights are the unbiased scores of those experts, divided by (their sum + 1e-20) unless the scoring
+// function is softmax, times the route scale. One thread per token; the sum runs over k in increasing order.
+__global__ void gate_hash_route_kernel(uint32_t *__restrict__ idx, float *__restrict__ w,
+                                       const float *__restrict__ scores, const int32_t *__restrict__ tid2eid,
+                                       const uint32_t *__restrict__ ids, int T, int E, int K, int vocab, int renorm,
+                                       float route_scale) {
+    const int t = (int)(blockIdx.x * blockDim.x + threadIdx.x);
+    if (t >= T) return;
+    uint32_t id = ids[t];
+    if (id >= (uint32_t)vocab) id = (uint32_t)vocab - 1; // ids are validated by the caller's contract; stay in bounds
+    float sum = 0.0f;
+    for (int j = 0; j < K; ++j) {
+        int e = tid2eid[(size_t)id * K + j];
+        e = e < 0 ? 0 : (e >= E ? E - 1 : e);
+        const float s = scores[(size_t)t * E + e];
+        idx[(size_t)t * K + j] = (uint32_t)e;
+        w[(size_t)t * K + j] = s;
+        sum = sum + s;
+    }
+    const float denom = sum + 1e-20f;
+    for (int j = 0; j < K; ++j) {
+        float v = w[(size_t)t * K + j];
+        if (renorm) v = v / denom;
+        w[(size_t)t * K + j] = v * route_scale;
+    }
+}
+
 } // namespace dmoe
 
 using namespace dmoe;
@@ -261,7 +291,8 @@ int dmoe_gate_create(dmoe_gate *out, const dmoe_gate_desc *d, dmoe_stream s) {
                  "gate_create: unknown scoring function %d", d->scoring_func);
     DMOE_REQUIRE(d->weight_source == DMOE_WEIGHTS_COPY_FROM_HOST || d->weight_source == DMOE_WEIGHTS_COPY_FROM_DEVICE,
                  "gate_create: weight_source must be a copying one (the weight is re-ordered)");
-    DMOE_REQUIRE(!d->is_hash, "gate_create: hash routing (tid2eid) is not supported");
+    DMOE_REQUIRE(!d->is_hash || (d->tid2eid != nullptr && d->vocab_size >= 1),
+                 "gate_create: a hash gate needs tid2eid [vocab_size, top_k]");
     Gate *G = new (std::nothrow) Gate();
     DMOE_REQUIRE(G != nullptr, "gate_create: out of host memory");
     hipStream_t st = to_hip(s);
@@ -287,6 +318,12 @@ int dmoe_gate_create(dmoe_gate *out, const dmoe_gate_desc *d, dmoe_stream s) {
             if ((e = hipMalloc((void **)&G->mask, (size_t)G->E)) != hipSuccess) { rc = hip_fail(e, "gate mask"); break; }
             if ((e = hipMemcpyAsync(G->mask, d->resident_mask, (size_t)G->E, kind, st)) != hipSuccess) { rc = hip_fail(e, "gate mask upload"); break; }
         }
+        if (d->is_hash) {
+            const size_t tb = sizeof(int32_t) * (size_t)d->vocab_size * G->K;
+            G->vocab = d->vocab_size;
+            if ((e = hipMalloc((void **)&G->tid2eid, tb)) != hipSuccess) { rc = hip_fail(e, "gate tid2eid"); break; }
+            if ((e = hipMemcpyAsync(G->tid2eid, d->tid2eid, tb, kind, st)) != hipSuccess) { rc = hip_fail(e, "gate tid2eid upload"); break; }
+        }
         // host sources may be pageable and may be released by the caller right after this call
         if ((e = hipStreamSynchronize(st)) != hipSuccess) { rc = hip_fail(e, "gate_create sync"); break; }
     } while (0);
@@ -295,6 +332,7 @@ int dmoe_gate_create(dmoe_gate *out, const dmoe_gate_desc *d, dmoe_stream s) {
         if (G->wgp) (void)hipFree(G->wgp);
         if (G->bias) (void)hipFree(G->bias);
         if (G->mask) (void)hipFree(G->mask);
+        if (G->tid2eid) (void)hipFree(G->tid2eid);
         delete G;
         return rc;
     }
@@ -308,12 +346,13 @@ int dmoe_gate_destroy(dmoe_gate gate) {
     if (G->wgp) (void)hipFree(G->wgp);
     if (G->bias) (void)hipFree(G->bias);
     if (G->mask) (void)hipFree(G->mask);
+    if (G->tid2eid) (void)hipFree(G->tid2eid);
     delete G;
     return DMOE_OK;
 }
 
 int dmoe_gate_forward(uint32_t *d_out_indices, float *d_out_weights, float *d_out_scores, dmoe_gate gate,
-                      const uint16_t *d_x, int T, dmoe_workspace ws, dmoe_stream s) {
+                      const uint16_t *d_x, const uint32_t *d_input_ids, int T, dmoe_workspace ws, dmoe_stream s) {
     Gate *G = (Gate *)gate.ctx;
     DMOE_REQUIRE(G != nullptr, "gate_forward: null gate");
     DMOE_REQUIRE(T >= 0, "gate_forward: T=%d", T);
@@ -347,6 +386,13 @@ int dmoe_gate_forward(uint32_t *d_out_indices, float *d_out_weights, float *d_ou
                        n_out_seg, G->scoring);
     DMOE_LAUNCH_CHECK();
     // the reference renormalises for every scoring function except softmax (:663)
+    if (G->tid2eid && d_input_ids) { // hash layer with token ids: the table replaces the top-k (:619-636)
+        hipLaunchKernelGGL(gate_hash_route_kernel, dim3((unsigned)ceil_div(T, 256)), dim3(256), 0, st, d_out_indices,
+                           d_out_weights, scores, G->tid2eid, d_input_ids, T, G->E, G->K, G->vocab,
+                           G->scoring != DMOE_SCORE_SOFTMAX ? 1 : 0, G->route_scale);
+        DMOE_LAUNCH_CHECK();
+        return DMOE_OK;
+    }
     return dmoe_gate_route(d_out_indices, d_out_weights, scores, G->bias, G->mask, T, G->E, G->K,
                            G->scoring != DMOE_SCORE_SOFTMAX, G->route_scale, s);
 }

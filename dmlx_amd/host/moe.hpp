@@ -217,7 +217,7 @@ struct DSV4Gate {
 
     // uploads `weight` (HOST bf16 [n_routed_experts, dim]) together with the bias / mask given as host vectors
     void load(const Context &ctx, const uint16_t *weight, int dim, const float *host_bias = nullptr,
-              const uint8_t *host_mask = nullptr) {
+              const uint8_t *host_mask = nullptr, const int32_t *host_tid2eid = nullptr, int vocab_size = 0) {
         deinit();
         dmoe_gate_desc d{};
         d.weight = weight;
@@ -229,6 +229,8 @@ struct DSV4Gate {
         d.scoring_func = (int)scoring_func;
         d.route_scale = route_scale;
         d.is_hash = is_hash ? 1 : 0;
+        d.tid2eid = host_tid2eid; // [vocab_size, topk] for hash layers (deepseek_v4.zig:525)
+        d.vocab_size = vocab_size;
         d.weight_source = DMOE_WEIGHTS_COPY_FROM_HOST;
         check(dmoe_gate_create(&handle_, &d, ctx.stream()));
     }
@@ -244,8 +246,10 @@ struct DSV4Gate {
         return {w, idx};
     }
 
-    // hidden_states bf16 [T, dim] (or [B, S, dim]) -> (weights, indices); needs load()
-    std::pair<Array, Array> forwardHidden(const Context &ctx, const Array &hidden_states) const {
+    // hidden_states bf16 [T, dim] (or [B, S, dim]), optional input_ids u32 [T] (hash layers) -> (weights, indices);
+    // needs load()
+    std::pair<Array, Array> forwardHidden(const Context &ctx, const Array &hidden_states,
+                                          const Array *input_ids = nullptr) const {
         if (!handle_.ctx) throw Error(DMOE_ERR_INVALID, "DSV4Gate.forwardHidden: no router weight loaded");
         const auto &sh = hidden_states.shape();
         int T = 1;
@@ -253,7 +257,9 @@ struct DSV4Gate {
         const int K = (int)topk;
         Array idx(ctx, DType::uint32, {T, K}), w(ctx, DType::float32, {T, K});
         check(dmoe_gate_forward((uint32_t *)idx.data(), (float *)w.data(), nullptr, handle_,
-                                (const uint16_t *)hidden_states.data(), T, ctx.workspace(), ctx.stream()));
+                                (const uint16_t *)hidden_states.data(),
+                                input_ids ? (const uint32_t *)input_ids->data() : nullptr, T, ctx.workspace(),
+                                ctx.stream()));
         return {w, idx};
     }
 

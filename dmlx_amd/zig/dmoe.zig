@@ -168,12 +168,12 @@ pub const ResidentGate = struct {
         _ = c.dmoe_gate_destroy(self.handle);
     }
 
-    pub fn forward(self: *ResidentGate, ctx: Context, hidden_states: DeviceArray(u16), num_tokens: usize) Error!RouteResult {
+    pub fn forward(self: *ResidentGate, ctx: Context, hidden_states: DeviceArray(u16), input_ids: ?DeviceArray(u32), num_tokens: usize) Error!RouteResult {
         const idx = try DeviceArray(u32).alloc(num_tokens * self.topk);
         errdefer idx.deinit();
         const w = try DeviceArray(f32).alloc(num_tokens * self.topk);
         errdefer w.deinit();
-        try check(c.dmoe_gate_forward(@ptrCast(@alignCast(idx.ptr)), @ptrCast(@alignCast(w.ptr)), null, self.handle, @ptrCast(@alignCast(hidden_states.ptr)), @intCast(num_tokens), ctx.ws, ctx.stream));
+        try check(c.dmoe_gate_forward(@ptrCast(@alignCast(idx.ptr)), @ptrCast(@alignCast(w.ptr)), null, self.handle, @ptrCast(@alignCast(hidden_states.ptr)), if (input_ids) |ids| @ptrCast(@alignCast(ids.ptr)) else null, @intCast(num_tokens), ctx.ws, ctx.stream));
         return .{ .indices = idx, .weights = w, .k = self.topk, .num_tokens = num_tokens };
     }
 };

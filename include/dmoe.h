@@ -287,23 +287,27 @@ typedef struct {
     int n_experts, dim, top_k;
     int scoring_func;             /* dmoe_scoring_func */
     float route_scale;            /* :528 */
-    int is_hash;                  /* hash routing through tid2eid (:525, :619-636): must be 0, not supported */
+    int is_hash;                  /* hash routing layer (:529): experts come from tid2eid[input_ids] (:619-636) */
+    const int32_t *tid2eid;       /* i32 [vocab_size, top_k] when is_hash, else ignored (:525)    */
+    int vocab_size;
     int weight_source;            /* dmoe_weight_source */
 } dmoe_gate_desc;
 
 int dmoe_gate_create(dmoe_gate *out, const dmoe_gate_desc *desc, dmoe_stream s);
 int dmoe_gate_destroy(dmoe_gate gate);
 
-/* DSV4Gate.forward(hidden_states, input_ids = null) (deepseek_v4.zig:546-681): logits = (x @ W^T) in bf16
+/* DSV4Gate.forward(hidden_states, input_ids, stream) (deepseek_v4.zig:546-681): logits = (x @ W^T) in bf16
  * widened to f32, scoring function, then dmoe_gate_route with the gate's bias, mask, top_k and route scale
  * (renormalised unless the scoring function is softmax). Returns (weights, indices) like the reference.
  *   d_out_indices u32 [T,K]; d_out_weights f32 [T,K]; d_out_scores nullable f32 [T,n_experts]: the
- *   unbiased scores, for inspection; d_x bf16 [T,dim], 16-byte aligned.
+ *   unbiased scores, for inspection; d_x bf16 [T,dim], 16-byte aligned; d_input_ids nullable u32 [T]: on a
+ *   hash gate the indices are tid2eid[input_ids] and only the weights come from the scores (:619-636); a hash
+ *   gate called without ids selects by top-k like the reference (:618-622).
  * The order of the f32 additions in the matmul and the evaluation of exp / log are fixed by this library
  * (segments of 128 reduction elements summed left to right; polynomial exp / log), so the selected experts
  * do not depend on tile shapes or library versions; MLX's own choices are not observable from the reference. */
 int dmoe_gate_forward(uint32_t *d_out_indices, float *d_out_weights, float *d_out_scores, dmoe_gate gate,
-                      const uint16_t *d_x, int T, dmoe_workspace ws, dmoe_stream s);
+                      const uint16_t *d_x, const uint32_t *d_input_ids, int T, dmoe_workspace ws, dmoe_stream s);
 
 /* Inspection of the last dmoe_moe_forward / dmoe_switch_glu_forward_no_scores on this workspace:
  * the SwiGLU activations in flat (t*K+k) row order, bf16 [T*K, F]. For parity tests. */

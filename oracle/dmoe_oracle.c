@@ -285,6 +285,26 @@ void orc_gate_route(const float *scores, const float *bias, const uint8_t *resid
 
 /* ------------------------------------------------ remap / mask / dedup ---- */
 
+/* deepseek_v4.zig:619-636 (mlx_take_axis(tid2eid, ids, 0) -> [T,K]) followed by the common tail
+ * :655-678 (gatherScores on the unbiased scores, w / (sum_k w + 1e-20) unless softmax, * scale). */
+void orc_gate_hash_route(const float *scores, const int32_t *tid2eid, const uint32_t *ids, int T, int E,
+                         int K, int renorm, float route_scale, uint32_t *idx_out, float *w_out) {
+    for (int t = 0; t < T; t++) {
+        float sum = 0.0f;
+        for (int j = 0; j < K; j++) {
+            uint32_t e = (uint32_t)tid2eid[(size_t)ids[t] * K + j];
+            idx_out[(size_t)t * K + j] = e;
+            w_out[(size_t)t * K + j] = scores[(size_t)t * E + e];
+            sum += w_out[(size_t)t * K + j];
+        }
+        for (int j = 0; j < K; j++) {
+            float v = w_out[(size_t)t * K + j];
+            if (renorm) v = v / (sum + 1e-20f);
+            w_out[(size_t)t * K + j] = v * route_scale;
+        }
+    }
+}
+
 /* mlx_take(remap, indices) then astype(u32): deepseek_v4.zig:1035-1039,
  * expert_preload.zig:200-206, expert_stream.zig:522-529 (host loop) */
 void orc_remap(const int32_t *remap, const uint32_t *idx, size_t n, uint32_t *out) {

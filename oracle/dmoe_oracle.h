@@ -76,6 +76,10 @@ float orc_det_logf(float x);
 void orc_gate_route(const float *scores, const float *bias, const uint8_t *resident,
                     int T, int E, int K, int renorm, float route_scale,
                     uint32_t *idx_out, float *w_out);
+/* hash layers, deepseek_v4.zig:619-636 + :655-678: indices = tid2eid[input_ids], weights from the
+ * unbiased scores, renorm when not softmax, * route_scale */
+void orc_gate_hash_route(const float *scores, const int32_t *tid2eid, const uint32_t *ids, int T, int E,
+                         int K, int renorm, float route_scale, uint32_t *idx_out, float *w_out);
 /* mlx_take(remap, indices): deepseek_v4.zig:1037, expert_preload.zig:202 */
 void orc_remap(const int32_t *remap, const uint32_t *idx, size_t n, uint32_t *out);
 /* deepseek_v4_loader.zig:272-293; returns the number of resident experts */

@@ -165,6 +165,18 @@ def gate_route(scores, bias, resident, K, renorm, route_scale):
     return idx, w
 
 
+def gate_hash_route(scores, tid2eid, ids, renorm, route_scale):
+    s = _c(scores, np.float32)
+    t2e = _c(tid2eid, np.int32)
+    i = _c(ids, np.uint32)
+    T, E = s.shape
+    K = t2e.shape[1]
+    idx = np.empty((T, K), np.uint32)
+    w = np.empty((T, K), np.float32)
+    lib().orc_gate_hash_route(_p(s), _p(t2e), _p(i), T, E, K, int(renorm), C.c_float(route_scale), _p(idx), _p(w))
+    return idx, w
+
+
 def remap(remap_table, idx):
     r = _c(remap_table, np.int32)
     i = _c(idx, np.uint32)

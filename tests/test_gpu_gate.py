@@ -64,6 +64,30 @@ def test_gate_extreme_logits(dmoe, orc, ws):
         gate.close()
 
 
+@pytest.mark.parametrize("func", [0, 2])
+def test_hash_gate_takes_experts_from_the_table(dmoe, orc, ws, func):
+    """Hash layers (deepseek_v4.zig:619-636): indices = tid2eid[input_ids]; weights from the unbiased scores."""
+    T, D, E, K, vocab = 37, 256, 64, 6, 500
+    x, wg, bias, _ = _case(21, T, D, E, True, False, spread=2.0)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    tid2eid = torch.stack([torch.randperm(E, generator=g, device="cuda")[:K] for _ in range(vocab)]).to(torch.int32)
+    ids = torch.randint(0, vocab, (T,), generator=g, device="cuda", dtype=torch.int32)
+    gate = dmoe.Gate(wg, K, func, route_scale=2.5, bias=bias, tid2eid=tid2eid)
+    idx, w, scores = gate.forward(x, ws, want_scores=True, input_ids=ids)
+    want_scores = orc.gate_scores_det(orc.gate_logits(bf16_bits(x), bf16_bits(wg)), func)
+    np.testing.assert_array_equal(scores.cpu().numpy().view(np.uint32), want_scores.view(np.uint32))
+    want_idx, want_w = orc.gate_hash_route(want_scores, tid2eid.cpu().numpy(), to_np_u32(ids), func != 0, 2.5)
+    np.testing.assert_array_equal(to_np_u32(idx), want_idx)
+    np.testing.assert_array_equal(w.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
+    # the table decides, not the scores: the indices are exactly the rows of the table
+    np.testing.assert_array_equal(to_np_u32(idx), tid2eid.cpu().numpy()[to_np_u32(ids).astype(np.int64)].astype(np.uint32))
+    # without token ids a hash gate falls back to score-based top-k, like the reference
+    idx2, w2 = gate.forward(x, ws)
+    ref_idx, ref_w = orc.gate_route(want_scores, bias.cpu().numpy(), None, K, func != 0, 2.5)
+    np.testing.assert_array_equal(to_np_u32(idx2), ref_idx)
+    gate.close()
+
+
 def test_gate_rejects_bad_arguments(dmoe):
     wg = torch.zeros((8, 64), device="cuda", dtype=torch.bfloat16)
     with pytest.raises(dmoe.DmoeError):

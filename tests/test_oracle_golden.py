@@ -436,3 +436,18 @@ def test_gate_scores_det_agree_with_libm(orc):
         np.testing.assert_allclose(a, b, rtol=2e-6, atol=1e-12)
     sm = orc.gate_scores_det(logits, 0)
     np.testing.assert_allclose(sm.sum(1), 1.0, rtol=1e-6)
+
+
+def test_hash_route_is_a_table_lookup_with_renormalised_scores(orc):
+    rng = np.random.default_rng(8)
+    T, E, K, vocab = 11, 16, 3, 40
+    scores = rng.random((T, E)).astype(np.float32)
+    t2e = np.stack([rng.permutation(E)[:K] for _ in range(vocab)]).astype(np.int32)
+    ids = rng.integers(0, vocab, T).astype(np.uint32)
+    idx, w = orc.gate_hash_route(scores, t2e, ids, True, 1.5)
+    np.testing.assert_array_equal(idx, t2e[ids].astype(np.uint32))
+    picked = np.take_along_axis(scores, t2e[ids].astype(np.int64), 1).astype(np.float64)
+    np.testing.assert_allclose(w, 1.5 * picked / picked.sum(1, keepdims=True), rtol=1e-6)
+    np.testing.assert_allclose(w.sum(1), 1.5, rtol=1e-6)
+    _, w_raw = orc.gate_hash_route(scores, t2e, ids, False, 1.0)
+    np.testing.assert_array_equal(w_raw, np.take_along_axis(scores, t2e[ids].astype(np.int64), 1))
