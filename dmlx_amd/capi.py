@@ -70,7 +70,7 @@ EXPORTS = [
     "dmoe_layer_create", "dmoe_layer_destroy", "dmoe_moe_forward",
     "dmoe_switch_glu_forward_no_scores", "dmoe_moe_layer_forward", "dmoe_debug_last_activations",
     "dmoe_gate_create", "dmoe_gate_destroy", "dmoe_gate_forward",
-    "dmoe_layer_create_from_safetensors", "dmoe_layer_dims",
+    "dmoe_layer_create_from_safetensors", "dmoe_layer_dims", "dmoe_batch_build",
 ]
 
 _lib = None
@@ -261,6 +261,22 @@ def gather_qmm(x, qw, rhs_indices, ws, lhs_indices=None, sorted_indices=False):
     check(lib().dmoe_gather_qmm(_ptr(out), _ptr(x), C.byref(c), _ptr(lhs_indices), _ptr(rhs_indices), R,
                                 int(sorted_indices), ws.h, _stream()))
     return out
+
+
+def batch_build(tokens, seq_lens, base_pos, ws, want_mask=True):
+    """dmoe_batch_build: host lists in, (tokens u32 [T], positions i32 [T], mask f32 [T,T] | None, request_of_token)"""
+    T, n = len(tokens), len(seq_lens)
+    dev = "cuda"
+    d_tok = torch.empty(T, dtype=torch.int32, device=dev)
+    d_pos = torch.empty(T, dtype=torch.int32, device=dev)
+    d_req = torch.empty(T, dtype=torch.int32, device=dev)
+    d_mask = torch.empty((T, T), dtype=torch.float32, device=dev) if want_mask else None
+    h_tok = (C.c_uint32 * max(T, 1))(*[int(v) for v in tokens])
+    h_len = (C.c_int32 * max(n, 1))(*[int(v) for v in seq_lens])
+    h_base = (C.c_int32 * max(n, 1))(*[int(v) for v in base_pos])
+    check(lib().dmoe_batch_build(_ptr(d_tok), _ptr(d_pos), _ptr(d_mask), _ptr(d_req), h_tok, h_len, h_base, n, T,
+                                 ws.h, _stream()))
+    return d_tok, d_pos, d_mask, d_req
 
 
 class Gate:

@@ -502,6 +502,34 @@ inline BatchResult build(const std::vector<const Request *> &prefill_requests, c
     out.request_offsets.push_back((int32_t)out.total_tokens);
     return out;
 }
+// the same batch on the device: tokens, positions, [T,T] mask (optional) and the token -> request map
+struct DeviceBatch {
+    Array batched_tokens, position_ids, attention_mask, request_of_token;
+    size_t total_tokens = 0, num_requests = 0;
+};
+inline DeviceBatch buildOnDevice(const Context &ctx, const std::vector<const Request *> &prefill_requests,
+                                 const std::vector<const Request *> &decode_requests, bool want_mask) {
+    const BatchResult host = build(prefill_requests, decode_requests);
+    DeviceBatch out;
+    out.total_tokens = host.total_tokens;
+    out.num_requests = host.num_requests;
+    const int T = (int)host.total_tokens, n = (int)host.num_requests;
+    if (T == 0) return out; // emptyBatch
+    std::vector<int32_t> lens((size_t)n), base((size_t)n);
+    for (int i = 0; i < n; ++i) {
+        lens[(size_t)i] = host.request_offsets[(size_t)i + 1] - host.request_offsets[(size_t)i];
+        base[(size_t)i] = lens[(size_t)i] ? host.position_ids[(size_t)host.request_offsets[(size_t)i]] : 0;
+    }
+    out.batched_tokens = Array(ctx, DType::uint32, {T});
+    out.position_ids = Array(ctx, DType::int32, {T});
+    out.request_of_token = Array(ctx, DType::uint32, {T});
+    if (want_mask) out.attention_mask = Array(ctx, DType::float32, {T, T});
+    check(dmoe_batch_build((uint32_t *)out.batched_tokens.data(), (int32_t *)out.position_ids.data(),
+                           want_mask ? (float *)out.attention_mask.data() : nullptr,
+                           (uint32_t *)out.request_of_token.data(), host.batched_tokens.data(), lens.data(), base.data(), n, T,
+                           ctx.workspace(), ctx.stream()));
+    return out;
+}
 } // namespace batch_builder
 
 } // namespace dmoe

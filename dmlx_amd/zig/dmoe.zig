@@ -178,6 +178,12 @@ pub const ResidentGate = struct {
     }
 };
 
+/// batch_builder.build with the per-token work on the device (src/batch_builder.zig:90-214): `tokens` are the
+/// concatenated getRequestTokens results, prefill requests first.
+pub fn batchBuild(ctx: Context, tokens: []const u32, seq_lens: []const i32, base_pos: []const i32, out_tokens: DeviceArray(u32), out_positions: DeviceArray(i32), out_mask: ?DeviceArray(f32)) Error!void {
+    try check(c.dmoe_batch_build(@ptrCast(@alignCast(out_tokens.ptr)), @ptrCast(@alignCast(out_positions.ptr)), if (out_mask) |m| @ptrCast(@alignCast(m.ptr)) else null, null, tokens.ptr, seq_lens.ptr, base_pos.ptr, @intCast(seq_lens.len), @intCast(tokens.len), ctx.ws, ctx.stream));
+}
+
 /// One-time resident upload of a layer's experts from MLX-format safetensors shards (what
 /// model_registry.zig:255-329 prepares for on-demand reads). `paths` are NUL-terminated.
 pub fn layerFromSafetensors(ctx: Context, paths: []const [*:0]const u8, layer_idx: usize, top_k: usize, mode: [*:0]const u8, group_size: i32, bits: i32, swiglu_limit: f32, smelt_mask: ?[]const u8) Error!c.dmoe_layer {

@@ -309,6 +309,23 @@ int dmoe_gate_destroy(dmoe_gate gate);
 int dmoe_gate_forward(uint32_t *d_out_indices, float *d_out_weights, float *d_out_scores, dmoe_gate gate,
                       const uint16_t *d_x, const uint32_t *d_input_ids, int T, dmoe_workspace ws, dmoe_stream s);
 
+/* ---- continuous-batch assembly ---------------------------------------------------------------- */
+
+/* batch_builder.build (batch_builder.zig:90-214) with the per-token work on the device. The caller walks its
+ * requests (prefill requests first, then decode ones, :104-111), concatenates their tokens
+ * (getRequestTokens, :47-83) and passes per request the token count and the position of its first token
+ * (:146-153). Outputs, each nullable:
+ *   d_out_tokens u32 [T]           batched_tokens (a copy of h_tokens)
+ *   d_out_positions i32 [T]        position_ids: base_pos[r] + index within request r
+ *   d_out_mask f32 [T,T]           attention_mask: 0 where row and column belong to the same request and
+ *                                  column <= row, -inf elsewhere (:140-177); 16-byte aligned, T <= 65535
+ *   d_out_request_of_token u32 [T] request index of every token (no counterpart in the reference; the
+ *                                  per-request view of a packed batch)
+ * Host inputs are read before the call returns. T = sum of h_seq_lens; T == 0 is the empty batch. */
+int dmoe_batch_build(uint32_t *d_out_tokens, int32_t *d_out_positions, float *d_out_mask,
+                     uint32_t *d_out_request_of_token, const uint32_t *h_tokens, const int32_t *h_seq_lens,
+                     const int32_t *h_base_pos, int n_requests, int T, dmoe_workspace ws, dmoe_stream s);
+
 /* Inspection of the last dmoe_moe_forward / dmoe_switch_glu_forward_no_scores on this workspace:
  * the SwiGLU activations in flat (t*K+k) row order, bf16 [T*K, F]. For parity tests. */
 int dmoe_debug_last_activations(uint16_t *d_out, dmoe_layer layer, int T, dmoe_workspace ws, dmoe_stream s);

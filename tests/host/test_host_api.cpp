@@ -166,6 +166,16 @@ static void test_remap_smelt_batch(const Context &ctx) {
     c.state = Request::State::waiting;
     c.prompt_tokens = {40};
     auto br = batch_builder::build({&a, &c}, {&b});
+    {
+        auto db = batch_builder::buildOnDevice(ctx, {&a, &c}, {&b}, true);
+        EXPECT(db.total_tokens == br.total_tokens && db.num_requests == br.num_requests);
+        auto pos = db.position_ids.dataSlice<int32_t>();
+        auto tok = db.batched_tokens.dataSlice<uint32_t>();
+        auto msk = db.attention_mask.dataSlice<float>();
+        for (size_t i = 0; i < br.total_tokens; ++i) EXPECT(pos[i] == br.position_ids[i] && tok[i] == br.batched_tokens[i]);
+        const size_t T = br.total_tokens;
+        EXPECT(msk[0] == 0.0f && std::isinf(msk[1]) && msk[(T - 1) * T + (T - 1)] == 0.0f);
+    }
     EXPECT(br.total_tokens == 5 && br.num_requests == 3);
     EXPECT(br.batched_tokens == std::vector<uint32_t>({12, 13, 14, 40, 31}));
     EXPECT(br.position_ids == std::vector<int32_t>({2, 3, 4, 0, 4}));
