@@ -138,9 +138,9 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArg
     }
     if (!wave_on) return;
 
-    // A-operand source of this lane: tile row ln (zeros beyond the tile), reduction half h
-    const bool x_on = ln < nrows;
-    const uint8_t *xlane = xs_lds + (x_on ? ln : 0) * pitch + h * KV * 2;
+    // A-operand source of this lane: tile row ln, reduction half h. Lanes past the tile's rows read row 0 again:
+    // their operand rows only reach accumulator rows that are never stored.
+    const uint8_t *xlane = xs_lds + (ln < nrows ? ln : 0) * pitch + h * KV * 2;
 
     f32x16_t acc[NM];
 #pragma unroll
@@ -152,56 +152,80 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArg
     for (int mi = 0; mi < NM; ++mi)
 #pragma unroll
         for (int r = 0; r < 4; ++r) facc[mi][r] = 0.0f;
+    const uint32_t mask = vgpr_const32(0x000f000fu), magic = vgpr_const32(0x43004300u);
 
+    // One step: decode every projection's chunk first, then issue the matrix instructions of the projections
+    // alternately (two independent accumulation chains: a dependent MFMA never follows its producer directly),
+    // then apply the scales.
     auto consume = [&](int step, const SkinnyStage<NM> &s) {
         bf16x8_t xf[NJ];
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
-            uint4 q = make_uint4(0, 0, 0, 0);
-            if (x_on) q = *(const uint4 *)(xlane + (size_t)step * KSTEP * 2 + j * 16);
+            uint4 q = *(const uint4 *)(xlane + (size_t)step * KSTEP * 2 + j * 16);
             xf[j] = __builtin_bit_cast(bf16x8_t, q);
         }
         float4 gsum = make_float4(0.f, 0.f, 0.f, 0.f);
         if (FACTORED) gsum = *(const float4 *)(gs_lds + step * kSkinnyTileM + 4 * h);
+        uint32_t wp[NM][KV / 2];
+        Meta meta[NM];
 #pragma unroll
         for (int mi = 0; mi < NM; ++mi) {
-            const Meta meta = CS::meta(s.sb[mi]);
-            uint32_t wp[KV / 2];
+            meta[mi] = CS::meta(s.sb[mi]);
             if (FACTORED) {
-                const uint32_t mask = vgpr_const32(0x000f000fu), magic = vgpr_const32(0x43004300u);
-                codes_to_bf16(s.raw[mi].x, mask, magic, wp);
-                codes_to_bf16(s.raw[mi].y, mask, magic, wp + 4);
-                codes_to_bf16(s.raw[mi].z, mask, magic, wp + 8);
-                codes_to_bf16(s.raw[mi].w, mask, magic, wp + 12);
-                f32x16_t p;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) p[r] = 0.0f;
-#pragma unroll
-                for (int j = 0; j < NJ; ++j) {
-                    uint4 q = make_uint4(wp[4 * j], wp[4 * j + 1], wp[4 * j + 2], wp[4 * j + 3]);
-                    p = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[j], __builtin_bit_cast(bf16x8_t, q), p, 0, 0, 0);
-                }
-                const float boff = fmaf(-128.0f, meta.s, meta.b);
-                facc[mi][0] = fmaf(meta.s, p[0], fmaf(boff, gsum.x, facc[mi][0]));
-                facc[mi][1] = fmaf(meta.s, p[1], fmaf(boff, gsum.y, facc[mi][1]));
-                facc[mi][2] = fmaf(meta.s, p[2], fmaf(boff, gsum.z, facc[mi][2]));
-                facc[mi][3] = fmaf(meta.s, p[3], fmaf(boff, gsum.w, facc[mi][3]));
+                codes_to_bf16(s.raw[mi].x, mask, magic, wp[mi]);
+                codes_to_bf16(s.raw[mi].y, mask, magic, wp[mi] + 4);
+                codes_to_bf16(s.raw[mi].z, mask, magic, wp[mi] + 8);
+                codes_to_bf16(s.raw[mi].w, mask, magic, wp[mi] + 12);
             } else {
-                Fmt::decode_fast(s.raw[mi], meta, wp);
+                Fmt::decode_fast(s.raw[mi], meta[mi], wp[mi]);
+            }
+        }
+        f32x16_t p[NM];
+        if (FACTORED) {
 #pragma unroll
-                for (int j = 0; j < NJ; ++j) {
-                    uint4 q = make_uint4(wp[4 * j], wp[4 * j + 1], wp[4 * j + 2], wp[4 * j + 3]);
+            for (int mi = 0; mi < NM; ++mi)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) p[mi][r] = 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+            for (int mi = 0; mi < NM; ++mi) {
+                uint4 q = make_uint4(wp[mi][4 * j], wp[mi][4 * j + 1], wp[mi][4 * j + 2], wp[mi][4 * j + 3]);
+                if (FACTORED)
+                    p[mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[j], __builtin_bit_cast(bf16x8_t, q), p[mi], 0, 0, 0);
+                else
                     acc[mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[j], __builtin_bit_cast(bf16x8_t, q), acc[mi], 0, 0, 0);
-                }
+            }
+        }
+        if (FACTORED) {
+#pragma unroll
+            for (int mi = 0; mi < NM; ++mi) {
+                const float boff = fmaf(-128.0f, meta[mi].s, meta[mi].b);
+                facc[mi][0] = fmaf(meta[mi].s, p[mi][0], fmaf(boff, gsum.x, facc[mi][0]));
+                facc[mi][1] = fmaf(meta[mi].s, p[mi][1], fmaf(boff, gsum.y, facc[mi][1]));
+                facc[mi][2] = fmaf(meta[mi].s, p[mi][2], fmaf(boff, gsum.z, facc[mi][2]));
+                facc[mi][3] = fmaf(meta[mi].s, p[mi][3], fmaf(boff, gsum.w, facc[mi][3]));
             }
         }
     };
 
+    // whole rounds of the ring run without guards (the look-ahead is clamped onto the last step: a few repeated
+    // loads at the very end instead of a branch per step); a partial last round runs the guarded copy
+    const int full = n_steps / kSkinnyStages * kSkinnyStages;
 #pragma unroll 1
-    for (int s0 = 0; s0 < n_steps; s0 += kSkinnyStages) {
+    for (int s0 = 0; s0 < full; s0 += kSkinnyStages) {
 #pragma unroll
         for (int j = 0; j < kSkinnyStages; ++j) {
-            const int step = s0 + j;
+            const int step = s0 + j, ahead = step + kSkinnyStages - 1;
+            load_stage(ahead < n_steps ? ahead : n_steps - 1, ring[(j + kSkinnyStages - 1) % kSkinnyStages]);
+            consume(step, ring[j]);
+        }
+    }
+    if (full < n_steps) {
+#pragma unroll
+        for (int j = 0; j < kSkinnyStages; ++j) {
+            const int step = full + j;
             if (step + kSkinnyStages - 1 < n_steps) load_stage(step + kSkinnyStages - 1, ring[(j + kSkinnyStages - 1) % kSkinnyStages]);
             if (step < n_steps) consume(step, ring[j]);
         }
