@@ -335,6 +335,12 @@ struct ChunkStream {
             brow = q.biases ? q.biases + mat * q.s_mat + (size_t)n_clamped * q.s_row : nullptr;
         }
     }
+    // compiler-level fence on the chunk addresses: chunk loads issued after pin() stay behind every earlier asm
+    // statement (used to keep them younger than hand-issued memory requests)
+    __device__ __forceinline__ void pin() {
+        if (PACKED) asm volatile("" : "+v"(wlane));
+        else asm volatile("" : "+v"(w));
+    }
     __device__ __forceinline__ uint4 load_chunk(int step) const {
         return *(const uint4 *)(w + (size_t)step * (PACKED ? 1024 : 32) + wlane);
     }

@@ -40,6 +40,15 @@ __device__ __forceinline__ void codes_to_bf16(uint32_t w, uint32_t mask, uint32_
     o[3] = ((w >> 12) & mask) | magic;
 }
 
+// s_waitcnt immediate for "at most n vector-memory loads outstanding" (gfx9: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14])
+constexpr int skinny_wait_vmcnt(int n) { return 0x0f70 | (n & 15) | ((n >> 4) << 14); }
+
+template <int CTRL>
+__device__ __forceinline__ float skinny_dpp(float x) {
+    const int v = __float_as_int(x);
+    return __int_as_float(__builtin_amdgcn_update_dpp(v, v, CTRL, 0xf, 0xf, false));
+}
+
 template <int NM>
 struct SkinnyStage {
     uint4 raw[NM];
@@ -90,49 +99,70 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArg
         }
     };
 
-    // the first weight loads depend on the tile only: issue them before anything else
-    SkinnyStage<NM> ring[kSkinnyStages];
-    if (wave_on) {
-#pragma unroll
-        for (int j = 0; j < kSkinnyStages - 1; ++j)
-            if (j < n_steps) load_stage(j, ring[j]);
-    }
-
-    // ---- activations of the tile -> LDS ---------------------------------------------------------------
+    // ---- activations of the tile -> LDS, ahead of the weights ---------------------------------------------
+    // Loads return in issue order, so the tile's activation rows are requested first (straight into LDS, no
+    // registers), then the first stages of the weight ring; the wait below lets the ring stay in flight.
     // Only the rows the tile has are staged (most decode tiles hold one to three): row m of the A operand only
-    // reaches accumulator row m, and accumulator rows past the tile are never stored, so whatever the lanes of the
-    // missing rows feed the matrix core does not matter (they feed zeros, see x_on below).
+    // reaches accumulator row m, and accumulator rows past the tile are never stored.
     const int pitch = cols * 2 + 16; // bytes per LDS row; +16 keeps the 8 rows on different banks
-    const int nrows = (int)t.nrows;
+    const int nrows = __builtin_amdgcn_readfirstlane((int)t.nrows);
     uint8_t *xs_lds = skinny_lds;
     float *gs_lds = (float *)(skinny_lds + kSkinnyTileM * pitch); // [n_steps][8]: per-step sums of x (factored)
     {
-        const int pieces = cols / 8; // 16-byte pieces per row
-        for (int idx = tid; idx < nrows * pieces; idx += kSkinnyWaves * 64) {
-            const int r = idx / pieces, pc = idx - r * pieces;
-            const uint32_t p = t.row0 + (uint32_t)r;
-            const size_t src = g.a_rows ? g.a_rows[p] : p;
-            uint4 v = *(const uint4 *)(g.a + src * (size_t)cols + pc * 8);
-            if (FACTORED) { // (x0..x7) -> (x0,x4,x1,x5,x2,x6,x3,x7), the order the code pairs come out in
-                uint4 o;
-                o.x = (v.x & 0xffffu) | (v.z << 16);
-                o.y = (v.x >> 16) | (v.z & 0xffff0000u);
-                o.z = (v.y & 0xffffu) | (v.w << 16);
-                o.w = (v.y >> 16) | (v.w & 0xffff0000u);
-                v = o;
+        const uint32_t lds_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)skinny_lds;
+        const uint32_t row0 = __builtin_amdgcn_readfirstlane(t.row0);
+        const int row_bytes = cols * 2;
+        // source rows of the tile: one load for all of them (lane r holds row r's), then uniform reads
+        uint32_t src_of_lane = row0 + (uint32_t)(lane < nrows ? lane : 0);
+        if (g.a_rows) src_of_lane = g.a_rows[src_of_lane];
+        for (int r = 0; r < nrows; ++r) {
+            const size_t src = (uint32_t)__builtin_amdgcn_readlane((int)src_of_lane, r);
+            const uint8_t *row = (const uint8_t *)(g.a + src * (size_t)cols) + lane * 16;
+            for (int c = wave * 1024; c < row_bytes; c += kSkinnyWaves * 1024) {
+                const uint32_t la = lds_addr + (uint32_t)(r * pitch + c); // uniform; lane i lands at la + 16 i
+                const uint8_t *gp = row + c;
+                if (c + lane * 16 < row_bytes)
+                    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gp), "s"(la) : "memory"); // nothing else in this kernel uses M0
             }
-            *(uint4 *)(xs_lds + r * pitch + pc * 16) = v;
         }
+    }
+    SkinnyStage<NM> ring[kSkinnyStages];
+    const bool ring_full = n_steps >= kSkinnyStages - 1;
+    if (wave_on) {
+#pragma unroll
+        for (int mi = 0; mi < NM; ++mi) cs[mi].pin(); // keeps the weight loads behind the requests above
+#pragma unroll
+        for (int j = 0; j < kSkinnyStages - 1; ++j)
+            if (j < n_steps) load_stage(j, ring[j]);
+        // every ring stage holds at least NM loads younger than the activation requests
+        if (ring_full) __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt((kSkinnyStages - 1) * NM));
+        else __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt(0));
+    } else {
+        __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt(0));
     }
     __syncthreads();
     if (FACTORED) {
-        for (int idx = tid; idx < n_steps * nrows; idx += kSkinnyWaves * 64) {
-            const int step = idx / nrows, r = idx - step * nrows;
-            const uint32_t *px = (const uint32_t *)(xs_lds + r * pitch + step * KSTEP * 2);
-            float sum = 0.0f;
-#pragma unroll 8
-            for (int i = 0; i < KSTEP / 2; ++i) sum += bf16_bits_to_f32(px[i] & 0xffffu) + bf16_bits_to_f32(px[i] >> 16);
-            gs_lds[step * kSkinnyTileM + r] = sum;
+        // per 16-byte piece: (x0..x7) -> (x0,x4,x1,x5,x2,x6,x3,x7), the order the code pairs come out in, and the
+        // sum of each step's 64 activations (eight pieces, eight neighbouring lanes)
+        const int pieces = cols / 8;
+        for (int idx = tid; idx < nrows * pieces; idx += kSkinnyWaves * 64) {
+            const int r = idx / pieces, pc = idx - r * pieces;
+            uint4 *px = (uint4 *)(xs_lds + r * pitch + pc * 16);
+            const uint4 v = *px;
+            float sum = (bf16_bits_to_f32(v.x & 0xffffu) + bf16_bits_to_f32(v.x >> 16)) +
+                        (bf16_bits_to_f32(v.y & 0xffffu) + bf16_bits_to_f32(v.y >> 16)) +
+                        (bf16_bits_to_f32(v.z & 0xffffu) + bf16_bits_to_f32(v.z >> 16)) +
+                        (bf16_bits_to_f32(v.w & 0xffffu) + bf16_bits_to_f32(v.w >> 16));
+            uint4 o;
+            o.x = (v.x & 0xffffu) | (v.z << 16);
+            o.y = (v.x >> 16) | (v.z & 0xffff0000u);
+            o.z = (v.y & 0xffffu) | (v.w << 16);
+            o.w = (v.y >> 16) | (v.w & 0xffff0000u);
+            *px = o;
+            sum += skinny_dpp<0xB1>(sum);  // lane ^ 1 (quad_perm 1,0,3,2)
+            sum += skinny_dpp<0x4E>(sum);  // lane ^ 2 (quad_perm 2,3,0,1)
+            sum += skinny_dpp<0x141>(sum); // the other quad of the eight lanes (row_half_mirror)
+            if ((pc & 7) == 0) gs_lds[(pc >> 3) * kSkinnyTileM + r] = sum;
         }
         __syncthreads();
     }
