@@ -392,17 +392,21 @@ static int forward_common(uint16_t *d_out, uint16_t *y_out, Layer *L, const uint
     }
     // The shared expert does not depend on the routing: it runs on the workspace's side stream, forked
     // here and joined before the combine, so its two small dense GEMMs overlap pack and the routed GEMMs.
+    // The routed launches are enqueued first: they are the critical path, and the host has all of their run
+    // time to enqueue the side stream's work.
     const bool shared = with_shared && L->has_shared && !y_out;
     if (shared) {
         DMOE_TRY(side_stream_ready(w));
         DMOE_HIP(hipEventRecord(w->fork, st));
+    }
+    DMOE_TRY(routed_forward(L, w, f, d_x, slots, d_scores, T, y_out, st));
+    if (shared) {
         DMOE_HIP(hipStreamWaitEvent(w->side, w->fork, 0));
         DMOE_TRY(stage_begin(w, DMOE_STAGE_SHARED, w->side));
         DMOE_TRY(shared_forward(L, w, f, d_x, T, w->side));
         DMOE_TRY(stage_end(w, DMOE_STAGE_SHARED, w->side));
         DMOE_HIP(hipEventRecord(w->join, w->side));
     }
-    DMOE_TRY(routed_forward(L, w, f, d_x, slots, d_scores, T, y_out, st));
     if (y_out) return DMOE_OK;
     if (shared) DMOE_HIP(hipStreamWaitEvent(st, w->join, 0));
     DMOE_TRY(stage_begin(w, DMOE_STAGE_COMBINE, st));

@@ -23,7 +23,10 @@
 
 namespace dmoe {
 
-constexpr int kSkinnyWaves = 4;
+constexpr int kSkinnyWaves = 4;          // 32-row blocks of weight rows per workgroup
+// gate/up launches give each projection its own wavefront (eight per workgroup, paired through LDS at the end):
+// half the registers per wavefront, twice the wavefronts per SIMD to overlap decode, matrix and memory waits
+constexpr bool kSkinnySplitGateUp = true;
 constexpr int kSkinnyStages = 8;
 
 __device__ __forceinline__ uint32_t vgpr_const32(uint32_t c) {
@@ -56,12 +59,14 @@ struct SkinnyStage {
 };
 
 template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED>
-__global__ __launch_bounds__(kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArgs g) {
+__global__ __launch_bounds__((GATE_UP && kSkinnySplitGateUp ? 2 : 1) * kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArgs g) {
     using CS = ChunkStream<Fmt, PACKED>;
     constexpr int KV = Fmt::kVals;   // values per 16-byte chunk
     constexpr int KSTEP = 2 * KV;    // reduction elements per step (both lane halves)
     constexpr int NJ = KV / 8;       // MFMAs (K = 16) per step
-    constexpr int NM = GATE_UP ? 2 : 1;
+    constexpr bool SPLIT = GATE_UP && kSkinnySplitGateUp;
+    constexpr int NM = GATE_UP && !SPLIT ? 2 : 1;   // projections per wavefront
+    constexpr int WAVES = (SPLIT ? 2 : 1) * kSkinnyWaves;
     extern __shared__ __attribute__((aligned(16))) uint8_t skinny_lds[];
 
     Tile t;
@@ -84,18 +89,19 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArg
     const size_t e = t.expert;
 
     // ---- this lane's weight row ------------------------------------------------------------------------
-    const int col0 = ((int)blockIdx.x * kSkinnyWaves + wave) * 32;
+    const int proj = SPLIT ? (wave & 1) : 0;        // split: even wavefronts take gate rows, odd ones up rows
+    const int col0 = ((int)blockIdx.x * kSkinnyWaves + (SPLIT ? wave >> 1 : wave)) * 32;
     const bool wave_on = col0 < n_out;
     int n = col0 + ln;
     if (n >= n_out) n = n_out - 1; // stay inside the matrix; such rows are never stored
     CS cs[NM];
 #pragma unroll
-    for (int mi = 0; mi < NM; ++mi) cs[mi].init(mi == 0 ? g.b0 : g.b1, e, col0 >> 5, ln, h, n);
+    for (int mi = 0; mi < NM; ++mi) cs[mi].init((mi + proj) == 0 ? g.b0 : g.b1, e, col0 >> 5, ln, h, n);
     auto load_stage = [&](int step, SkinnyStage<NM> &s) {
 #pragma unroll
         for (int mi = 0; mi < NM; ++mi) {
             s.raw[mi] = cs[mi].load_chunk_stream(step);
-            cs[mi].load_meta(mi == 0 ? g.b0 : g.b1, step, s.sb[mi]);
+            cs[mi].load_meta((mi + proj) == 0 ? g.b0 : g.b1, step, s.sb[mi]);
         }
     };
 
@@ -118,7 +124,7 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArg
         for (int r = 0; r < nrows; ++r) {
             const size_t src = (uint32_t)__builtin_amdgcn_readlane((int)src_of_lane, r);
             const uint8_t *row = (const uint8_t *)(g.a + src * (size_t)cols) + lane * 16;
-            for (int c = wave * 1024; c < row_bytes; c += kSkinnyWaves * 1024) {
+            for (int c = wave * 1024; c < row_bytes; c += WAVES * 1024) {
                 const uint32_t la = lds_addr + (uint32_t)(r * pitch + c); // uniform; lane i lands at la + 16 i
                 const uint8_t *gp = row + c;
                 if (c + lane * 16 < row_bytes)
@@ -145,7 +151,7 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArg
         // per 16-byte piece: (x0..x7) -> (x0,x4,x1,x5,x2,x6,x3,x7), the order the code pairs come out in, and the
         // sum of each step's 64 activations (eight pieces, eight neighbouring lanes)
         const int pieces = cols / 8;
-        for (int idx = tid; idx < nrows * pieces; idx += kSkinnyWaves * 64) {
+        for (int idx = tid; idx < nrows * pieces; idx += WAVES * 64) {
             const int r = idx / pieces, pc = idx - r * pieces;
             uint4 *px = (uint4 *)(xs_lds + r * pitch + pc * 16);
             const uint4 v = *px;
@@ -262,22 +268,31 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArg
     }
 
     // ---- epilogue: this lane holds rows 4h..4h+3 of the tile for weight row n --------------------------
-    if (col0 + ln >= n_out) return;
-    float rs[NM];
+    const bool lane_on = col0 + ln < n_out;
+    float v[2][4];
 #pragma unroll
     for (int mi = 0; mi < NM; ++mi) {
-        const QView &q = mi == 0 ? g.b0 : g.b1;
-        rs[mi] = Fmt::kRowScale ? *(const float *)(q.scales + e * q.s_mat + (size_t)n * q.s_row) : 1.0f;
+        const QView &q = (mi + proj) == 0 ? g.b0 : g.b1;
+        const float rs = Fmt::kRowScale ? *(const float *)(q.scales + e * q.s_mat + (size_t)n * q.s_row) : 1.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[mi][r] = (FACTORED ? facc[mi][r] : acc[mi][r]) * rs;
     }
+    if (SPLIT) {
+        // the up wavefront hands its four values per lane to the gate wavefront of the same weight rows
+        float4 *xch = (float4 *)(gs_lds + n_steps * kSkinnyTileM) + (wave >> 1) * 64 + lane;
+        if (proj == 1) *xch = make_float4(v[0][0], v[0][1], v[0][2], v[0][3]);
+        __syncthreads();
+        if (proj == 1) return;
+        const float4 u = *xch;
+        v[1][0] = u.x, v[1][1] = u.y, v[1][2] = u.z, v[1][3] = u.w;
+    }
+    if (!lane_on) return;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int i = 4 * h + r;
         if (i >= (int)t.nrows) continue;
-        float v[NM];
-#pragma unroll
-        for (int mi = 0; mi < NM; ++mi) v[mi] = (FACTORED ? facc[mi][r] : acc[mi][r]) * rs[mi];
         const uint32_t p = t.row0 + (uint32_t)i;
-        float val = GATE_UP ? limited_swiglu(v[0], v[NM - 1], g.swiglu_limit) : v[0];
+        float val = GATE_UP ? limited_swiglu(v[0][r], v[1][r], g.swiglu_limit) : v[0][r];
         if (g.row_scale) val *= g.row_scale[g.row_scale_idx ? g.row_scale_idx[p] : p];
         const size_t dst = g.out_rows ? g.out_rows[p] : p;
         g.out[dst * (size_t)g.ldo + n] = f32_to_bf16_bits(val);
@@ -287,10 +302,11 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArg
 static int skinny_vals(const QView &b) {
     return (b.mode == DMOE_QUANT_AFFINE && b.bits == 4) || b.mode == DMOE_QUANT_MXFP4 ? 32 : 16;
 }
-static size_t skinny_lds_bytes(const QView &b) {
+static size_t skinny_lds_bytes(const QView &b, bool gate_up = true) {
     size_t x = (size_t)kSkinnyTileM * ((size_t)b.cols * 2 + 16);
     size_t sums = (size_t)(b.cols / (2 * skinny_vals(b))) * kSkinnyTileM * sizeof(float);
-    return x + sums;
+    size_t exchange = gate_up && kSkinnySplitGateUp ? (size_t)kSkinnyWaves * 64 * sizeof(float4) : 0;
+    return x + sums + exchange;
 }
 
 bool qgemm_skinny_supports(const QView &b) {
@@ -303,13 +319,14 @@ struct SkinnyLaunch {
     template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED>
     int go() {
         auto kern = qgemm_skinny_kernel<Fmt, GATE_UP, FACTORED, PACKED>;
-        const size_t lds = skinny_lds_bytes(g.b0);
+        const size_t lds = skinny_lds_bytes(g.b0, GATE_UP);
         static thread_local size_t allowed = 0; // per instantiation: raise the dynamic LDS limit once
         if (lds > allowed) {
             DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(150 * 1024)));
             allowed = 150 * 1024;
         }
-        dim3 grid((unsigned)ceil_div(g.b0.rows, kSkinnyWaves * 32), (unsigned)g.max_tiles), block(kSkinnyWaves * 64);
+        dim3 grid((unsigned)ceil_div(g.b0.rows, kSkinnyWaves * 32), (unsigned)g.max_tiles);
+        dim3 block((GATE_UP && kSkinnySplitGateUp ? 2 : 1) * kSkinnyWaves * 64);
         hipLaunchKernelGGL(kern, grid, block, lds, st, g);
         DMOE_LAUNCH_CHECK();
         return DMOE_OK;
