@@ -55,8 +55,12 @@ struct Workspace {
     // side stream (default priority) + fork/join events for work that overlaps the main stream
     hipStream_t side = nullptr;
     hipEvent_t fork = nullptr, join = nullptr;
+    // second side stream: the two tile classes of the skinny GEMMs run side by side
+    hipStream_t side2 = nullptr;
+    hipEvent_t packed = nullptr, small_done = nullptr;
 };
-int side_stream_ready(Workspace *w); // creates the side stream and its events on first use
+int side_stream_ready(Workspace *w);  // creates the side stream and its events on first use
+int side2_stream_ready(Workspace *w); // same for the second side stream
 
 // stage timing helpers (no-ops unless enabled on the workspace)
 int stage_begin(Workspace *w, int stage, hipStream_t st);
@@ -150,13 +154,19 @@ struct GemmArgs {
     float swiglu_limit = 0.0f;
 };
 // tile_m the kernels were built for
-constexpr int kSkinnyTileM = 8;
+constexpr int kSkinnyTileM = 32;          // most rows a skinny tile can hold (see qgemm_skinny_tile_m)
+constexpr int kSkinnyDenseTileM = 8;      // dense (one matrix) launches: small tiles, many workgroups per row block
 constexpr int kMfmaTileM = 128;
 constexpr int kMfmaWideTileM = 256;
-int launch_qgemm_skinny(const GemmArgs &g, hipStream_t st);
+// The skinny path serves tiles of up to 8 rows and larger tiles with separate launches (the classes are disjoint,
+// so they may run on different streams); kSkinnyAll issues both on `st`.
+enum { kSkinnySmallTiles = 1, kSkinnyBigTiles = 2, kSkinnyAll = 3 };
+int launch_qgemm_skinny(const GemmArgs &g, hipStream_t st, int classes = kSkinnyAll);
+bool qgemm_skinny_has_big_tiles(const GemmArgs &g); // whether the kSkinnyBigTiles launch does anything
 int launch_qgemm_mfma(const GemmArgs &g, hipStream_t st); // picks the wide kernel when the format allows it
 int launch_qgemm_wide(const GemmArgs &g, hipStream_t st);
 bool qgemm_skinny_supports(const QView &b);
+int qgemm_skinny_tile_m(const QView &b);  // rows per tile to build tile lists with for the skinny path
 bool qgemm_mfma_supports(const QView &b);
 bool qgemm_wide_supports(const QView &b);
 // tile size to build tile lists with for the MFMA path of this weight matrix

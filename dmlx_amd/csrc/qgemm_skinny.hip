@@ -1,13 +1,19 @@
-// Grouped quantized GEMM, skinny path (decode): at most kSkinnyTileM rows per expert tile.
+// Grouped quantized GEMM, skinny path (decode): at most kSkinnyTileM (32) rows per expert tile.
 //
-// The step is bound by streaming every live expert's packed weights once from HBM. Each of the four
-// wavefronts of a workgroup owns 32 weight rows (per projection) and walks the whole reduction
-// dimension on its own: lane (n = lane % 32, h = lane / 32) loads the 16-byte chunk h of row n for the
-// current 64-wide step straight into registers, a ring of kSkinnyStages steps deep, so ~14 KiB per
-// wavefront are in flight while one step is consumed and the wavefronts never wait for each other.
-// The tile's activations (<= 8 rows) sit in LDS for the whole kernel and feed the A operand of
-// v_mfma_f32_32x32x16_bf16; the weights feed the B operand, so every lane's accumulators belong to ITS
-// weight row and rows 4h..4h+3 of the tile, and nothing has to be reduced across lanes.
+// The step is bound by streaming every live expert's packed weights once from HBM. Each wavefront of a
+// workgroup owns 32 weight rows of a projection and walks the whole reduction dimension on its own: lane
+// (n = lane % 32, h = lane / 32) loads the 16-byte chunk h of row n for the current 64-wide step straight into
+// registers, a ring of kSkinnyStages steps deep, so the wavefronts never wait for each other while several
+// KiB per wavefront are in flight. The tile's activations sit in LDS (put there by direct global->LDS loads,
+// requested ahead of the weight ring) and feed the A operand of v_mfma_f32_32x32x16_bf16; the weights feed the
+// B operand, so every lane's accumulators belong to ITS weight row and rows 8j+4h..8j+4h+3 of the tile, and
+// nothing has to be reduced across lanes.
+//
+// Two instances serve two classes of tiles with separate launches (a launch skips the tiles of the other
+// class). Up to 8 rows - nearly every tile at decode - the rows stay whole in LDS and a lane keeps 4
+// accumulators; gate and up rows go to separate wavefronts. 9 to 32 rows: LDS holds a quarter of every row,
+// restaged three times on the way, and a lane keeps 16 accumulators; an expert with many rows then still
+// streams its weights once instead of once per 8 rows.
 //
 // 4-bit affine weights (group >= 64) are never multiplied out. Codes become the bf16 numbers (128 + q)
 // with one AND-OR per pair; both halves of a step lie in the same scale group, so the matrix core
@@ -24,10 +30,13 @@
 namespace dmoe {
 
 constexpr int kSkinnyWaves = 4;          // 32-row blocks of weight rows per workgroup
-// gate/up launches give each projection its own wavefront (eight per workgroup, paired through LDS at the end):
-// half the registers per wavefront, twice the wavefronts per SIMD to overlap decode, matrix and memory waits
-constexpr bool kSkinnySplitGateUp = true;
+// Two instances per format. Tiles of at most one row block (the bulk at decode): gate/up launches give each
+// projection its own wavefront (eight per workgroup, paired through LDS at the end) - half the registers per
+// wavefront, twice the wavefronts per SIMD to overlap decode, matrix and memory waits. Larger tiles: four
+// wavefronts with both projections each; their extra accumulators would cost the first instance its occupancy.
+constexpr int kSkinnyBigRowBlocks = 4;   // row blocks of the big-tile instance (the other instance has one)
 constexpr int kSkinnyStages = 8;
+constexpr int kSkinnyRowBlock = 8;       // tile rows per row block: the LDS window holds 8 whole rows of activations
 
 __device__ __forceinline__ uint32_t vgpr_const32(uint32_t c) {
     uint32_t v;
@@ -58,13 +67,14 @@ struct SkinnyStage {
     uint32_t sb[NM][2];
 };
 
-template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED>
-__global__ __launch_bounds__((GATE_UP && kSkinnySplitGateUp ? 2 : 1) * kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArgs g) {
+template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED, int RJ>
+__global__ __launch_bounds__((GATE_UP && RJ == 1 ? 2 : 1) * kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArgs g) {
     using CS = ChunkStream<Fmt, PACKED>;
     constexpr int KV = Fmt::kVals;   // values per 16-byte chunk
     constexpr int KSTEP = 2 * KV;    // reduction elements per step (both lane halves)
     constexpr int NJ = KV / 8;       // MFMAs (K = 16) per step
-    constexpr bool SPLIT = GATE_UP && kSkinnySplitGateUp;
+    constexpr bool SPLIT = GATE_UP && RJ == 1;      // see kSkinnyBigRowBlocks
+    constexpr int RP = RJ * kSkinnyRowBlock;        // rows the LDS layout is made for
     constexpr int NM = GATE_UP && !SPLIT ? 2 : 1;   // projections per wavefront
     constexpr int WAVES = (SPLIT ? 2 : 1) * kSkinnyWaves;
     extern __shared__ __attribute__((aligned(16))) uint8_t skinny_lds[];
@@ -77,10 +87,10 @@ __global__ __launch_bounds__((GATE_UP && kSkinnySplitGateUp ? 2 : 1) * kSkinnyWa
         if (slot >= n_tiles) return;
     } else {
         t.expert = 0;
-        t.row0 = slot * (uint32_t)kSkinnyTileM;
+        t.row0 = slot * (uint32_t)g.tile_m;
         if ((int)t.row0 >= g.dense_rows) return;
         uint32_t left = (uint32_t)g.dense_rows - t.row0;
-        t.nrows = left < (uint32_t)kSkinnyTileM ? left : (uint32_t)kSkinnyTileM;
+        t.nrows = left < (uint32_t)g.tile_m ? left : (uint32_t)g.tile_m;
     }
     const int tid = (int)threadIdx.x, lane = tid & 63, ln = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -89,9 +99,13 @@ __global__ __launch_bounds__((GATE_UP && kSkinnySplitGateUp ? 2 : 1) * kSkinnyWa
     const size_t e = t.expert;
 
     // ---- this lane's weight row ------------------------------------------------------------------------
+    // A wavefront past the last block of weight rows repeats that block (and stores nothing): every wavefront
+    // of the workgroup then runs the same control flow, which the barriers below rely on.
     const int proj = SPLIT ? (wave & 1) : 0;        // split: even wavefronts take gate rows, odd ones up rows
-    const int col0 = ((int)blockIdx.x * kSkinnyWaves + (SPLIT ? wave >> 1 : wave)) * 32;
-    const bool wave_on = col0 < n_out;
+    const int col_raw = ((int)blockIdx.x * kSkinnyWaves + (SPLIT ? wave >> 1 : wave)) * 32;
+    const int col_last = ((n_out - 1) >> 5) << 5;
+    const int col0 = col_raw < n_out ? col_raw : col_last;
+    const bool store_on = col_raw + ln < n_out;
     int n = col0 + ln;
     if (n >= n_out) n = n_out - 1; // stay inside the matrix; such rows are never stored
     CS cs[NM];
@@ -105,52 +119,40 @@ __global__ __launch_bounds__((GATE_UP && kSkinnySplitGateUp ? 2 : 1) * kSkinnyWa
         }
     };
 
-    // ---- activations of the tile -> LDS, ahead of the weights ---------------------------------------------
-    // Loads return in issue order, so the tile's activation rows are requested first (straight into LDS, no
-    // registers), then the first stages of the weight ring; the wait below lets the ring stay in flight.
-    // Only the rows the tile has are staged (most decode tiles hold one to three): row m of the A operand only
-    // reaches accumulator row m, and accumulator rows past the tile are never stored.
-    const int pitch = cols * 2 + 16; // bytes per LDS row; +16 keeps the 8 rows on different banks
+    // ---- activations of the tile in LDS -------------------------------------------------------------------
+    // The LDS window holds 8 full rows' worth of activations. A tile of up to 8 rows (RJ = 1) keeps its rows
+    // whole; a larger one (RJ = 4, up to 32 rows) keeps a quarter of every row and is restaged at the three span
+    // boundaries, so that an expert with many rows still streams its weights only once. Only the rows the tile
+    // has are staged: row m of the A operand only reaches accumulator row m, rows past the tile are never stored.
     const int nrows = __builtin_amdgcn_readfirstlane((int)t.nrows);
+    // each launch serves one class of tiles: up to one row block, or more (workgroup-uniform: nothing has synchronized yet)
+    if (RJ == 1 ? nrows > kSkinnyRowBlock : nrows <= kSkinnyRowBlock) return;
+    const int span_steps = n_steps / RJ;             // the launcher only builds larger tiles when this divides
+    const int span_bytes = span_steps * KSTEP * 2;   // bytes of one row in one span
+    const int pitch = span_bytes + 16;               // +16 keeps neighbouring rows on different banks
     uint8_t *xs_lds = skinny_lds;
-    float *gs_lds = (float *)(skinny_lds + kSkinnyTileM * pitch); // [n_steps][8]: per-step sums of x (factored)
-    {
-        const uint32_t lds_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)skinny_lds;
-        const uint32_t row0 = __builtin_amdgcn_readfirstlane(t.row0);
-        const int row_bytes = cols * 2;
-        // source rows of the tile: one load for all of them (lane r holds row r's), then uniform reads
-        uint32_t src_of_lane = row0 + (uint32_t)(lane < nrows ? lane : 0);
-        if (g.a_rows) src_of_lane = g.a_rows[src_of_lane];
-        for (int r = 0; r < nrows; ++r) {
+    float *gs_lds = (float *)(skinny_lds + kSkinnyRowBlock * cols * 2 + kSkinnyTileM * 16); // [span_steps][rp] sums of x
+    const uint32_t lds_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)skinny_lds;
+    // source rows of the tile: one load for all of them (lane r holds row r's), then uniform reads
+    uint32_t src_of_lane = __builtin_amdgcn_readfirstlane(t.row0) + (uint32_t)(lane < nrows ? lane : 0);
+    if (g.a_rows) src_of_lane = g.a_rows[src_of_lane];
+    // requests span `span` of every row straight into LDS (no registers); completion is the caller's wait
+    auto issue_x = [&](int span) {
+        const int cpr = (span_bytes + 1023) >> 10; // 1 KiB operations per row
+        const int ops = nrows * cpr;
+        for (int o = wave; o < ops; o += WAVES) {
+            const int r = o / cpr, c = (o - r * cpr) << 10;
             const size_t src = (uint32_t)__builtin_amdgcn_readlane((int)src_of_lane, r);
-            const uint8_t *row = (const uint8_t *)(g.a + src * (size_t)cols) + lane * 16;
-            for (int c = wave * 1024; c < row_bytes; c += WAVES * 1024) {
-                const uint32_t la = lds_addr + (uint32_t)(r * pitch + c); // uniform; lane i lands at la + 16 i
-                const uint8_t *gp = row + c;
-                if (c + lane * 16 < row_bytes)
-                    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gp), "s"(la) : "memory"); // nothing else in this kernel uses M0
-            }
+            const uint8_t *gp = (const uint8_t *)(g.a + src * (size_t)cols) + (size_t)span * span_bytes + c + lane * 16;
+            const uint32_t la = lds_addr + (uint32_t)(r * pitch + c); // uniform; lane i lands at la + 16 i
+            if (c + lane * 16 < span_bytes)
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gp), "s"(la) : "memory"); // nothing else in this kernel uses M0
         }
-    }
-    SkinnyStage<NM> ring[kSkinnyStages];
-    const bool ring_full = n_steps >= kSkinnyStages - 1;
-    if (wave_on) {
-#pragma unroll
-        for (int mi = 0; mi < NM; ++mi) cs[mi].pin(); // keeps the weight loads behind the requests above
-#pragma unroll
-        for (int j = 0; j < kSkinnyStages - 1; ++j)
-            if (j < n_steps) load_stage(j, ring[j]);
-        // every ring stage holds at least NM loads younger than the activation requests
-        if (ring_full) __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt((kSkinnyStages - 1) * NM));
-        else __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt(0));
-    } else {
-        __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt(0));
-    }
-    __syncthreads();
-    if (FACTORED) {
-        // per 16-byte piece: (x0..x7) -> (x0,x4,x1,x5,x2,x6,x3,x7), the order the code pairs come out in, and the
-        // sum of each step's 64 activations (eight pieces, eight neighbouring lanes)
-        const int pieces = cols / 8;
+    };
+    // factored form: per 16-byte piece (x0..x7) -> (x0,x4,x1,x5,x2,x6,x3,x7), the order the code pairs come out
+    // in, and the sum of each step's 64 activations (eight pieces, eight neighbouring lanes)
+    auto fix_x = [&]() {
+        const int pieces = span_bytes >> 4;
         for (int idx = tid; idx < nrows * pieces; idx += WAVES * 64) {
             const int r = idx / pieces, pc = idx - r * pieces;
             uint4 *px = (uint4 *)(xs_lds + r * pitch + pc * 16);
@@ -168,145 +170,200 @@ __global__ __launch_bounds__((GATE_UP && kSkinnySplitGateUp ? 2 : 1) * kSkinnyWa
             sum += skinny_dpp<0xB1>(sum);  // lane ^ 1 (quad_perm 1,0,3,2)
             sum += skinny_dpp<0x4E>(sum);  // lane ^ 2 (quad_perm 2,3,0,1)
             sum += skinny_dpp<0x141>(sum); // the other quad of the eight lanes (row_half_mirror)
-            if ((pc & 7) == 0) gs_lds[(pc >> 3) * kSkinnyTileM + r] = sum;
+            if ((pc & 7) == 0) gs_lds[(pc >> 3) * RP + r] = sum;
         }
+    };
+
+    // Loads return in issue order: the first span is requested ahead of the first stages of the weight ring, and
+    // the wait below lets the ring stay in flight.
+    issue_x(0);
+    SkinnyStage<NM> ring[kSkinnyStages];
+#pragma unroll
+    for (int mi = 0; mi < NM; ++mi) cs[mi].pin(); // keeps the weight loads behind the requests above
+#pragma unroll
+    for (int j = 0; j < kSkinnyStages - 1; ++j)
+        if (j < n_steps) load_stage(j, ring[j]);
+    // every ring stage holds at least NM loads younger than the activation requests
+    if (n_steps >= kSkinnyStages - 1) __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt((kSkinnyStages - 1) * NM));
+    else __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt(0));
+    __syncthreads();
+    if (FACTORED) {
+        fix_x();
         __syncthreads();
     }
-    if (!wave_on) return;
 
     // A-operand source of this lane: tile row ln, reduction half h. Lanes past the tile's rows read row 0 again:
     // their operand rows only reach accumulator rows that are never stored.
     const uint8_t *xlane = xs_lds + (ln < nrows ? ln : 0) * pitch + h * KV * 2;
-
-    f32x16_t acc[NM];
-#pragma unroll
-    for (int mi = 0; mi < NM; ++mi)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[mi][r] = 0.0f;
-    float facc[NM][4];
-#pragma unroll
-    for (int mi = 0; mi < NM; ++mi)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) facc[mi][r] = 0.0f;
     const uint32_t mask = vgpr_const32(0x000f000fu), magic = vgpr_const32(0x43004300u);
 
-    // One step: decode every projection's chunk first, then issue the matrix instructions of the projections
-    // alternately (two independent accumulation chains: a dependent MFMA never follows its producer directly),
-    // then apply the scales.
-    auto consume = [&](int step, const SkinnyStage<NM> &s) {
-        bf16x8_t xf[NJ];
+    // RJ row blocks of the tile: accumulator registers 4 j + r of a lane belong to tile row 8 j + 4 h + r
+    {
+        f32x16_t acc[NM];
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            uint4 q = *(const uint4 *)(xlane + (size_t)step * KSTEP * 2 + j * 16);
-            xf[j] = __builtin_bit_cast(bf16x8_t, q);
+        for (int mi = 0; mi < NM; ++mi)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[mi][r] = 0.0f;
+        float facc[NM][4 * RJ];
+#pragma unroll
+        for (int mi = 0; mi < NM; ++mi)
+#pragma unroll
+            for (int r = 0; r < 4 * RJ; ++r) facc[mi][r] = 0.0f;
+
+        // One step: decode every projection's chunk first, then issue the matrix instructions of the projections
+        // alternately (independent accumulation chains), then apply the scales. `xs` = step within the span.
+        auto consume = [&](int xs, const SkinnyStage<NM> &s) {
+            bf16x8_t xf[NJ];
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                uint4 q = *(const uint4 *)(xlane + (size_t)xs * KSTEP * 2 + j * 16);
+                xf[j] = __builtin_bit_cast(bf16x8_t, q);
+            }
+            float4 gsum[RJ];
+            if (FACTORED) {
+#pragma unroll
+                for (int j = 0; j < RJ; ++j) gsum[j] = *(const float4 *)(gs_lds + xs * RP + 8 * j + 4 * h);
+            }
+            uint32_t wp[NM][KV / 2];
+            Meta meta[NM];
+#pragma unroll
+            for (int mi = 0; mi < NM; ++mi) {
+                meta[mi] = CS::meta(s.sb[mi]);
+                if (FACTORED) {
+                    codes_to_bf16(s.raw[mi].x, mask, magic, wp[mi]);
+                    codes_to_bf16(s.raw[mi].y, mask, magic, wp[mi] + 4);
+                    codes_to_bf16(s.raw[mi].z, mask, magic, wp[mi] + 8);
+                    codes_to_bf16(s.raw[mi].w, mask, magic, wp[mi] + 12);
+                } else {
+                    Fmt::decode_fast(s.raw[mi], meta[mi], wp[mi]);
+                }
+            }
+            f32x16_t p[NM];
+            if (FACTORED) {
+#pragma unroll
+                for (int mi = 0; mi < NM; ++mi)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) p[mi][r] = 0.0f;
+            }
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+                for (int mi = 0; mi < NM; ++mi) {
+                    uint4 q = make_uint4(wp[mi][4 * j], wp[mi][4 * j + 1], wp[mi][4 * j + 2], wp[mi][4 * j + 3]);
+                    if (FACTORED)
+                        p[mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[j], __builtin_bit_cast(bf16x8_t, q), p[mi], 0, 0, 0);
+                    else
+                        acc[mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[j], __builtin_bit_cast(bf16x8_t, q), acc[mi], 0, 0, 0);
+                }
+            }
+            if (FACTORED) {
+#pragma unroll
+                for (int mi = 0; mi < NM; ++mi) {
+                    const float boff = fmaf(-128.0f, meta[mi].s, meta[mi].b);
+#pragma unroll
+                    for (int j = 0; j < RJ; ++j) {
+                        facc[mi][4 * j + 0] = fmaf(meta[mi].s, p[mi][4 * j + 0], fmaf(boff, gsum[j].x, facc[mi][4 * j + 0]));
+                        facc[mi][4 * j + 1] = fmaf(meta[mi].s, p[mi][4 * j + 1], fmaf(boff, gsum[j].y, facc[mi][4 * j + 1]));
+                        facc[mi][4 * j + 2] = fmaf(meta[mi].s, p[mi][4 * j + 2], fmaf(boff, gsum[j].z, facc[mi][4 * j + 2]));
+                        facc[mi][4 * j + 3] = fmaf(meta[mi].s, p[mi][4 * j + 3], fmaf(boff, gsum[j].w, facc[mi][4 * j + 3]));
+                    }
+                }
+            }
+        };
+
+        // whole rounds of the ring run without guards (the look-ahead is clamped onto the last step: a few repeated
+        // loads at the very end instead of a branch per step); a partial last round runs the guarded copy
+        const int full = n_steps / kSkinnyStages * kSkinnyStages;
+        int x0 = 0, next_span = span_steps; // first step of the span in LDS, first step of the next one
+#pragma unroll 1
+        for (int s0 = 0; s0 < full; s0 += kSkinnyStages) {
+            if (RJ > 1 && s0 == next_span) {
+                // the next span of the activations replaces the one in LDS (the weight ring stays in flight; its
+                // loads are older than these requests, so the wait covers nothing that was not due anyway)
+                __syncthreads();
+                issue_x(s0 / span_steps);
+                __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt(0));
+                __syncthreads();
+                if (FACTORED) {
+                    fix_x();
+                    __syncthreads();
+                }
+                x0 = s0;
+                next_span += span_steps;
+            }
+#pragma unroll
+            for (int j = 0; j < kSkinnyStages; ++j) {
+                const int step = s0 + j, ahead = step + kSkinnyStages - 1;
+                load_stage(ahead < n_steps ? ahead : n_steps - 1, ring[(j + kSkinnyStages - 1) % kSkinnyStages]);
+                consume(step - x0, ring[j]);
+            }
         }
-        float4 gsum = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (FACTORED) gsum = *(const float4 *)(gs_lds + step * kSkinnyTileM + 4 * h);
-        uint32_t wp[NM][KV / 2];
-        Meta meta[NM];
+        if (full < n_steps) { // only tiles of one row block get here (larger ones need whole rounds per span)
+#pragma unroll
+            for (int j = 0; j < kSkinnyStages; ++j) {
+                const int step = full + j;
+                if (step + kSkinnyStages - 1 < n_steps) load_stage(step + kSkinnyStages - 1, ring[(j + kSkinnyStages - 1) % kSkinnyStages]);
+                if (step < n_steps) consume(step, ring[j]);
+            }
+        }
+
+        // ---- epilogue: this lane holds rows 8 j + 4 h + r of the tile for weight row n ----------------------
+        float v[2][4 * RJ];
 #pragma unroll
         for (int mi = 0; mi < NM; ++mi) {
-            meta[mi] = CS::meta(s.sb[mi]);
-            if (FACTORED) {
-                codes_to_bf16(s.raw[mi].x, mask, magic, wp[mi]);
-                codes_to_bf16(s.raw[mi].y, mask, magic, wp[mi] + 4);
-                codes_to_bf16(s.raw[mi].z, mask, magic, wp[mi] + 8);
-                codes_to_bf16(s.raw[mi].w, mask, magic, wp[mi] + 12);
-            } else {
-                Fmt::decode_fast(s.raw[mi], meta[mi], wp[mi]);
+            const QView &q = (mi + proj) == 0 ? g.b0 : g.b1;
+            const float rs = Fmt::kRowScale ? *(const float *)(q.scales + e * q.s_mat + (size_t)n * q.s_row) : 1.0f;
+#pragma unroll
+            for (int r = 0; r < 4 * RJ; ++r) v[mi][r] = (FACTORED ? facc[mi][r] : acc[mi][r]) * rs;
+        }
+        if (SPLIT) {
+            // the up wavefront hands its values to the gate wavefront of the same weight rows, through the
+            // activation window (free once every wavefront has left the main loop)
+            float4 *xch = (float4 *)xs_lds + ((wave >> 1) * 64 + lane) * RJ;
+            __syncthreads();
+            if (proj == 1) {
+#pragma unroll
+                for (int j = 0; j < RJ; ++j) xch[j] = make_float4(v[0][4 * j], v[0][4 * j + 1], v[0][4 * j + 2], v[0][4 * j + 3]);
+            }
+            __syncthreads();
+            if (proj == 1) return;
+#pragma unroll
+            for (int j = 0; j < RJ; ++j) {
+                const float4 u = xch[j];
+                v[1][4 * j] = u.x, v[1][4 * j + 1] = u.y, v[1][4 * j + 2] = u.z, v[1][4 * j + 3] = u.w;
             }
         }
-        f32x16_t p[NM];
-        if (FACTORED) {
+        if (!store_on) return;
 #pragma unroll
-            for (int mi = 0; mi < NM; ++mi)
+        for (int j = 0; j < RJ; ++j) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) p[mi][r] = 0.0f;
-        }
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-#pragma unroll
-            for (int mi = 0; mi < NM; ++mi) {
-                uint4 q = make_uint4(wp[mi][4 * j], wp[mi][4 * j + 1], wp[mi][4 * j + 2], wp[mi][4 * j + 3]);
-                if (FACTORED)
-                    p[mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[j], __builtin_bit_cast(bf16x8_t, q), p[mi], 0, 0, 0);
-                else
-                    acc[mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[j], __builtin_bit_cast(bf16x8_t, q), acc[mi], 0, 0, 0);
+            for (int r = 0; r < 4; ++r) {
+                const int i = 8 * j + 4 * h + r;
+                if (i >= nrows) continue;
+                const uint32_t p = t.row0 + (uint32_t)i;
+                float val = GATE_UP ? limited_swiglu(v[0][4 * j + r], v[1][4 * j + r], g.swiglu_limit) : v[0][4 * j + r];
+                if (g.row_scale) val *= g.row_scale[g.row_scale_idx ? g.row_scale_idx[p] : p];
+                const size_t dst = g.out_rows ? g.out_rows[p] : p;
+                g.out[dst * (size_t)g.ldo + n] = f32_to_bf16_bits(val);
             }
         }
-        if (FACTORED) {
-#pragma unroll
-            for (int mi = 0; mi < NM; ++mi) {
-                const float boff = fmaf(-128.0f, meta[mi].s, meta[mi].b);
-                facc[mi][0] = fmaf(meta[mi].s, p[mi][0], fmaf(boff, gsum.x, facc[mi][0]));
-                facc[mi][1] = fmaf(meta[mi].s, p[mi][1], fmaf(boff, gsum.y, facc[mi][1]));
-                facc[mi][2] = fmaf(meta[mi].s, p[mi][2], fmaf(boff, gsum.z, facc[mi][2]));
-                facc[mi][3] = fmaf(meta[mi].s, p[mi][3], fmaf(boff, gsum.w, facc[mi][3]));
-            }
-        }
-    };
-
-    // whole rounds of the ring run without guards (the look-ahead is clamped onto the last step: a few repeated
-    // loads at the very end instead of a branch per step); a partial last round runs the guarded copy
-    const int full = n_steps / kSkinnyStages * kSkinnyStages;
-#pragma unroll 1
-    for (int s0 = 0; s0 < full; s0 += kSkinnyStages) {
-#pragma unroll
-        for (int j = 0; j < kSkinnyStages; ++j) {
-            const int step = s0 + j, ahead = step + kSkinnyStages - 1;
-            load_stage(ahead < n_steps ? ahead : n_steps - 1, ring[(j + kSkinnyStages - 1) % kSkinnyStages]);
-            consume(step, ring[j]);
-        }
-    }
-    if (full < n_steps) {
-#pragma unroll
-        for (int j = 0; j < kSkinnyStages; ++j) {
-            const int step = full + j;
-            if (step + kSkinnyStages - 1 < n_steps) load_stage(step + kSkinnyStages - 1, ring[(j + kSkinnyStages - 1) % kSkinnyStages]);
-            if (step < n_steps) consume(step, ring[j]);
-        }
-    }
-
-    // ---- epilogue: this lane holds rows 4h..4h+3 of the tile for weight row n --------------------------
-    const bool lane_on = col0 + ln < n_out;
-    float v[2][4];
-#pragma unroll
-    for (int mi = 0; mi < NM; ++mi) {
-        const QView &q = (mi + proj) == 0 ? g.b0 : g.b1;
-        const float rs = Fmt::kRowScale ? *(const float *)(q.scales + e * q.s_mat + (size_t)n * q.s_row) : 1.0f;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) v[mi][r] = (FACTORED ? facc[mi][r] : acc[mi][r]) * rs;
-    }
-    if (SPLIT) {
-        // the up wavefront hands its four values per lane to the gate wavefront of the same weight rows
-        float4 *xch = (float4 *)(gs_lds + n_steps * kSkinnyTileM) + (wave >> 1) * 64 + lane;
-        if (proj == 1) *xch = make_float4(v[0][0], v[0][1], v[0][2], v[0][3]);
-        __syncthreads();
-        if (proj == 1) return;
-        const float4 u = *xch;
-        v[1][0] = u.x, v[1][1] = u.y, v[1][2] = u.z, v[1][3] = u.w;
-    }
-    if (!lane_on) return;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int i = 4 * h + r;
-        if (i >= (int)t.nrows) continue;
-        const uint32_t p = t.row0 + (uint32_t)i;
-        float val = GATE_UP ? limited_swiglu(v[0][r], v[1][r], g.swiglu_limit) : v[0][r];
-        if (g.row_scale) val *= g.row_scale[g.row_scale_idx ? g.row_scale_idx[p] : p];
-        const size_t dst = g.out_rows ? g.out_rows[p] : p;
-        g.out[dst * (size_t)g.ldo + n] = f32_to_bf16_bits(val);
     }
 }
 
 static int skinny_vals(const QView &b) {
     return (b.mode == DMOE_QUANT_AFFINE && b.bits == 4) || b.mode == DMOE_QUANT_MXFP4 ? 32 : 16;
 }
-static size_t skinny_lds_bytes(const QView &b, bool gate_up = true) {
-    size_t x = (size_t)kSkinnyTileM * ((size_t)b.cols * 2 + 16);
-    size_t sums = (size_t)(b.cols / (2 * skinny_vals(b))) * kSkinnyTileM * sizeof(float);
-    size_t exchange = gate_up && kSkinnySplitGateUp ? (size_t)kSkinnyWaves * 64 * sizeof(float4) : 0;
-    return x + sums + exchange;
+static size_t skinny_lds_bytes(const QView &b) {
+    size_t x = (size_t)kSkinnyRowBlock * (size_t)b.cols * 2 + (size_t)kSkinnyTileM * 16;
+    size_t sums = (size_t)(b.cols / (2 * skinny_vals(b))) * kSkinnyRowBlock * sizeof(float);
+    return x + sums;
+}
+
+// Rows per tile to build tile lists with for this weight shape: the big-tile instance splits the reduction into
+// kSkinnyBigRowBlocks spans, each a whole number of ring rounds.
+int qgemm_skinny_tile_m(const QView &b) {
+    const int n_steps = b.cols / (2 * skinny_vals(b));
+    return n_steps % (kSkinnyBigRowBlocks * kSkinnyStages) == 0 ? kSkinnyBigRowBlocks * kSkinnyRowBlock : kSkinnyRowBlock;
 }
 
 bool qgemm_skinny_supports(const QView &b) {
@@ -316,19 +373,28 @@ bool qgemm_skinny_supports(const QView &b) {
 struct SkinnyLaunch {
     const GemmArgs &g;
     hipStream_t st;
-    template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED>
-    int go() {
-        auto kern = qgemm_skinny_kernel<Fmt, GATE_UP, FACTORED, PACKED>;
-        const size_t lds = skinny_lds_bytes(g.b0, GATE_UP);
+    int classes;
+    template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED, int RJ>
+    int go_class() {
+        auto kern = qgemm_skinny_kernel<Fmt, GATE_UP, FACTORED, PACKED, RJ>;
+        const size_t lds = skinny_lds_bytes(g.b0);
         static thread_local size_t allowed = 0; // per instantiation: raise the dynamic LDS limit once
         if (lds > allowed) {
             DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(150 * 1024)));
             allowed = 150 * 1024;
         }
         dim3 grid((unsigned)ceil_div(g.b0.rows, kSkinnyWaves * 32), (unsigned)g.max_tiles);
-        dim3 block((GATE_UP && kSkinnySplitGateUp ? 2 : 1) * kSkinnyWaves * 64);
+        dim3 block((GATE_UP && RJ == 1 ? 2 : 1) * kSkinnyWaves * 64);
         hipLaunchKernelGGL(kern, grid, block, lds, st, g);
         DMOE_LAUNCH_CHECK();
+        return DMOE_OK;
+    }
+    template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED>
+    int go() {
+        if (classes & kSkinnySmallTiles) DMOE_TRY((go_class<Fmt, GATE_UP, FACTORED, PACKED, 1>()));
+        // tile lists built with one row block per tile hold no larger tile
+        if ((classes & kSkinnyBigTiles) && g.tile_m > kSkinnyRowBlock)
+            DMOE_TRY((go_class<Fmt, GATE_UP, FACTORED, PACKED, kSkinnyBigRowBlocks>()));
         return DMOE_OK;
     }
     template <typename Fmt>
@@ -345,16 +411,20 @@ struct SkinnyLaunch {
     }
 };
 
-int launch_qgemm_skinny(const GemmArgs &g, hipStream_t st) {
+bool qgemm_skinny_has_big_tiles(const GemmArgs &g) { return g.tile_m > kSkinnyRowBlock; }
+
+int launch_qgemm_skinny(const GemmArgs &g, hipStream_t st, int classes) {
     DMOE_REQUIRE(qgemm_skinny_supports(g.b0), "skinny GEMM: unsupported weight shape (cols=%d)", g.b0.cols);
     DMOE_REQUIRE(g.max_tiles >= 0 && g.max_tiles <= 65535, "skinny GEMM: %d tiles exceed the grid limit", g.max_tiles);
     DMOE_REQUIRE(g.a && g.out && g.ldo > 0 && ((uintptr_t)g.a % 16) == 0, "skinny GEMM: bad pointer");
+    DMOE_REQUIRE(g.tile_m > 0 && g.tile_m <= qgemm_skinny_tile_m(g.b0), "skinny GEMM: tiles of %d rows, this shape takes %d",
+                 g.tile_m, qgemm_skinny_tile_m(g.b0));
     if (g.gate_up)
         DMOE_REQUIRE(g.b1.rows == g.b0.rows && g.b1.cols == g.b0.cols && g.b1.mode == g.b0.mode &&
                          g.b1.bits == g.b0.bits && g.b1.group == g.b0.group && g.b1.packed == g.b0.packed,
                      "skinny GEMM: gate and up projections differ in shape or format");
     if (g.max_tiles == 0) return DMOE_OK;
-    return dispatch_format(g.b0, SkinnyLaunch{g, st});
+    return dispatch_format(g.b0, SkinnyLaunch{g, st, classes});
 }
 
 } // namespace dmoe

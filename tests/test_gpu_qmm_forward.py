@@ -62,7 +62,9 @@ def test_dequantize_bit_exact(dmoe, orc, fmt):
                                                 (700, 4, 256, 512),     # MFMA path, ragged segments
                                                 (130, 1, 128, 2048),    # single expert, MFMA, partial tile
                                                 (700, 4, 256, 384),     # reduction not a multiple of the pipeline depth
-                                                (1200, 2, 192, 640)])   # 256-row tiles, idle wavefronts in the last strip
+                                                (1200, 2, 192, 640),    # 256-row tiles, idle wavefronts in the last strip
+                                                (60, 8, 256, 2048),     # small-M path, some experts above 8 rows (restaged tiles)
+                                                (30, 4, 192, 2048)])    # same, weight rows not a multiple of the workgroup's
 def test_gather_qmm_matches_oracle(dmoe, orc, ws, fmt, R, n_mats, rows, cols):
     qw = _stack(fmt, n_mats, rows, cols, 2)
     g = torch.Generator(device="cuda").manual_seed(3)
@@ -79,6 +81,20 @@ def test_gather_qmm_matches_oracle(dmoe, orc, ws, fmt, R, n_mats, rows, cols):
     got_s = dmoe.gather_qmm(x, qw, srt, ws, None, sorted_indices=True).float().cpu().numpy()
     want_s = orc.gather_qmm(bf16_bits(x), qm, to_np_u32(srt), None)
     assert max_abs_rel(got_s, want_s) < OUT_TOL
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("R", [9, 16, 17, 29, 32])
+def test_gather_qmm_one_expert_takes_every_row(dmoe, orc, ws, fmt, R):
+    """Small-M path with a single tile of 9..32 rows (activations restaged span by span) beside empty experts."""
+    n_mats, rows, cols = 4, 160, 2048
+    qw = _stack(fmt, n_mats, rows, cols, 5)
+    g = torch.Generator(device="cuda").manual_seed(R)
+    x = torch.randn((R, cols), generator=g, device="cuda").to(torch.bfloat16)
+    rhs = torch.full((R,), 2, device="cuda", dtype=torch.int32)
+    got = dmoe.gather_qmm(x, qw, rhs, ws, None).float().cpu().numpy()
+    want = orc.gather_qmm(bf16_bits(x), qmat(qw), to_np_u32(rhs), None)
+    assert max_abs_rel(got, want) < OUT_TOL, (fmt, R, max_abs_rel(got, want))
 
 
 def _route(dmoe, orc, wl):
