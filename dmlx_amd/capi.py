@@ -70,7 +70,7 @@ EXPORTS = [
     "dmoe_layer_create", "dmoe_layer_destroy", "dmoe_moe_forward",
     "dmoe_switch_glu_forward_no_scores", "dmoe_moe_layer_forward", "dmoe_debug_last_activations",
     "dmoe_gate_create", "dmoe_gate_destroy", "dmoe_gate_forward",
-    "dmoe_layer_create_from_safetensors", "dmoe_layer_dims", "dmoe_batch_build",
+    "dmoe_layer_create_from_safetensors", "dmoe_layer_dims", "dmoe_batch_build", "dmoe_block_post",
 ]
 
 _lib = None
@@ -277,6 +277,18 @@ def batch_build(tokens, seq_lens, base_pos, ws, want_mask=True):
     check(lib().dmoe_batch_build(_ptr(d_tok), _ptr(d_pos), _ptr(d_mask), _ptr(d_req), h_tok, h_len, h_base, n, T,
                                  ws.h, _stream()))
     return d_tok, d_pos, d_mask, d_req
+
+
+def block_post(ffn_out, residual, post_mix=None, comb_mix=None):
+    """dmoe_block_post: residual add (no mixes; residual [T,D]) or mhcPost (residual [T,m,D], post_mix [T,m] or
+    [T,m,1], comb_mix [T,m,m])"""
+    T, D = ffn_out.shape
+    m = 0 if post_mix is None else residual.shape[1]
+    out = torch.empty_like(residual)
+    pm = None if post_mix is None else post_mix.reshape(T, m).contiguous()
+    cm = None if comb_mix is None else comb_mix.reshape(T, m, m).contiguous()
+    check(lib().dmoe_block_post(_ptr(out), _ptr(ffn_out), _ptr(residual), _ptr(pm), _ptr(cm), T, D, m, _stream()))
+    return out
 
 
 class Gate:

@@ -532,4 +532,36 @@ inline DeviceBatch buildOnDevice(const Context &ctx, const std::vector<const Req
 }
 } // namespace batch_builder
 
+// ---- the step after the layer (deepseek_v4.zig:2450-2499, 2652-2654, 2674) ---------------------------------
+// mhcPost(x, residual, post_mix, comb_mix): x [T,H] bf16, residual [T,hc_mult,H] bf16, post_mix [T,hc_mult(,1)]
+// f32, comb_mix [T,hc_mult,hc_mult] f32 -> [T,hc_mult,H] in x's dtype.
+inline Array mhcPost(const Context &ctx, const Array &x, const Array &residual, const Array &post_mix,
+                     const Array &comb_mix) {
+    if (x.dtype() != DType::bfloat16 || residual.dtype() != DType::bfloat16)
+        throw Error(DMOE_ERR_INVALID, "mhcPost: x and residual must be bfloat16");
+    if (post_mix.dtype() != DType::float32 || comb_mix.dtype() != DType::float32)
+        throw Error(DMOE_ERR_INVALID, "mhcPost: mixes must be float32");
+    const std::vector<int> &xs = x.shape(), &rs = residual.shape();
+    if (xs.size() != 2 || rs.size() != 3 || rs[0] != xs[0] || rs[2] != xs[1])
+        throw Error(DMOE_ERR_INVALID, "mhcPost: x [T,H] and residual [T,hc_mult,H] do not match");
+    const int T = xs[0], H = xs[1], m = rs[1];
+    if (post_mix.size() != (size_t)T * m || comb_mix.size() != (size_t)T * m * m)
+        throw Error(DMOE_ERR_INVALID, "mhcPost: post_mix must hold T*hc_mult values, comb_mix T*hc_mult*hc_mult");
+    Array out(ctx, DType::bfloat16, {T, m, H});
+    check(dmoe_block_post((uint16_t *)out.data(), (const uint16_t *)x.data(), (const uint16_t *)residual.data(),
+                          (const float *)post_mix.data(), (const float *)comb_mix.data(), T, H, m, ctx.stream()));
+    return out;
+}
+// the standard residual connection of the block (mHC disabled): after_attn + ffn_out
+inline Array residualAdd(const Context &ctx, const Array &residual, const Array &ffn_out) {
+    if (ffn_out.dtype() != DType::bfloat16 || residual.dtype() != DType::bfloat16)
+        throw Error(DMOE_ERR_INVALID, "residualAdd: bfloat16 only");
+    const std::vector<int> &xs = ffn_out.shape();
+    if (xs.size() != 2 || residual.shape() != xs) throw Error(DMOE_ERR_INVALID, "residualAdd: shapes differ");
+    Array out(ctx, DType::bfloat16, {xs[0], xs[1]});
+    check(dmoe_block_post((uint16_t *)out.data(), (const uint16_t *)ffn_out.data(), (const uint16_t *)residual.data(), nullptr,
+                          nullptr, xs[0], xs[1], 0, ctx.stream()));
+    return out;
+}
+
 } // namespace dmoe

@@ -184,6 +184,12 @@ pub fn batchBuild(ctx: Context, tokens: []const u32, seq_lens: []const i32, base
     try check(c.dmoe_batch_build(@ptrCast(@alignCast(out_tokens.ptr)), @ptrCast(@alignCast(out_positions.ptr)), if (out_mask) |m| @ptrCast(@alignCast(m.ptr)) else null, null, tokens.ptr, seq_lens.ptr, base_pos.ptr, @intCast(seq_lens.len), @intCast(tokens.len), ctx.ws, ctx.stream));
 }
 
+/// DSV4HyperConn.post / mhcPost (src/models/deepseek_v4.zig:2450-2499) when `hc_mult` > 0, the plain residual add
+/// of the block (:2674) when it is 0 (mixes null).
+pub fn blockPost(ctx: Context, out: DeviceArray(u16), ffn_out: DeviceArray(u16), residual: DeviceArray(u16), post_mix: ?DeviceArray(f32), comb_mix: ?DeviceArray(f32), n_tokens: usize, dim: usize, hc_mult: usize) Error!void {
+    try check(c.dmoe_block_post(@ptrCast(@alignCast(out.ptr)), @ptrCast(@alignCast(ffn_out.ptr)), @ptrCast(@alignCast(residual.ptr)), if (post_mix) |p| @ptrCast(@alignCast(p.ptr)) else null, if (comb_mix) |p| @ptrCast(@alignCast(p.ptr)) else null, @intCast(n_tokens), @intCast(dim), @intCast(hc_mult), ctx.stream));
+}
+
 /// One-time resident upload of a layer's experts from MLX-format safetensors shards (what
 /// model_registry.zig:255-329 prepares for on-demand reads). `paths` are NUL-terminated.
 pub fn layerFromSafetensors(ctx: Context, paths: []const [*:0]const u8, layer_idx: usize, top_k: usize, mode: [*:0]const u8, group_size: i32, bits: i32, swiglu_limit: f32, smelt_mask: ?[]const u8) Error!c.dmoe_layer {

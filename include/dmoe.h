@@ -309,6 +309,19 @@ int dmoe_gate_destroy(dmoe_gate gate);
 int dmoe_gate_forward(uint32_t *d_out_indices, float *d_out_weights, float *d_out_scores, dmoe_gate gate,
                       const uint16_t *d_x, const uint32_t *d_input_ids, int T, dmoe_workspace ws, dmoe_stream s);
 
+/* ---- the step after the layer ------------------------------------------------------------------ */
+
+/* What DSV4TransformerBlock.forward does with the layer's output (deepseek_v4.zig:2652-2654, 2674).
+ *   hc_mult == 0: ops.add(after_attn, ffn_out) (:2674): d_out bf16 [T,D] = d_residual [T,D] + d_ffn_out [T,D];
+ *                 the mixes are ignored (may be null).
+ *   hc_mult  > 0: DSV4HyperConn.post = mhcPost (:2450-2499, :2585-2588): d_residual and d_out are bf16
+ *                 [T,hc_mult,D], d_post_mix f32 [T,hc_mult] (the reference's [B,S,hc_mult,1]), d_comb_mix f32
+ *                 [T,hc_mult,hc_mult]; out[t,i,:] = x[t,:] * post_mix[t,i] + sum_j comb_mix[t,j,i] * residual[t,j,:]
+ *                 in f32 (terms in ascending j, fused multiply-adds), rounded once to bf16. hc_mult <= 8.
+ * d_out may alias d_residual only when hc_mult == 0. Pointers 16-byte aligned, D a multiple of 8. */
+int dmoe_block_post(uint16_t *d_out, const uint16_t *d_ffn_out, const uint16_t *d_residual,
+                    const float *d_post_mix, const float *d_comb_mix, int T, int D, int hc_mult, dmoe_stream s);
+
 /* ---- continuous-batch assembly ---------------------------------------------------------------- */
 
 /* batch_builder.build (batch_builder.zig:90-214) with the per-token work on the device. The caller walks its

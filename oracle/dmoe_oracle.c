@@ -305,6 +305,35 @@ void orc_gate_hash_route(const float *scores, const int32_t *tid2eid, const uint
     }
 }
 
+/* The step after the MoE layer in DSV4TransformerBlock.forward (deepseek_v4.zig:2652-2654, 2674).
+ * hc_mult == 0: ops.add(after_attn, ffn_out) (:2674), bf16 + bf16 rounded once.
+ * hc_mult  > 0: mhcPost (:2450-2499): everything widened to f32 (:2468-2473),
+ *   out[t,i,:] = x[t,:] * post_mix[t,i] + sum_j comb[t,j,i] * residual[t,j,:]   (comb transposed, :2481-2490)
+ *   rounded to the dtype of x (:2498). The f32 matmul's accumulation order is MLX's and unknown (u8): this
+ *   restatement takes j ascending, one fused multiply-add per term starting from comb[t,0,i] * residual[t,0,:],
+ *   then adds term1 = x * post_mix with one rounding. Parity unpinned vs MLX in the last f32 bit only. */
+void orc_block_post(const uint16_t *x, const uint16_t *residual, const float *post_mix, const float *comb_mix,
+                    int T, int D, int hc_mult, uint16_t *out) {
+    if (hc_mult == 0) {
+        for (size_t i = 0; i < (size_t)T * D; i++)
+            out[i] = orc_f32_to_bf16(orc_bf16_to_f32(residual[i]) + orc_bf16_to_f32(x[i]));
+        return;
+    }
+    const int m = hc_mult;
+    for (int t = 0; t < T; t++)
+        for (int i = 0; i < m; i++) {
+            const float post = post_mix[(size_t)t * m + i];
+            for (int d = 0; d < D; d++) {
+                const uint16_t *res = residual + (size_t)t * m * D + d;
+                float term2 = comb_mix[((size_t)t * m + 0) * m + i] * orc_bf16_to_f32(res[0]);
+                for (int j = 1; j < m; j++)
+                    term2 = fmaf(comb_mix[((size_t)t * m + j) * m + i], orc_bf16_to_f32(res[(size_t)j * D]), term2);
+                const float term1 = orc_bf16_to_f32(x[(size_t)t * D + d]) * post;
+                out[((size_t)t * m + i) * D + d] = orc_f32_to_bf16(term1 + term2);
+            }
+        }
+}
+
 /* mlx_take(remap, indices) then astype(u32): deepseek_v4.zig:1035-1039,
  * expert_preload.zig:200-206, expert_stream.zig:522-529 (host loop) */
 void orc_remap(const int32_t *remap, const uint32_t *idx, size_t n, uint32_t *out) {

@@ -26,6 +26,8 @@
  *        one order and one explicit polynomial exp / log (stated at their
  *        definitions) so that a GPU implementation of the same arithmetic can be
  *        compared bit for bit; against libm they agree to a few ulp (tests).
+ *   (u8) the f32 matmul inside mhcPost sums its hc_mult terms in MLX's order, unknown;
+ *        orc_block_post takes them in ascending order with fused multiply-adds.
  * Functions whose results depend on one of (u1), (u3)..(u6) are marked
  * "parity unpinned vs MLX" at their definition.
  *
@@ -78,6 +80,11 @@ void orc_gate_route(const float *scores, const float *bias, const uint8_t *resid
                     uint32_t *idx_out, float *w_out);
 /* hash layers, deepseek_v4.zig:619-636 + :655-678: indices = tid2eid[input_ids], weights from the
  * unbiased scores, renorm when not softmax, * route_scale */
+/* residual add / mhcPost after the layer (deepseek_v4.zig:2450-2499, 2652-2654, 2674); x bf16 [T,D];
+ * hc_mult == 0: residual, out bf16 [T,D]; else residual, out bf16 [T,hc_mult,D], post_mix f32 [T,hc_mult],
+ * comb_mix f32 [T,hc_mult,hc_mult] */
+void orc_block_post(const uint16_t *x, const uint16_t *residual, const float *post_mix, const float *comb_mix,
+                    int T, int D, int hc_mult, uint16_t *out);
 void orc_gate_hash_route(const float *scores, const int32_t *tid2eid, const uint32_t *ids, int T, int E,
                          int K, int renorm, float route_scale, uint32_t *idx_out, float *w_out);
 /* mlx_take(remap, indices): deepseek_v4.zig:1037, expert_preload.zig:202 */

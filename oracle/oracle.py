@@ -45,7 +45,8 @@ _lib = None
 def lib():
     global _lib
     if _lib is None:
-        if not os.path.exists(_LIB_PATH):
+        srcs = [os.path.join(os.path.dirname(os.path.abspath(__file__)), f) for f in ("dmoe_oracle.c", "dmoe_oracle.h")]
+        if not os.path.exists(_LIB_PATH) or any(os.path.getmtime(f) > os.path.getmtime(_LIB_PATH) for f in srcs):
             build()
         _lib = C.CDLL(_LIB_PATH)
         _lib.orc_dequant_value.restype = C.c_float
@@ -175,6 +176,19 @@ def gate_hash_route(scores, tid2eid, ids, renorm, route_scale):
     w = np.empty((T, K), np.float32)
     lib().orc_gate_hash_route(_p(s), _p(t2e), _p(i), T, E, K, int(renorm), C.c_float(route_scale), _p(idx), _p(w))
     return idx, w
+
+
+def block_post(x_bits, residual_bits, post_mix=None, comb_mix=None):
+    """residual add (no mixes) or mhcPost; bf16 bit patterns in and out"""
+    x = _c(x_bits, np.uint16)
+    r = _c(residual_bits, np.uint16)
+    T, D = x.shape
+    m = 0 if post_mix is None else r.shape[1]
+    out = np.empty_like(r)
+    pm = None if post_mix is None else _c(post_mix, np.float32).reshape(T, m)
+    cm = None if comb_mix is None else _c(comb_mix, np.float32).reshape(T, m, m)
+    lib().orc_block_post(_p(x), _p(r), _p(pm), _p(cm), T, D, m, _p(out))
+    return out
 
 
 def remap(remap_table, idx):

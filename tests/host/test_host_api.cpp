@@ -272,6 +272,35 @@ static void test_gate_from_hidden(Context &ctx) {
     EXPECT(threw);
 }
 
+// mhcPost on values exact in bf16: out[t,i,:] = x * post[i] + sum_j comb[j][i] * residual[j]
+static void test_block_post(Context &ctx) {
+    const int T = 2, H = 16, M = 2;
+    std::vector<uint16_t> x((size_t)T * H), res((size_t)T * M * H);
+    for (int t = 0; t < T; ++t)
+        for (int d = 0; d < H; ++d) {
+            x[(size_t)t * H + d] = bf16((float)(d + 1));
+            for (int j = 0; j < M; ++j) res[((size_t)t * M + j) * H + d] = bf16((float)(j + 1) * (t + 1));
+        }
+    const std::vector<float> post = {0.5f, 2.0f, 1.0f, 0.25f};                      // [T,M]
+    const std::vector<float> comb = {1.0f, 0.5f, 0.25f, 2.0f, 0.0f, 1.0f, 1.0f, 0.0f}; // [T,M,M]
+    Array out = mhcPost(ctx, Array::fromData(ctx, x.data(), {T, H}, DType::bfloat16),
+                        Array::fromData(ctx, res.data(), {T, M, H}, DType::bfloat16),
+                        Array::fromData(ctx, post.data(), {T, M, 1}, DType::float32),
+                        Array::fromData(ctx, comb.data(), {T, M, M}, DType::float32));
+    auto o = out.dataSlice<uint16_t>();
+    for (int t = 0; t < T; ++t)
+        for (int i = 0; i < M; ++i)
+            for (int d = 0; d < H; ++d) {
+                float want = (float)(d + 1) * post[(size_t)t * M + i];
+                for (int j = 0; j < M; ++j) want += comb[((size_t)t * M + j) * M + i] * (float)(j + 1) * (t + 1);
+                EXPECT(o[((size_t)t * M + i) * H + d] == bf16(want));
+            }
+    Array sum = residualAdd(ctx, Array::fromData(ctx, x.data(), {T, H}, DType::bfloat16),
+                            Array::fromData(ctx, x.data(), {T, H}, DType::bfloat16));
+    auto sv = sum.dataSlice<uint16_t>();
+    for (int d = 0; d < H; ++d) EXPECT(sv[d] == bf16(2.0f * (d + 1)));
+}
+
 int main() {
     try {
         Context ctx(0);
@@ -281,6 +310,7 @@ int main() {
         test_remap_smelt_batch(ctx);
         test_layer_closed_form(ctx);
         test_gate_from_hidden(ctx);
+        test_block_post(ctx);
         ctx.synchronize();
     } catch (const Error &e) {
         std::printf("dmoe::Error %d: %s\n", e.code, e.what());

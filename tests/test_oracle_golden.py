@@ -451,3 +451,39 @@ def test_hash_route_is_a_table_lookup_with_renormalised_scores(orc):
     np.testing.assert_allclose(w.sum(1), 1.5, rtol=1e-6)
     _, w_raw = orc.gate_hash_route(scores, t2e, ids, False, 1.0)
     np.testing.assert_array_equal(w_raw, np.take_along_axis(scores, t2e[ids].astype(np.int64), 1))
+
+
+def _bf16(a):
+    return torch.from_numpy(np.asarray(a, np.float32)).to(torch.bfloat16)
+
+
+def test_block_post_matches_float64_einsum_and_hand_values(orc):
+    """mhcPost (deepseek_v4.zig:2450-2499): comb is used TRANSPOSED and post_mix multiplies the layer output, not
+    the residual. Hand values that a swapped index or operand would miss, then a float64 einsum on random data."""
+    from tests.helpers import bf16_bits
+    # T=1, D=8, two streams; comb = [[1, 2], [4, 8]]: out_0 = 1*r0 + 4*r1, out_1 = 2*r0 + 8*r1 (plus x * post)
+    x = _bf16(np.full((1, 8), 2.0))
+    res = _bf16(np.stack([np.full(8, 1.0), np.full(8, 3.0)])[None])
+    post = np.array([[0.5, 4.0]], np.float32)
+    comb = np.array([[[1.0, 2.0], [4.0, 8.0]]], np.float32)
+    out = orc.block_post(bf16_bits(x), bf16_bits(res), post, comb)
+    got = torch.from_numpy(out.view(np.int16)).view(torch.bfloat16).float().numpy()
+    np.testing.assert_array_equal(got[0, 0], np.full(8, 2.0 * 0.5 + 1.0 + 12.0))
+    np.testing.assert_array_equal(got[0, 1], np.full(8, 2.0 * 4.0 + 2.0 + 24.0))
+    # random data against float64
+    rng = np.random.default_rng(11)
+    T, D, m = 9, 64, 4
+    x = _bf16(rng.standard_normal((T, D)))
+    res = _bf16(rng.standard_normal((T, m, D)) * 3)
+    post = rng.random((T, m)).astype(np.float32) * 2
+    comb = rng.random((T, m, m)).astype(np.float32)
+    out = orc.block_post(bf16_bits(x), bf16_bits(res), post, comb)
+    got = torch.from_numpy(out.view(np.int16)).view(torch.bfloat16).float().numpy()
+    x64, r64 = x.double().numpy(), res.double().numpy()
+    want = x64[:, None, :] * post.astype(np.float64)[:, :, None] + np.einsum("tji,tjd->tid", comb.astype(np.float64), r64)
+    assert np.max(np.abs(got - want) / (np.abs(want) + 1.0)) < 2 ** -8   # one bf16 rounding
+    # residual add: exactly the correctly rounded sum
+    a, b = _bf16(rng.standard_normal((5, 16))), _bf16(rng.standard_normal((5, 16)))
+    out = orc.block_post(bf16_bits(a), bf16_bits(b))
+    want = (a.float() + b.float()).to(torch.bfloat16)
+    np.testing.assert_array_equal(out, bf16_bits(want))
