@@ -153,6 +153,13 @@ constexpr int kSharedSkinnyRows = 64;
 static bool use_small_path(size_t rows, int n_experts, const QView &b) {
     return qgemm_skinny_supports(b) && rows <= (size_t)kSkinnyAvgRows * (size_t)n_experts;
 }
+// Rows per tile on the small path. Tiles above 8 rows take a second launch on a second stream (and a join),
+// which pays once a fair share of the experts holds that many rows: from an average of kSkinnyBigTileAvgRows
+// rows per expert on. Below that nearly every tile has a few rows, and 8-row tiles in one launch are as fast.
+constexpr int kSkinnyBigTileAvgRows = 3;
+static int small_path_tile_m(size_t rows, int n_experts, int shape_tile_m) {
+    return rows >= (size_t)kSkinnyBigTileAvgRows * (size_t)n_experts ? shape_tile_m : std::min(shape_tile_m, kSkinnyDenseTileM);
+}
 
 struct FwdLayout {
     size_t slot_idx, order, inv, token, sorted_e, counts, offsets, live, n_live, tiles, n_tiles, scratch;
@@ -167,7 +174,7 @@ static FwdLayout forward_layout(const Layer *L, int T) {
     size_t n = (size_t)T * L->K;
     f.small = use_small_path(n, L->E, L->gate.view) && qgemm_skinny_supports(L->down.view);
     // one tile list serves both GEMMs: the smaller of their tile sizes
-    f.tile_m = f.small ? std::min(qgemm_skinny_tile_m(L->gate.view), qgemm_skinny_tile_m(L->down.view))
+    f.tile_m = f.small ? small_path_tile_m(n, L->E, std::min(qgemm_skinny_tile_m(L->gate.view), qgemm_skinny_tile_m(L->down.view)))
                        : std::min(qgemm_mfma_tile_m(L->gate.view), qgemm_mfma_tile_m(L->down.view));
     f.max_tiles = pack_max_tiles(n, L->E, f.tile_m);
     f.slot_idx = b.take(n * 4);
@@ -513,7 +520,7 @@ int dmoe_gather_qmm(uint16_t *d_out, const uint16_t *d_x, const dmoe_qweight *qw
     hipStream_t st = to_hip(s);
     const bool small = use_small_path((size_t)R, v.n_mats, v);
     DMOE_REQUIRE(small || qgemm_mfma_supports(v), "gather_qmm: unsupported weight shape rows=%d cols=%d", v.rows, v.cols);
-    const int tile_m = small ? qgemm_skinny_tile_m(v) : qgemm_mfma_tile_m(v);
+    const int tile_m = small ? small_path_tile_m((size_t)R, v.n_mats, qgemm_skinny_tile_m(v)) : qgemm_mfma_tile_m(v);
     const int max_tiles = pack_max_tiles((size_t)R, v.n_mats, tile_m);
     Bump b;
     size_t o_order = b.take((size_t)R * 4), o_arows = b.take((size_t)R * 4);
