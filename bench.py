@@ -27,7 +27,7 @@ COPY_PROBE_BYTES = 256 << 20  # --copy-probe: bytes read (and written) by each c
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
 # (scaled by the same counters' reading for the --copy-probe copies; profiles/hbm_traffic_gemm_kernels.txt).
 # A counter cannot be read from inside the timed run, so these are the recorded values for the default workloads.
-MEASURED_TRAFFIC = {(1, "gate_up"): 1052284000, (1, "down"): 529434000,
+MEASURED_TRAFFIC = {(1, "gate_up"): 1051430000, (1, "down"): 538685000,
                     (3, "gate_up"): 5182157000, (3, "down"): 2804555000}
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
@@ -160,7 +160,7 @@ def main():
     gate_up_w = (wl.gate.nbytes() + wl.up.nbytes()) // wl.E
     down_w = wl.down.nbytes() // wl.E
     kern = "gate_up" if stages["gate_up"] >= stages["down"] else "down"
-    decode = rows <= 4 * wl.E
+    decode = rows <= 8 * wl.E   # the library's own rule for the small-M path (8 rows per resident expert on average)
     if kern == "gate_up":
         k_bytes = U * gate_up_w + wl.T * wl.D * 2 + rows * wl.F * 2
         k_flops = 2.0 * rows * 2 * wl.D * wl.F
