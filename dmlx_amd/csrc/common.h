@@ -56,6 +56,7 @@ struct Workspace {
     hipStream_t side = nullptr;
     hipEvent_t fork = nullptr, join = nullptr;
     // second side stream: the two tile classes of the skinny GEMMs run side by side
+    bool last_with_shared = true; // layout of the last forward on this workspace (for dmoe_debug_last_activations)
     hipStream_t side2 = nullptr;
     hipEvent_t packed = nullptr, small_done = nullptr;
 };
@@ -92,14 +93,19 @@ struct Tile {
     uint32_t expert;
     uint32_t row0;
     uint32_t nrows;
-    uint32_t pad;
+    uint32_t flags; // kTileDense: rows of the always-on expert folded into a routed launch
 };
+constexpr uint32_t kTileDense = 1u;
 
 struct PackOut {
     uint32_t *order = nullptr, *inv = nullptr, *token = nullptr, *sorted_e = nullptr;
     uint32_t *counts = nullptr, *offsets = nullptr, *live = nullptr, *n_live = nullptr;
-    Tile *tiles = nullptr;       // capacity pack_max_tiles(n, E, tile_m)
+    Tile *tiles = nullptr;       // capacity pack_max_tiles(n, E, tile_m) (+ the dense tiles below)
     uint32_t *n_tiles = nullptr; // device scalar
+    // Optional always-on expert folded into the same tile list: `dense_rows` extra sorted rows n .. n+dense_rows-1
+    // (row n+t = token t) of matrix `dense_expert`, cut into tiles of kSkinnyDenseTileM rows that come FIRST in the
+    // list, flagged kTileDense. order / token / sorted_e then hold n + dense_rows entries.
+    uint32_t dense_rows = 0, dense_expert = 0;
 };
 
 inline int pack_max_tiles(size_t n, int E, int tile_m) {
@@ -152,6 +158,8 @@ struct GemmArgs {
     int tile_m = 0;               // rows per tile the tile list (or the dense split) was built with
     int dense_rows = 0;
     float swiglu_limit = 0.0f;
+    float swiglu_limit_dense = 0.0f;    // the limit for tiles flagged kTileDense
+    uint32_t row_scale_rows = 0xffffffffu; // row_scale applies to sorted rows below this
 };
 // tile_m the kernels were built for
 constexpr int kSkinnyTileM = 32;          // most rows a skinny tile can hold (see qgemm_skinny_tile_m)

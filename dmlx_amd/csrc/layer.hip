@@ -20,6 +20,9 @@ struct Layer {
     int D = 0, F = 0, K = 0, E = 0, Fs = 0;
     QOwned gate, up, down, sgate, sup, sdown;
     bool has_shared = false;
+    // the shared expert's packed weights also sit behind the routed experts' as matrix E of the same buffers: at
+    // decode sizes it then rides in the routed launches as an always-on expert (no side stream, no fork / join)
+    bool shared_folded = false;
     float swiglu_limit = 0.0f, shared_swiglu_limit = 0.0f;
     bool score_before_down = false;
     int32_t *remap = nullptr; // device
@@ -45,7 +48,8 @@ static void free_layer(Layer *L) {
     delete L;
 }
 
-static int adopt(QOwned *dst, const dmoe_qweight *src, int source, const char *name, hipStream_t st) {
+// `spare_mats`: room for that many more matrices behind the stack in the packed buffers
+static int adopt(QOwned *dst, const dmoe_qweight *src, int source, const char *name, hipStream_t st, int spare_mats = 0) {
     dst->q = *src;
     if (source != DMOE_WEIGHTS_BORROW_DEVICE) {
         DMOE_REQUIRE(src->w && src->scales, "%s: weight / scales pointer is null", name);
@@ -71,8 +75,9 @@ static int adopt(QOwned *dst, const dmoe_qweight *src, int source, const char *n
     if (!can_pack(dst->view)) return DMOE_OK; // odd shapes stay in the MLX layout (slower addressing, same results)
     // resident layout: re-order once so that every wavefront streams its 32 weight rows linearly
     const size_t wb = packed_w_bytes(dst->view), mb = packed_meta_bytes(dst->view);
-    DMOE_HIP(hipMalloc(&dst->own[3], wb));
-    if (mb) DMOE_HIP(hipMalloc(&dst->own[4], mb));
+    const size_t n_mats = (size_t)dst->view.n_mats;
+    DMOE_HIP(hipMalloc(&dst->own[3], wb + wb / n_mats * (size_t)spare_mats));
+    if (mb) DMOE_HIP(hipMalloc(&dst->own[4], mb + mb / n_mats * (size_t)spare_mats));
     DMOE_TRY(launch_repack(dst->own[3], dst->own[4], dst->view, st));
     DMOE_HIP(hipStreamSynchronize(st));
     // the MLX-layout copies are no longer needed (fp8 keeps its per-row scales)
@@ -88,6 +93,27 @@ static int adopt(QOwned *dst, const dmoe_qweight *src, int source, const char *n
     dst->view.m_mat = mb / (size_t)dst->view.n_mats;
     if (!keep_scales) dst->view.scales = nullptr;
     dst->view.biases = nullptr;
+    return DMOE_OK;
+}
+
+// Copies the shared expert's packed weights behind the routed experts' (matrix index E of the routed buffers), when
+// the two have the same shape and format. Needs the spare matrix adopt() left room for.
+static bool same_packed_format(const QView &a, const QView &b) {
+    return a.packed && b.packed && a.rows == b.rows && a.cols == b.cols && a.mode == b.mode && a.bits == b.bits &&
+           a.group == b.group && a.mode != DMOE_QUANT_FP8_ROW;
+}
+static int fold_shared(Layer *L, hipStream_t st) {
+    QOwned *routed[3] = {&L->gate, &L->up, &L->down}, *shared[3] = {&L->sgate, &L->sup, &L->sdown};
+    for (int i = 0; i < 3; ++i)
+        if (!same_packed_format(routed[i]->view, shared[i]->view)) return DMOE_OK;
+    for (int i = 0; i < 3; ++i) {
+        const QView &r = routed[i]->view, &s = shared[i]->view;
+        DMOE_HIP(hipMemcpyAsync((uint8_t *)routed[i]->own[3] + (size_t)L->E * r.w_mat, s.w, s.w_mat, hipMemcpyDeviceToDevice, st));
+        if (r.m_mat)
+            DMOE_HIP(hipMemcpyAsync((uint8_t *)routed[i]->own[4] + (size_t)L->E * r.m_mat, s.meta, s.m_mat, hipMemcpyDeviceToDevice, st));
+    }
+    DMOE_HIP(hipStreamSynchronize(st));
+    L->shared_folded = true;
     return DMOE_OK;
 }
 
@@ -166,9 +192,10 @@ struct FwdLayout {
     size_t h, y, sh_h, sh_y, total;
     int max_tiles, tile_m;
     bool small;
+    bool fold; // the shared expert rides in the routed launches: T more sorted rows behind the T*K routed ones
 };
 
-static FwdLayout forward_layout(const Layer *L, int T) {
+static FwdLayout forward_layout(const Layer *L, int T, bool with_shared = true) {
     FwdLayout f;
     Bump b;
     size_t n = (size_t)T * L->K;
@@ -176,12 +203,14 @@ static FwdLayout forward_layout(const Layer *L, int T) {
     // one tile list serves both GEMMs: the smaller of their tile sizes
     f.tile_m = f.small ? small_path_tile_m(n, L->E, std::min(qgemm_skinny_tile_m(L->gate.view), qgemm_skinny_tile_m(L->down.view)))
                        : std::min(qgemm_mfma_tile_m(L->gate.view), qgemm_mfma_tile_m(L->down.view));
-    f.max_tiles = pack_max_tiles(n, L->E, f.tile_m);
+    f.fold = with_shared && f.small && L->shared_folded;
+    const size_t rows = n + (f.fold ? (size_t)T : 0); // sorted rows of the GEMMs
+    f.max_tiles = pack_max_tiles(n, L->E, f.tile_m) + (f.fold ? ceil_div(T, kSkinnyDenseTileM) : 0);
     f.slot_idx = b.take(n * 4);
-    f.order = b.take(n * 4);
+    f.order = b.take(rows * 4);
     f.inv = b.take(n * 4);
-    f.token = b.take(n * 4);
-    f.sorted_e = b.take(n * 4);
+    f.token = b.take(rows * 4);
+    f.sorted_e = b.take(rows * 4);
     f.counts = b.take((size_t)L->E * 4);
     f.offsets = b.take((size_t)(L->E + 1) * 4);
     f.live = b.take((size_t)L->E * 4);
@@ -189,10 +218,10 @@ static FwdLayout forward_layout(const Layer *L, int T) {
     f.tiles = b.take((size_t)(f.max_tiles > 0 ? f.max_tiles : 1) * sizeof(Tile));
     f.n_tiles = b.take(4);
     f.scratch = b.take(pack_scratch_bytes(n, L->E));
-    f.h = b.take(n * (size_t)L->F * 2);
-    f.y = b.take(n * (size_t)L->D * 2);
-    f.sh_h = b.take(L->has_shared ? (size_t)T * L->Fs * 2 : 0);
-    f.sh_y = b.take(L->has_shared ? (size_t)T * L->D * 2 : 0);
+    f.h = b.take(rows * (size_t)L->F * 2);
+    f.y = b.take(rows * (size_t)L->D * 2);
+    f.sh_h = b.take(L->has_shared && !f.fold ? (size_t)T * L->Fs * 2 : 0);
+    f.sh_y = b.take(L->has_shared && !f.fold ? (size_t)T * L->D * 2 : 0);
     f.total = b.off;
     return f;
 }
@@ -230,6 +259,10 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     po.n_live = at<uint32_t>(w, f.n_live);
     po.tiles = at<Tile>(w, f.tiles);
     po.n_tiles = at<uint32_t>(w, f.n_tiles);
+    if (f.fold) {
+        po.dense_rows = (uint32_t)T;
+        po.dense_expert = (uint32_t)L->E;
+    }
     DMOE_TRY(launch_pack(po, d_slots, n, L->K, L->E, f.tile_m, at<void>(w, f.scratch), st));
     DMOE_TRY(stage_end(w, DMOE_STAGE_PACK, st));
 
@@ -246,9 +279,11 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     gu.max_tiles = f.max_tiles;
     gu.tile_m = f.tile_m;
     gu.swiglu_limit = L->swiglu_limit;
+    gu.swiglu_limit_dense = L->shared_swiglu_limit;
     if (L->score_before_down && d_scores) {
         gu.row_scale = d_scores;
         gu.row_scale_idx = po.order;
+        gu.row_scale_rows = (uint32_t)n; // the folded shared expert's rows carry no routing weight
     }
     // Decode-sized batches: the few experts with more than 8 rows go through the big-tile instance, whose tiles
     // depend on nothing the small-tile launches write: two chains (gate/up -> down) on two streams, joined after
@@ -344,9 +379,10 @@ int dmoe_layer_create(dmoe_layer *out, const dmoe_layer_desc *d, dmoe_stream s) 
         L->E = d->gate.n_mats;
         L->swiglu_limit = d->swiglu_limit;
         L->score_before_down = d->score_before_down != 0;
-        if ((rc = adopt(&L->gate, &d->gate, d->weight_source, "gate_proj", st))) break;
-        if ((rc = adopt(&L->up, &d->up, d->weight_source, "up_proj", st))) break;
-        if ((rc = adopt(&L->down, &d->down, d->weight_source, "down_proj", st))) break;
+        const int spare = d->has_shared ? 1 : 0; // room for the shared expert behind the routed ones (fold_shared)
+        if ((rc = adopt(&L->gate, &d->gate, d->weight_source, "gate_proj", st, spare))) break;
+        if ((rc = adopt(&L->up, &d->up, d->weight_source, "up_proj", st, spare))) break;
+        if ((rc = adopt(&L->down, &d->down, d->weight_source, "down_proj", st, spare))) break;
         if (d->has_shared) {
             L->has_shared = true;
             L->Fs = d->shared_gate.rows;
@@ -361,6 +397,7 @@ int dmoe_layer_create(dmoe_layer *out, const dmoe_layer_desc *d, dmoe_stream s) 
             if ((rc = adopt(&L->sgate, &d->shared_gate, d->weight_source, "shared gate_proj", st))) break;
             if ((rc = adopt(&L->sup, &d->shared_up, d->weight_source, "shared up_proj", st))) break;
             if ((rc = adopt(&L->sdown, &d->shared_down, d->weight_source, "shared down_proj", st))) break;
+            if (L->Fs == L->F && (rc = fold_shared(L, st))) break;
         }
         if (d->remap) {
             if (d->n_experts_total < 1) { set_error("layer_create: n_experts_total must be >= 1 with a remap"); rc = DMOE_ERR_INVALID; break; }
@@ -413,9 +450,10 @@ static int forward_common(uint16_t *d_out, uint16_t *y_out, Layer *L, const uint
     DMOE_REQUIRE(((uintptr_t)d_x % 16) == 0, "forward: x must be 16-byte aligned");
     DMOE_REQUIRE(y_out || (d_out && ((uintptr_t)d_out % 16) == 0), "forward: out must be 16-byte aligned and non-null");
     hipStream_t st = to_hip(s);
-    FwdLayout f = forward_layout(L, T);
+    FwdLayout f = forward_layout(L, T, with_shared && !y_out);
     Workspace *w = nullptr;
     DMOE_TRY(workspace_reserve(ws, f.total, &w));
+    w->last_with_shared = with_shared && !y_out;
     const uint32_t *slots = d_indices;
     size_t n = (size_t)T * L->K;
     DMOE_TRY(stage_begin(w, DMOE_STAGE_PACK, st));
@@ -429,12 +467,13 @@ static int forward_common(uint16_t *d_out, uint16_t *y_out, Layer *L, const uint
     // The routed launches are enqueued first: they are the critical path, and the host has all of their run
     // time to enqueue the side stream's work.
     const bool shared = with_shared && L->has_shared && !y_out;
-    if (shared) {
+    const bool side_shared = shared && !f.fold; // else the shared expert is part of the routed launches
+    if (side_shared) {
         DMOE_TRY(side_stream_ready(w));
         DMOE_HIP(hipEventRecord(w->fork, st));
     }
     DMOE_TRY(routed_forward(L, w, f, d_x, slots, d_scores, T, y_out, st));
-    if (shared) {
+    if (side_shared) {
         DMOE_HIP(hipStreamWaitEvent(w->side, w->fork, 0));
         DMOE_TRY(stage_begin(w, DMOE_STAGE_SHARED, w->side));
         DMOE_TRY(shared_forward(L, w, f, d_x, T, w->side));
@@ -442,12 +481,13 @@ static int forward_common(uint16_t *d_out, uint16_t *y_out, Layer *L, const uint
         DMOE_HIP(hipEventRecord(w->join, w->side));
     }
     if (y_out) return DMOE_OK;
-    if (shared) DMOE_HIP(hipStreamWaitEvent(st, w->join, 0));
+    if (side_shared) DMOE_HIP(hipStreamWaitEvent(st, w->join, 0));
     DMOE_TRY(stage_begin(w, DMOE_STAGE_COMBINE, st));
     size_t total = (size_t)T * (L->D / 8);
     hipLaunchKernelGGL(combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, d_out,
                        at<uint16_t>(w, f.y), L->score_before_down ? nullptr : d_scores,
-                       shared ? at<uint16_t>(w, f.sh_y) : nullptr, T, L->K, L->D);
+                       !shared ? nullptr : f.fold ? at<uint16_t>(w, f.y) + (size_t)T * L->K * L->D : at<uint16_t>(w, f.sh_y), T,
+                       L->K, L->D);
     DMOE_LAUNCH_CHECK();
     DMOE_TRY(stage_end(w, DMOE_STAGE_COMBINE, st));
     return DMOE_OK;
@@ -498,7 +538,7 @@ int dmoe_debug_last_activations(uint16_t *d_out, dmoe_layer layer, int T, dmoe_w
     DMOE_REQUIRE(layer.ctx && ws.ctx && d_out, "debug_last_activations: null argument");
     Layer *L = (Layer *)layer.ctx;
     Workspace *w = (Workspace *)ws.ctx;
-    FwdLayout f = forward_layout(L, T);
+    FwdLayout f = forward_layout(L, T, w->last_with_shared);
     DMOE_REQUIRE(w->bytes >= f.total, "debug_last_activations: no forward of this size has run on the workspace");
     size_t n = (size_t)T * L->K, rv = (size_t)L->F / 8, total = n * rv;
     if (total == 0) return DMOE_OK;

@@ -78,7 +78,23 @@ __device__ uint32_t emit_segments(uint32_t count, int e, int E, size_t n, int ti
         if (count > 0 && o.live) o.live[lb] = (uint32_t)e;
         if (e == 0 && o.n_live) *o.n_live = lt;
     }
+    // the folded always-on expert: identity rows behind the routed ones, its tiles ahead of the routed tiles
+    const uint32_t nt_dense = (o.dense_rows + (uint32_t)kSkinnyDenseTileM - 1) / (uint32_t)kSkinnyDenseTileM;
+    for (uint32_t i = threadIdx.x; i < o.dense_rows; i += blockDim.x) {
+        o.order[n + i] = (uint32_t)n + i;
+        if (o.token) o.token[n + i] = i;
+        if (o.sorted_e) o.sorted_e[n + i] = o.dense_expert;
+    }
     if (tile_m > 0 && o.tiles) {
+        for (uint32_t j = threadIdx.x; j < nt_dense; j += blockDim.x) {
+            Tile t;
+            t.expert = o.dense_expert;
+            t.row0 = (uint32_t)n + j * (uint32_t)kSkinnyDenseTileM;
+            uint32_t left = o.dense_rows - j * (uint32_t)kSkinnyDenseTileM;
+            t.nrows = left < (uint32_t)kSkinnyDenseTileM ? left : (uint32_t)kSkinnyDenseTileM;
+            t.flags = kTileDense;
+            o.tiles[j] = t;
+        }
         // tiles stay grouped by expert: tiles of one expert that run together share its weights through L2
         // (emitting the full tiles of all experts first, to shorten the tail of the GEMM launches, measured slower)
         uint32_t nt = (count + (uint32_t)tile_m - 1) / (uint32_t)tile_m, tf;
@@ -89,10 +105,10 @@ __device__ uint32_t emit_segments(uint32_t count, int e, int E, size_t n, int ti
             t.row0 = off + j * (uint32_t)tile_m;
             uint32_t left = count - j * (uint32_t)tile_m;
             t.nrows = left < (uint32_t)tile_m ? left : (uint32_t)tile_m;
-            t.pad = 0;
-            o.tiles[tb + j] = t;
+            t.flags = 0;
+            o.tiles[nt_dense + tb + j] = t;
         }
-        if (e == 0 && o.n_tiles) *o.n_tiles = tf;
+        if (e == 0 && o.n_tiles) *o.n_tiles = nt_dense + tf;
     }
     return off;
 }
@@ -105,16 +121,12 @@ __device__ __forceinline__ void place_row(const PackOut &o, uint32_t pos, uint32
 }
 
 // ---- one launch, n <= 1024 ---------------------------------------------------------------------------------
-__global__ __launch_bounds__(kPackThreads) void pack_fused_kernel(PackOut o, const uint32_t *__restrict__ idx,
-                                                                  uint32_t n, int K, int E, int tile_m) {
-    extern __shared__ uint32_t pack_sm[]; // hist[kPackWaves][E]
-    __shared__ uint32_t scan_sm[kPackWaves + 1];
+// `e` = this thread's expert id (row i = tid), `pack_sm` = hist[kPackWaves][E] in LDS
+__device__ __forceinline__ void pack_fused_body(const PackOut &o, uint32_t e, bool active, uint32_t n, int K, int E,
+                                                int tile_m, uint32_t *pack_sm, uint32_t *scan_sm) {
     const int tid = (int)threadIdx.x, lane = lane_id(), wave = tid >> 6;
     for (int i = tid; i < kPackWaves * E; i += kPackThreads) pack_sm[i] = 0;
     __syncthreads();
-    const uint32_t i = (uint32_t)tid;
-    const bool active = i < n;
-    uint32_t e = active ? idx[i] : 0u;
     if (active && e >= (uint32_t)E) e = (uint32_t)E - 1; // ids are validated by the caller's contract; stay in bounds
     if (active) atomicAdd(&pack_sm[wave * E + e], 1u);
     __syncthreads();
@@ -133,8 +145,17 @@ __global__ __launch_bounds__(kPackThreads) void pack_fused_kernel(PackOut o, con
     uint64_t peers = match_expert(e, active, log2_ceil(E));
     if (active) {
         uint32_t rank = (uint32_t)__popcll(peers & ((1ull << lane) - 1ull));
-        place_row(o, pack_sm[wave * E + e] + rank, i, e, K);
+        place_row(o, pack_sm[wave * E + e] + rank, (uint32_t)tid, e, K);
     }
+}
+
+__global__ __launch_bounds__(kPackThreads) void pack_fused_kernel(PackOut o, const uint32_t *__restrict__ idx,
+                                                                  uint32_t n, int K, int E, int tile_m) {
+    extern __shared__ uint32_t pack_sm[]; // hist[kPackWaves][E]
+    __shared__ uint32_t scan_sm[kPackWaves + 1];
+    const bool active = threadIdx.x < n;
+    const uint32_t e = active ? idx[threadIdx.x] : 0u;
+    pack_fused_body(o, e, active, n, K, E, tile_m, pack_sm, scan_sm);
 }
 
 // ---- three launches, any n --------------------------------------------------------------------------------

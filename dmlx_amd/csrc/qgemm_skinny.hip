@@ -87,6 +87,7 @@ __global__ __launch_bounds__((GATE_UP && RJ == 1 ? 2 : 1) * kSkinnyWaves * 64) v
         if (slot >= n_tiles) return;
     } else {
         t.expert = 0;
+        t.flags = 0;
         t.row0 = slot * (uint32_t)g.tile_m;
         if ((int)t.row0 >= g.dense_rows) return;
         uint32_t left = (uint32_t)g.dense_rows - t.row0;
@@ -334,6 +335,7 @@ __global__ __launch_bounds__((GATE_UP && RJ == 1 ? 2 : 1) * kSkinnyWaves * 64) v
             }
         }
         if (!store_on) return;
+        const float swiglu_limit = (t.flags & kTileDense) ? g.swiglu_limit_dense : g.swiglu_limit;
 #pragma unroll
         for (int j = 0; j < RJ; ++j) {
 #pragma unroll
@@ -341,8 +343,8 @@ __global__ __launch_bounds__((GATE_UP && RJ == 1 ? 2 : 1) * kSkinnyWaves * 64) v
                 const int i = 8 * j + 4 * h + r;
                 if (i >= nrows) continue;
                 const uint32_t p = t.row0 + (uint32_t)i;
-                float val = GATE_UP ? limited_swiglu(v[0][4 * j + r], v[1][4 * j + r], g.swiglu_limit) : v[0][4 * j + r];
-                if (g.row_scale) val *= g.row_scale[g.row_scale_idx ? g.row_scale_idx[p] : p];
+                float val = GATE_UP ? limited_swiglu(v[0][4 * j + r], v[1][4 * j + r], swiglu_limit) : v[0][4 * j + r];
+                if (g.row_scale && p < g.row_scale_rows) val *= g.row_scale[g.row_scale_idx ? g.row_scale_idx[p] : p];
                 const size_t dst = g.out_rows ? g.out_rows[p] : p;
                 g.out[dst * (size_t)g.ldo + n] = f32_to_bf16_bits(val);
             }

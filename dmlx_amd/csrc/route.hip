@@ -4,66 +4,28 @@
 #include <string.h>
 
 #include "common.h"
+#include "route_device.h"
 
 namespace dmoe {
 
-// Monotone u32 key of an f32 for "ascending stable argsort, NaN last, -0 == +0".
-// Never returns 0, so 0 can mark an entry that was already taken.
-__device__ __forceinline__ uint32_t f32_sort_key(float c) {
-    if (c != c) return 0xffffffffu;
-    if (c == 0.0f) return 0x80000000u;
-    uint32_t b = __float_as_uint(c);
-    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
-}
-
 constexpr int kRouteWaves = 4;
 
-// One wavefront per token. The K winners are found by K rounds of a wave-wide arg-max over
-// (key, index) pairs: the pair order makes the HIGHER index win among equal scores, which is what
-// "take the last K columns of a stable ascending argsort" selects, and round r fills column K-1-r so
-// the columns come out in ascending score order.
+// One wavefront per token (route_tokens); EPL = experts per lane
+template <int EPL>
 __global__ __launch_bounds__(kRouteWaves * 64) void route_kernel(
     uint32_t *__restrict__ out_idx, float *__restrict__ out_w, const float *__restrict__ scores,
     const float *__restrict__ bias, const uint8_t *__restrict__ resident, int T, int E, int K,
     int normalize, int apply_scale, float route_scale) {
-    extern __shared__ uint32_t route_keys[]; // [kRouteWaves][E]
     const int wave = (int)(threadIdx.x >> 6), lane = lane_id();
     const int t = (int)blockIdx.x * kRouteWaves + wave;
-    if (t >= T) return; // no block-wide barrier below
-    uint32_t *key = route_keys + (size_t)wave * E;
-    const float *s = scores + (size_t)t * E;
-    // each lane only ever touches entries e == lane (mod 64): no cross-lane hazards on `key`
-    for (int e = lane; e < E; e += 64) {
-        float c = s[e];
-        if (bias) c = c + bias[e];
-        if (resident) c = c + (resident[e] ? 0.0f : -1e9f);
-        key[e] = f32_sort_key(c);
-    }
-    uint32_t my_idx = 0;
-    for (int it = 0; it < K; ++it) {
-        uint32_t bk = 0, bi = 0;
-        for (int e = lane; e < E; e += 64) {
-            uint32_t k = key[e];
-            if (k > bk || (k == bk && (uint32_t)e > bi)) { bk = k; bi = (uint32_t)e; }
-        }
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) {
-            uint32_t ok = (uint32_t)__shfl_xor((int)bk, off, 64);
-            uint32_t oi = (uint32_t)__shfl_xor((int)bi, off, 64);
-            if (ok > bk || (ok == bk && oi > bi)) { bk = ok; bi = oi; }
-        }
-        if ((int)(bi & 63u) == lane) key[bi] = 0; // taken
-        if (lane == K - 1 - it) my_idx = bi;
-    }
-    float my_w = (lane < K) ? s[my_idx] : 0.0f;
-    float sum = 0.0f;
-    for (int j = 0; j < K; ++j) sum += __shfl(my_w, j, 64); // left to right, like a row reduction
-    float w = my_w;
-    if (normalize) w = w / (sum + 1e-20f);
-    if (apply_scale) w = w * route_scale;
+    if (t >= T) return;
+    const float *const rows[1] = {scores + (size_t)t * E};
+    uint32_t my_idx[1];
+    float w[1];
+    route_tokens<1, EPL>(rows, bias, resident, E, K, normalize, apply_scale, route_scale, lane, my_idx, w);
     if (lane < K) {
-        out_idx[(size_t)t * K + lane] = my_idx;
-        out_w[(size_t)t * K + lane] = w;
+        out_idx[(size_t)t * K + lane] = my_idx[0];
+        out_w[(size_t)t * K + lane] = w[0];
     }
 }
 
@@ -75,9 +37,12 @@ static int launch_route(uint32_t *out_idx, float *out_w, const float *scores, co
     if (T == 0) return DMOE_OK;
     DMOE_REQUIRE(out_idx && out_w && scores, "route: null pointer");
     dim3 grid((unsigned)ceil_div(T, kRouteWaves)), block(kRouteWaves * 64);
-    size_t lds = sizeof(uint32_t) * (size_t)kRouteWaves * E;
-    hipLaunchKernelGGL(route_kernel, grid, block, lds, st, out_idx, out_w, scores, bias, resident, T, E,
-                       K, normalize, apply_scale, route_scale);
+    if (E <= 256)
+        hipLaunchKernelGGL(route_kernel<4>, grid, block, 0, st, out_idx, out_w, scores, bias, resident, T, E, K, normalize,
+                           apply_scale, route_scale);
+    else
+        hipLaunchKernelGGL(route_kernel<16>, grid, block, 0, st, out_idx, out_w, scores, bias, resident, T, E, K, normalize,
+                           apply_scale, route_scale);
     DMOE_LAUNCH_CHECK();
     return DMOE_OK;
 }

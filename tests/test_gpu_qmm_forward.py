@@ -167,6 +167,17 @@ def test_score_position_variants(dmoe, orc, ws, before):
     _check_layer(dmoe, orc, ws, wl)
 
 
+@pytest.mark.parametrize("config", [1, 2])
+@pytest.mark.parametrize("limit,shared_limit,before", [(0.05, 0.0, False), (0.05, 0.02, True), (0.0, 0.05, True)])
+def test_shared_expert_inside_the_routed_launches(dmoe, orc, ws, config, limit, shared_limit, before):
+    """Decode sizes with a shared expert of the routed experts' format: its rows ride in the routed GEMM launches as
+    an always-on expert. Limits small enough to clamp, different for routed and shared rows; with the routing weight
+    before the down projection the shared rows must stay unscaled."""
+    wl = workloads.make(config, scale=0.25)
+    wl.swiglu_limit, wl.shared_swiglu_limit, wl.score_before_down = limit, shared_limit, before
+    _check_layer(dmoe, orc, ws, wl)
+
+
 @pytest.mark.parametrize("config,T", [(1, 300), (2, 700)])
 def test_prefill_sized_batch_with_4bit_shared_expert(dmoe, orc, ws, config, T):
     """A prefill-sized batch on the decode configurations: routed experts AND the dense shared expert (4-bit) on the
