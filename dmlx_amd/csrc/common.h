@@ -55,13 +55,9 @@ struct Workspace {
     // side stream (default priority) + fork/join events for work that overlaps the main stream
     hipStream_t side = nullptr;
     hipEvent_t fork = nullptr, join = nullptr;
-    // second side stream: the two tile classes of the skinny GEMMs run side by side
     bool last_with_shared = true; // layout of the last forward on this workspace (for dmoe_debug_last_activations)
-    hipStream_t side2 = nullptr;
-    hipEvent_t packed = nullptr, small_done = nullptr;
 };
 int side_stream_ready(Workspace *w);  // creates the side stream and its events on first use
-int side2_stream_ready(Workspace *w); // same for the second side stream
 
 // stage timing helpers (no-ops unless enabled on the workspace)
 int stage_begin(Workspace *w, int stage, hipStream_t st);
@@ -103,8 +99,8 @@ struct PackOut {
     Tile *tiles = nullptr;       // capacity pack_max_tiles(n, E, tile_m) (+ the dense tiles below)
     uint32_t *n_tiles = nullptr; // device scalar
     // Optional always-on expert folded into the same tile list: `dense_rows` extra sorted rows n .. n+dense_rows-1
-    // (row n+t = token t) of matrix `dense_expert`, cut into tiles of kSkinnyDenseTileM rows that come FIRST in the
-    // list, flagged kTileDense. order / token / sorted_e then hold n + dense_rows entries.
+    // (row n+t = token t) of matrix `dense_expert`, cut into tiles of `tile_m` rows that come FIRST in the list,
+    // flagged kTileDense. order / token / sorted_e then hold n + dense_rows entries.
     uint32_t dense_rows = 0, dense_expert = 0;
 };
 
@@ -166,11 +162,7 @@ constexpr int kSkinnyTileM = 32;          // most rows a skinny tile can hold (s
 constexpr int kSkinnyDenseTileM = 8;      // dense (one matrix) launches: small tiles, many workgroups per row block
 constexpr int kMfmaTileM = 128;
 constexpr int kMfmaWideTileM = 256;
-// The skinny path serves tiles of up to 8 rows and larger tiles with separate launches (the classes are disjoint,
-// so they may run on different streams); kSkinnyAll issues both on `st`.
-enum { kSkinnySmallTiles = 1, kSkinnyBigTiles = 2, kSkinnyAll = 3 };
-int launch_qgemm_skinny(const GemmArgs &g, hipStream_t st, int classes = kSkinnyAll);
-bool qgemm_skinny_has_big_tiles(const GemmArgs &g); // whether the kSkinnyBigTiles launch does anything
+int launch_qgemm_skinny(const GemmArgs &g, hipStream_t st);
 int launch_qgemm_mfma(const GemmArgs &g, hipStream_t st); // picks the wide kernel when the format allows it
 int launch_qgemm_wide(const GemmArgs &g, hipStream_t st);
 bool qgemm_skinny_supports(const QView &b);

@@ -179,14 +179,6 @@ constexpr int kSharedSkinnyRows = 64;
 static bool use_small_path(size_t rows, int n_experts, const QView &b) {
     return qgemm_skinny_supports(b) && rows <= (size_t)kSkinnyAvgRows * (size_t)n_experts;
 }
-// Rows per tile on the small path. Tiles above 8 rows take a second launch on a second stream (and a join),
-// which pays once a fair share of the experts holds that many rows: from an average of kSkinnyBigTileAvgRows
-// rows per expert on. Below that nearly every tile has a few rows, and 8-row tiles in one launch are as fast.
-constexpr int kSkinnyBigTileAvgRows = 3;
-static int small_path_tile_m(size_t rows, int n_experts, int shape_tile_m) {
-    return rows >= (size_t)kSkinnyBigTileAvgRows * (size_t)n_experts ? shape_tile_m : std::min(shape_tile_m, kSkinnyDenseTileM);
-}
-
 struct FwdLayout {
     size_t slot_idx, order, inv, token, sorted_e, counts, offsets, live, n_live, tiles, n_tiles, scratch;
     size_t h, y, sh_h, sh_y, total;
@@ -201,11 +193,11 @@ static FwdLayout forward_layout(const Layer *L, int T, bool with_shared = true) 
     size_t n = (size_t)T * L->K;
     f.small = use_small_path(n, L->E, L->gate.view) && qgemm_skinny_supports(L->down.view);
     // one tile list serves both GEMMs: the smaller of their tile sizes
-    f.tile_m = f.small ? small_path_tile_m(n, L->E, std::min(qgemm_skinny_tile_m(L->gate.view), qgemm_skinny_tile_m(L->down.view)))
+    f.tile_m = f.small ? std::min(qgemm_skinny_tile_m(L->gate.view), qgemm_skinny_tile_m(L->down.view))
                        : std::min(qgemm_mfma_tile_m(L->gate.view), qgemm_mfma_tile_m(L->down.view));
     f.fold = with_shared && f.small && L->shared_folded;
     const size_t rows = n + (f.fold ? (size_t)T : 0); // sorted rows of the GEMMs
-    f.max_tiles = pack_max_tiles(n, L->E, f.tile_m) + (f.fold ? ceil_div(T, kSkinnyDenseTileM) : 0);
+    f.max_tiles = pack_max_tiles(n, L->E, f.tile_m) + (f.fold ? ceil_div(T, f.tile_m) : 0);
     f.slot_idx = b.take(n * 4);
     f.order = b.take(rows * 4);
     f.inv = b.take(n * 4);
@@ -228,20 +220,6 @@ static FwdLayout forward_layout(const Layer *L, int T, bool with_shared = true) 
 
 static int run_gemm(const GemmArgs &g, bool small, hipStream_t st) {
     return small ? launch_qgemm_skinny(g, st) : launch_qgemm_mfma(g, st);
-}
-
-// Skinny GEMM with its two tile classes side by side. The few large tiles are the long poles (one workgroup
-// walks a whole block of weight rows either way, and a large tile restages its activations on the way), so they
-// go first, on `st`; the many small tiles fill the rest of the chip from the workspace's second side stream
-// (which the caller has made wait for the tile list). With `join`, `st` continues only after both.
-static int run_skinny_classes(const GemmArgs &g, Workspace *w, hipStream_t st, bool join) {
-    DMOE_TRY(launch_qgemm_skinny(g, st, kSkinnyBigTiles));
-    DMOE_TRY(launch_qgemm_skinny(g, w->side2, kSkinnySmallTiles));
-    if (join) {
-        DMOE_HIP(hipEventRecord(w->small_done, w->side2));
-        DMOE_HIP(hipStreamWaitEvent(st, w->small_done, 0));
-    }
-    return DMOE_OK;
 }
 
 // routed experts on slot ids: fills ws->y ([T*K, D] bf16 in flat (t,k) order) or `y_out` when given
@@ -285,19 +263,8 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
         gu.row_scale_idx = po.order;
         gu.row_scale_rows = (uint32_t)n; // the folded shared expert's rows carry no routing weight
     }
-    // Decode-sized batches: the few experts with more than 8 rows go through the big-tile instance, whose tiles
-    // depend on nothing the small-tile launches write: two chains (gate/up -> down) on two streams, joined after
-    // the down projection. With stage timing on, the chains also meet between the two GEMMs, so
-    // that each stage's time covers both classes.
-    const bool two_class = f.small && qgemm_skinny_has_big_tiles(gu);
-    if (two_class) {
-        DMOE_TRY(side2_stream_ready(w));
-        DMOE_HIP(hipEventRecord(w->packed, st));
-        DMOE_HIP(hipStreamWaitEvent(w->side2, w->packed, 0));
-    }
     DMOE_TRY(stage_begin(w, DMOE_STAGE_GATE_UP, st));
-    if (two_class) DMOE_TRY(run_skinny_classes(gu, w, st, w->timer.enabled));
-    else DMOE_TRY(run_gemm(gu, f.small, st));
+    DMOE_TRY(run_gemm(gu, f.small, st));
     DMOE_TRY(stage_end(w, DMOE_STAGE_GATE_UP, st));
 
     GemmArgs dn;
@@ -311,8 +278,7 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     dn.max_tiles = f.max_tiles;
     dn.tile_m = f.tile_m;
     DMOE_TRY(stage_begin(w, DMOE_STAGE_DOWN, st));
-    if (two_class) DMOE_TRY(run_skinny_classes(dn, w, st, true));
-    else DMOE_TRY(run_gemm(dn, f.small, st));
+    DMOE_TRY(run_gemm(dn, f.small, st));
     DMOE_TRY(stage_end(w, DMOE_STAGE_DOWN, st));
     return DMOE_OK;
 }
@@ -560,7 +526,7 @@ int dmoe_gather_qmm(uint16_t *d_out, const uint16_t *d_x, const dmoe_qweight *qw
     hipStream_t st = to_hip(s);
     const bool small = use_small_path((size_t)R, v.n_mats, v);
     DMOE_REQUIRE(small || qgemm_mfma_supports(v), "gather_qmm: unsupported weight shape rows=%d cols=%d", v.rows, v.cols);
-    const int tile_m = small ? small_path_tile_m((size_t)R, v.n_mats, qgemm_skinny_tile_m(v)) : qgemm_mfma_tile_m(v);
+    const int tile_m = small ? qgemm_skinny_tile_m(v) : qgemm_mfma_tile_m(v);
     const int max_tiles = pack_max_tiles((size_t)R, v.n_mats, tile_m);
     Bump b;
     size_t o_order = b.take((size_t)R * 4), o_arows = b.take((size_t)R * 4);

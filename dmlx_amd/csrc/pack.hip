@@ -17,6 +17,7 @@ constexpr int kPackWaves = kPackThreads / 64;   // 16
 constexpr int kSubGroups = 4;                   // multi-launch path: groups of 64 rows per wavefront
 constexpr int kSubRows = 64 * kSubGroups;       // 256 rows per sub-chunk
 constexpr int kScatterWaves = 4;                // wavefronts per block in the multi-launch path
+constexpr uint32_t kPackSmallTileRows = 8;      // tiles of at most this many rows go behind the larger ones in the tile list
 
 // exclusive scan of one value per thread across a 1024-thread block; *total gets the block sum
 __device__ uint32_t block_excl_scan(uint32_t v, uint32_t *total, uint32_t *sm /*[kPackWaves + 1]*/) {
@@ -79,7 +80,8 @@ __device__ uint32_t emit_segments(uint32_t count, int e, int E, size_t n, int ti
         if (e == 0 && o.n_live) *o.n_live = lt;
     }
     // the folded always-on expert: identity rows behind the routed ones, its tiles ahead of the routed tiles
-    const uint32_t nt_dense = (o.dense_rows + (uint32_t)kSkinnyDenseTileM - 1) / (uint32_t)kSkinnyDenseTileM;
+    const uint32_t dense_m = tile_m > 0 ? (uint32_t)tile_m : 1u;
+    const uint32_t nt_dense = (o.dense_rows + dense_m - 1) / dense_m;
     for (uint32_t i = threadIdx.x; i < o.dense_rows; i += blockDim.x) {
         o.order[n + i] = (uint32_t)n + i;
         if (o.token) o.token[n + i] = i;
@@ -89,25 +91,34 @@ __device__ uint32_t emit_segments(uint32_t count, int e, int E, size_t n, int ti
         for (uint32_t j = threadIdx.x; j < nt_dense; j += blockDim.x) {
             Tile t;
             t.expert = o.dense_expert;
-            t.row0 = (uint32_t)n + j * (uint32_t)kSkinnyDenseTileM;
-            uint32_t left = o.dense_rows - j * (uint32_t)kSkinnyDenseTileM;
-            t.nrows = left < (uint32_t)kSkinnyDenseTileM ? left : (uint32_t)kSkinnyDenseTileM;
+            t.row0 = (uint32_t)n + j * dense_m;
+            uint32_t left = o.dense_rows - j * dense_m;
+            t.nrows = left < dense_m ? left : dense_m;
             t.flags = kTileDense;
             o.tiles[j] = t;
         }
-        // tiles stay grouped by expert: tiles of one expert that run together share its weights through L2
-        // (emitting the full tiles of all experts first, to shorten the tail of the GEMM launches, measured slower)
-        uint32_t nt = (count + (uint32_t)tile_m - 1) / (uint32_t)tile_m, tf;
-        uint32_t tb = block_excl_scan(nt, &tf, sm);
+        // Tiles above kPackSmallTileRows rows first, then the rest, each group in expert order. On the decode path a
+        // large tile takes about twice as long as a small one (it restages its activations on the way), so the few
+        // of them start with the launch instead of stretching its tail; on the prefill path this puts the full
+        // tiles of all experts ahead of the partial ones.
+        const uint32_t tm = (uint32_t)tile_m;
+        const uint32_t nt = (count + tm - 1) / tm;
+        const uint32_t last_rows = count - (nt ? (nt - 1) * tm : 0);           // rows of the expert's last tile
+        const uint32_t n_big = nt == 0 ? 0 : (nt - 1) + (last_rows > kPackSmallTileRows ? 1u : 0u);
+        uint32_t total_big, total_small;
+        const uint32_t big_base = block_excl_scan(n_big, &total_big, sm);
+        const uint32_t small_base = block_excl_scan(nt - n_big, &total_small, sm);
         for (uint32_t j = 0; j < nt; ++j) {
             Tile t;
             t.expert = (uint32_t)e;
-            t.row0 = off + j * (uint32_t)tile_m;
-            uint32_t left = count - j * (uint32_t)tile_m;
-            t.nrows = left < (uint32_t)tile_m ? left : (uint32_t)tile_m;
+            t.row0 = off + j * tm;
+            uint32_t left = count - j * tm;
+            t.nrows = left < tm ? left : tm;
             t.flags = 0;
-            o.tiles[nt_dense + tb + j] = t;
+            const uint32_t pos = j < n_big ? big_base + j : total_big + small_base;
+            o.tiles[nt_dense + pos] = t;
         }
+        const uint32_t tf = total_big + total_small;
         if (e == 0 && o.n_tiles) *o.n_tiles = nt_dense + tf;
     }
     return off;

@@ -9,11 +9,11 @@
 // B operand, so every lane's accumulators belong to ITS weight row and rows 8j+4h..8j+4h+3 of the tile, and
 // nothing has to be reduced across lanes.
 //
-// Two instances serve two classes of tiles with separate launches (a launch skips the tiles of the other
-// class). Up to 8 rows - nearly every tile at decode - the rows stay whole in LDS and a lane keeps 4
-// accumulators; gate and up rows go to separate wavefronts. 9 to 32 rows: LDS holds a quarter of every row,
-// restaged three times on the way, and a lane keeps 16 accumulators; an expert with many rows then still
-// streams its weights once instead of once per 8 rows.
+// Up to 8 rows - nearly every tile at decode - the tile's rows stay whole in LDS and a lane keeps 4 accumulators.
+// 9 to 32 rows: LDS holds a half or a quarter of every row, restaged on the way, and a lane keeps up to 16
+// accumulators; an expert with many rows then still streams its weights once instead of once per 8 rows.
+// Gate and up rows go to separate wavefronts (eight per workgroup, paired through LDS at the end): half the
+// registers per wavefront, twice the wavefronts per SIMD to overlap decode, matrix and memory waits.
 //
 // 4-bit affine weights (group >= 64) are never multiplied out. Codes become the bf16 numbers (128 + q)
 // with one AND-OR per pair; both halves of a step lie in the same scale group, so the matrix core
@@ -30,11 +30,6 @@
 namespace dmoe {
 
 constexpr int kSkinnyWaves = 4;          // 32-row blocks of weight rows per workgroup
-// Two instances per format. Tiles of at most one row block (the bulk at decode): gate/up launches give each
-// projection its own wavefront (eight per workgroup, paired through LDS at the end) - half the registers per
-// wavefront, twice the wavefronts per SIMD to overlap decode, matrix and memory waits. Larger tiles: four
-// wavefronts with both projections each; their extra accumulators would cost the first instance its occupancy.
-constexpr int kSkinnyBigRowBlocks = 4;   // row blocks of the big-tile instance (the other instance has one)
 constexpr int kSkinnyStages = 8;
 constexpr int kSkinnyRowBlock = 8;       // tile rows per row block: the LDS window holds 8 whole rows of activations
 
@@ -67,32 +62,19 @@ struct SkinnyStage {
     uint32_t sb[NM][2];
 };
 
-template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED, int RJ>
-__global__ __launch_bounds__((GATE_UP && RJ == 1 ? 2 : 1) * kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArgs g) {
+// One tile, start to finish. RJT = 1: tiles of one row block (4 accumulators per lane, no restaging); RJT = 4: larger
+// tiles (16 accumulators; a tile of two row blocks computes four, the surplus rows are never stored). The kernel
+// calls one or the other right after fetching the tile, so the two share nothing but the arguments and each keeps
+// its own register allocation.
+template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED, int RJT>
+__device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, uint8_t *skinny_lds) {
     using CS = ChunkStream<Fmt, PACKED>;
     constexpr int KV = Fmt::kVals;   // values per 16-byte chunk
     constexpr int KSTEP = 2 * KV;    // reduction elements per step (both lane halves)
     constexpr int NJ = KV / 8;       // MFMAs (K = 16) per step
-    constexpr bool SPLIT = GATE_UP && RJ == 1;      // see kSkinnyBigRowBlocks
-    constexpr int RP = RJ * kSkinnyRowBlock;        // rows the LDS layout is made for
+    constexpr bool SPLIT = GATE_UP;                 // gate and up rows on separate wavefronts
     constexpr int NM = GATE_UP && !SPLIT ? 2 : 1;   // projections per wavefront
     constexpr int WAVES = (SPLIT ? 2 : 1) * kSkinnyWaves;
-    extern __shared__ __attribute__((aligned(16))) uint8_t skinny_lds[];
-
-    Tile t;
-    const uint32_t slot = blockIdx.y;
-    if (g.tiles) {
-        const uint32_t n_tiles = *g.n_tiles; // both loads are issued before either is needed
-        t = g.tiles[slot];                   // the list has room for every launched slot
-        if (slot >= n_tiles) return;
-    } else {
-        t.expert = 0;
-        t.flags = 0;
-        t.row0 = slot * (uint32_t)g.tile_m;
-        if ((int)t.row0 >= g.dense_rows) return;
-        uint32_t left = (uint32_t)g.dense_rows - t.row0;
-        t.nrows = left < (uint32_t)g.tile_m ? left : (uint32_t)g.tile_m;
-    }
     const int tid = (int)threadIdx.x, lane = tid & 63, ln = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int cols = g.b0.cols, n_out = g.b0.rows;
@@ -121,14 +103,16 @@ __global__ __launch_bounds__((GATE_UP && RJ == 1 ? 2 : 1) * kSkinnyWaves * 64) v
     };
 
     // ---- activations of the tile in LDS -------------------------------------------------------------------
-    // The LDS window holds 8 full rows' worth of activations. A tile of up to 8 rows (RJ = 1) keeps its rows
-    // whole; a larger one (RJ = 4, up to 32 rows) keeps a quarter of every row and is restaged at the three span
-    // boundaries, so that an expert with many rows still streams its weights only once. Only the rows the tile
-    // has are staged: row m of the A operand only reaches accumulator row m, rows past the tile are never stored.
+    // The LDS window holds 8 full rows' worth of activations. A tile of up to 8 rows (one row block, the bulk at
+    // decode) keeps its rows whole; one of up to 16 (32) rows keeps a half (a quarter) of every row and is restaged
+    // at the span boundaries, so that an expert with many rows still streams its weights only once. Only the rows
+    // the tile has are staged: row m of the A operand only reaches accumulator row m, rows past the tile are never
+    // stored. The matrix instruction always covers 32 rows; what grows with the tile is the number of accumulators
+    // a lane scales and keeps (4 per row block), behind wave-uniform branches.
     const int nrows = __builtin_amdgcn_readfirstlane((int)t.nrows);
-    // each launch serves one class of tiles: up to one row block, or more (workgroup-uniform: nothing has synchronized yet)
-    if (RJ == 1 ? nrows > kSkinnyRowBlock : nrows <= kSkinnyRowBlock) return;
-    const int span_steps = n_steps / RJ;             // the launcher only builds larger tiles when this divides
+    const int rj = RJT == 1 ? 1 : nrows <= 2 * kSkinnyRowBlock ? 2 : 4; // row blocks = spans of the reduction
+    const int rp = rj * kSkinnyRowBlock;             // rows the LDS layout is made for
+    const int span_steps = n_steps / rj;             // the launcher only builds larger tiles when this divides
     const int span_bytes = span_steps * KSTEP * 2;   // bytes of one row in one span
     const int pitch = span_bytes + 16;               // +16 keeps neighbouring rows on different banks
     uint8_t *xs_lds = skinny_lds;
@@ -171,7 +155,7 @@ __global__ __launch_bounds__((GATE_UP && RJ == 1 ? 2 : 1) * kSkinnyWaves * 64) v
             sum += skinny_dpp<0xB1>(sum);  // lane ^ 1 (quad_perm 1,0,3,2)
             sum += skinny_dpp<0x4E>(sum);  // lane ^ 2 (quad_perm 2,3,0,1)
             sum += skinny_dpp<0x141>(sum); // the other quad of the eight lanes (row_half_mirror)
-            if ((pc & 7) == 0) gs_lds[(pc >> 3) * RP + r] = sum;
+            if ((pc & 7) == 0) gs_lds[(pc >> 3) * rp + r] = sum;
         }
     };
 
@@ -198,63 +182,65 @@ __global__ __launch_bounds__((GATE_UP && RJ == 1 ? 2 : 1) * kSkinnyWaves * 64) v
     const uint8_t *xlane = xs_lds + (ln < nrows ? ln : 0) * pitch + h * KV * 2;
     const uint32_t mask = vgpr_const32(0x000f000fu), magic = vgpr_const32(0x43004300u);
 
-    // RJ row blocks of the tile: accumulator registers 4 j + r of a lane belong to tile row 8 j + 4 h + r
+    // accumulator registers 4 j + r of a lane belong to tile row 8 j + 4 h + r (row block j)
     {
         f32x16_t acc[NM];
 #pragma unroll
         for (int mi = 0; mi < NM; ++mi)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[mi][r] = 0.0f;
-        float facc[NM][4 * RJ];
+        float facc[NM][4 * RJT];
 #pragma unroll
         for (int mi = 0; mi < NM; ++mi)
 #pragma unroll
-            for (int r = 0; r < 4 * RJ; ++r) facc[mi][r] = 0.0f;
+            for (int r = 0; r < 4 * RJT; ++r) facc[mi][r] = 0.0f;
 
         // One step: decode every projection's chunk first, then issue the matrix instructions of the projections
         // alternately (independent accumulation chains), then apply the scales. `xs` = step within the span.
         auto consume = [&](int xs, const SkinnyStage<NM> &s) {
-            bf16x8_t xf[NJ];
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                uint4 q = *(const uint4 *)(xlane + (size_t)xs * KSTEP * 2 + j * 16);
-                xf[j] = __builtin_bit_cast(bf16x8_t, q);
-            }
-            float4 gsum[RJ];
-            if (FACTORED) {
-#pragma unroll
-                for (int j = 0; j < RJ; ++j) gsum[j] = *(const float4 *)(gs_lds + xs * RP + 8 * j + 4 * h);
-            }
-            uint32_t wp[NM][KV / 2];
+            const uint8_t *xstep = xlane + (size_t)xs * KSTEP * 2;
+            const float *gs_step = gs_lds + xs * rp + 4 * h;
             Meta meta[NM];
 #pragma unroll
-            for (int mi = 0; mi < NM; ++mi) {
-                meta[mi] = CS::meta(s.sb[mi]);
-                if (FACTORED) {
-                    codes_to_bf16(s.raw[mi].x, mask, magic, wp[mi]);
-                    codes_to_bf16(s.raw[mi].y, mask, magic, wp[mi] + 4);
-                    codes_to_bf16(s.raw[mi].z, mask, magic, wp[mi] + 8);
-                    codes_to_bf16(s.raw[mi].w, mask, magic, wp[mi] + 12);
-                } else {
-                    Fmt::decode_fast(s.raw[mi], meta[mi], wp[mi]);
-                }
-            }
+            for (int mi = 0; mi < NM; ++mi) meta[mi] = CS::meta(s.sb[mi]);
             f32x16_t p[NM];
             if (FACTORED) {
+                // word j of the chunk is exactly the B operand of the step's j-th matrix instruction: decode it
+                // right before its use (the instructions of one projection are a dependent chain anyway), so only
+                // one operand pair is live at a time
 #pragma unroll
                 for (int mi = 0; mi < NM; ++mi)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) p[mi][r] = 0.0f;
-            }
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) {
+                for (int j = 0; j < NJ; ++j) {
+                    const uint4 xq = *(const uint4 *)(xstep + j * 16);
 #pragma unroll
-                for (int mi = 0; mi < NM; ++mi) {
-                    uint4 q = make_uint4(wp[mi][4 * j], wp[mi][4 * j + 1], wp[mi][4 * j + 2], wp[mi][4 * j + 3]);
-                    if (FACTORED)
-                        p[mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[j], __builtin_bit_cast(bf16x8_t, q), p[mi], 0, 0, 0);
-                    else
+                    for (int mi = 0; mi < NM; ++mi) {
+                        const uint32_t word = j == 0 ? s.raw[mi].x : j == 1 ? s.raw[mi].y : j == 2 ? s.raw[mi].z : s.raw[mi].w;
+                        uint32_t wp[4];
+                        codes_to_bf16(word, mask, magic, wp);
+                        const uint4 q = make_uint4(wp[0], wp[1], wp[2], wp[3]);
+                        p[mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, xq), __builtin_bit_cast(bf16x8_t, q), p[mi], 0, 0, 0);
+                    }
+                }
+            } else {
+                bf16x8_t xf[NJ];
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    uint4 q = *(const uint4 *)(xstep + j * 16);
+                    xf[j] = __builtin_bit_cast(bf16x8_t, q);
+                }
+                uint32_t wp[NM][KV / 2];
+#pragma unroll
+                for (int mi = 0; mi < NM; ++mi) Fmt::decode_fast(s.raw[mi], meta[mi], wp[mi]);
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+                    for (int mi = 0; mi < NM; ++mi) {
+                        uint4 q = make_uint4(wp[mi][4 * j], wp[mi][4 * j + 1], wp[mi][4 * j + 2], wp[mi][4 * j + 3]);
                         acc[mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[j], __builtin_bit_cast(bf16x8_t, q), acc[mi], 0, 0, 0);
+                    }
                 }
             }
             if (FACTORED) {
@@ -262,14 +248,18 @@ __global__ __launch_bounds__((GATE_UP && RJ == 1 ? 2 : 1) * kSkinnyWaves * 64) v
                 for (int mi = 0; mi < NM; ++mi) {
                     const float boff = fmaf(-128.0f, meta[mi].s, meta[mi].b);
 #pragma unroll
-                    for (int j = 0; j < RJ; ++j) {
-                        facc[mi][4 * j + 0] = fmaf(meta[mi].s, p[mi][4 * j + 0], fmaf(boff, gsum[j].x, facc[mi][4 * j + 0]));
-                        facc[mi][4 * j + 1] = fmaf(meta[mi].s, p[mi][4 * j + 1], fmaf(boff, gsum[j].y, facc[mi][4 * j + 1]));
-                        facc[mi][4 * j + 2] = fmaf(meta[mi].s, p[mi][4 * j + 2], fmaf(boff, gsum[j].z, facc[mi][4 * j + 2]));
-                        facc[mi][4 * j + 3] = fmaf(meta[mi].s, p[mi][4 * j + 3], fmaf(boff, gsum[j].w, facc[mi][4 * j + 3]));
+                    for (int j = 0; j < RJT; ++j) {
+                        const float4 gsum = *(const float4 *)(gs_step + 8 * j); // past the tile's row blocks: stale sums, unused rows
+                        facc[mi][4 * j + 0] = fmaf(meta[mi].s, p[mi][4 * j + 0], fmaf(boff, gsum.x, facc[mi][4 * j + 0]));
+                        facc[mi][4 * j + 1] = fmaf(meta[mi].s, p[mi][4 * j + 1], fmaf(boff, gsum.y, facc[mi][4 * j + 1]));
+                        facc[mi][4 * j + 2] = fmaf(meta[mi].s, p[mi][4 * j + 2], fmaf(boff, gsum.z, facc[mi][4 * j + 2]));
+                        facc[mi][4 * j + 3] = fmaf(meta[mi].s, p[mi][4 * j + 3], fmaf(boff, gsum.w, facc[mi][4 * j + 3]));
                     }
                 }
             }
+            // with 16 products per lane alive, letting the next step's matrix instructions start before this step's
+            // scaling has finished would double them: keep the steps apart (other wavefronts fill the wait)
+            if (RJT > 1) __builtin_amdgcn_sched_barrier(0);
         };
 
         // whole rounds of the ring run without guards (the look-ahead is clamped onto the last step: a few repeated
@@ -278,7 +268,7 @@ __global__ __launch_bounds__((GATE_UP && RJ == 1 ? 2 : 1) * kSkinnyWaves * 64) v
         int x0 = 0, next_span = span_steps; // first step of the span in LDS, first step of the next one
 #pragma unroll 1
         for (int s0 = 0; s0 < full; s0 += kSkinnyStages) {
-            if (RJ > 1 && s0 == next_span) {
+            if (RJT > 1 && s0 == next_span) {
                 // the next span of the activations replaces the one in LDS (the weight ring stays in flight; its
                 // loads are older than these requests, so the wait covers nothing that was not due anyway)
                 __syncthreads();
@@ -299,7 +289,7 @@ __global__ __launch_bounds__((GATE_UP && RJ == 1 ? 2 : 1) * kSkinnyWaves * 64) v
                 consume(step - x0, ring[j]);
             }
         }
-        if (full < n_steps) { // only tiles of one row block get here (larger ones need whole rounds per span)
+        if (RJT == 1 && full < n_steps) { // only tiles of one row block get here (larger ones need whole rounds per span)
 #pragma unroll
             for (int j = 0; j < kSkinnyStages; ++j) {
                 const int step = full + j;
@@ -309,27 +299,27 @@ __global__ __launch_bounds__((GATE_UP && RJ == 1 ? 2 : 1) * kSkinnyWaves * 64) v
         }
 
         // ---- epilogue: this lane holds rows 8 j + 4 h + r of the tile for weight row n ----------------------
-        float v[2][4 * RJ];
+        float v[2][4 * RJT];
 #pragma unroll
         for (int mi = 0; mi < NM; ++mi) {
             const QView &q = (mi + proj) == 0 ? g.b0 : g.b1;
             const float rs = Fmt::kRowScale ? *(const float *)(q.scales + e * q.s_mat + (size_t)n * q.s_row) : 1.0f;
 #pragma unroll
-            for (int r = 0; r < 4 * RJ; ++r) v[mi][r] = (FACTORED ? facc[mi][r] : acc[mi][r]) * rs;
+            for (int r = 0; r < 4 * RJT; ++r) v[mi][r] = (FACTORED ? facc[mi][r] : acc[mi][r]) * rs;
         }
         if (SPLIT) {
             // the up wavefront hands its values to the gate wavefront of the same weight rows, through the
             // activation window (free once every wavefront has left the main loop)
-            float4 *xch = (float4 *)xs_lds + ((wave >> 1) * 64 + lane) * RJ;
+            float4 *xch = (float4 *)xs_lds + ((wave >> 1) * 64 + lane) * RJT;
             __syncthreads();
             if (proj == 1) {
 #pragma unroll
-                for (int j = 0; j < RJ; ++j) xch[j] = make_float4(v[0][4 * j], v[0][4 * j + 1], v[0][4 * j + 2], v[0][4 * j + 3]);
+                for (int j = 0; j < RJT; ++j) xch[j] = make_float4(v[0][4 * j], v[0][4 * j + 1], v[0][4 * j + 2], v[0][4 * j + 3]);
             }
             __syncthreads();
             if (proj == 1) return;
 #pragma unroll
-            for (int j = 0; j < RJ; ++j) {
+            for (int j = 0; j < RJT; ++j) {
                 const float4 u = xch[j];
                 v[1][4 * j] = u.x, v[1][4 * j + 1] = u.y, v[1][4 * j + 2] = u.z, v[1][4 * j + 3] = u.w;
             }
@@ -337,7 +327,7 @@ __global__ __launch_bounds__((GATE_UP && RJ == 1 ? 2 : 1) * kSkinnyWaves * 64) v
         if (!store_on) return;
         const float swiglu_limit = (t.flags & kTileDense) ? g.swiglu_limit_dense : g.swiglu_limit;
 #pragma unroll
-        for (int j = 0; j < RJ; ++j) {
+        for (int j = 0; j < RJT; ++j) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int i = 8 * j + 4 * h + r;
@@ -352,20 +342,43 @@ __global__ __launch_bounds__((GATE_UP && RJ == 1 ? 2 : 1) * kSkinnyWaves * 64) v
     }
 }
 
+template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED>
+__global__ __launch_bounds__((GATE_UP ? 2 : 1) * kSkinnyWaves * 64, GATE_UP ? 4 : 1) void qgemm_skinny_kernel(GemmArgs g) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t skinny_lds[];
+    Tile t;
+    const uint32_t slot = blockIdx.y;
+    if (g.tiles) {
+        const uint32_t n_tiles = *g.n_tiles; // both loads are issued before either is needed
+        t = g.tiles[slot];                   // the list has room for every launched slot
+        if (slot >= n_tiles) return;
+    } else {
+        t.expert = 0;
+        t.flags = 0;
+        t.row0 = slot * (uint32_t)g.tile_m;
+        if ((int)t.row0 >= g.dense_rows) return;
+        uint32_t left = (uint32_t)g.dense_rows - t.row0;
+        t.nrows = left < (uint32_t)g.tile_m ? left : (uint32_t)g.tile_m;
+    }
+    if (__builtin_amdgcn_readfirstlane((int)t.nrows) <= kSkinnyRowBlock) skinny_tile<Fmt, GATE_UP, FACTORED, PACKED, 1>(g, t, skinny_lds);
+    else skinny_tile<Fmt, GATE_UP, FACTORED, PACKED, kSkinnyTileM / kSkinnyRowBlock>(g, t, skinny_lds);
+}
+
 static int skinny_vals(const QView &b) {
     return (b.mode == DMOE_QUANT_AFFINE && b.bits == 4) || b.mode == DMOE_QUANT_MXFP4 ? 32 : 16;
 }
 static size_t skinny_lds_bytes(const QView &b) {
     size_t x = (size_t)kSkinnyRowBlock * (size_t)b.cols * 2 + (size_t)kSkinnyTileM * 16;
     size_t sums = (size_t)(b.cols / (2 * skinny_vals(b))) * kSkinnyRowBlock * sizeof(float);
-    return x + sums;
+    return x + sums + 128; // a two-row-block tile reads (and ignores) up to 24 floats past its last step's sums
 }
 
-// Rows per tile to build tile lists with for this weight shape: the big-tile instance splits the reduction into
-// kSkinnyBigRowBlocks spans, each a whole number of ring rounds.
+// Rows per tile to build tile lists with for this weight shape: a tile of 2 (4) row blocks splits the reduction
+// into 2 (4) spans, each a whole number of ring rounds.
 int qgemm_skinny_tile_m(const QView &b) {
     const int n_steps = b.cols / (2 * skinny_vals(b));
-    return n_steps % (kSkinnyBigRowBlocks * kSkinnyStages) == 0 ? kSkinnyBigRowBlocks * kSkinnyRowBlock : kSkinnyRowBlock;
+    if (n_steps % (4 * kSkinnyStages) == 0) return 4 * kSkinnyRowBlock;
+    if (n_steps % (2 * kSkinnyStages) == 0) return 2 * kSkinnyRowBlock;
+    return kSkinnyRowBlock;
 }
 
 bool qgemm_skinny_supports(const QView &b) {
@@ -375,10 +388,9 @@ bool qgemm_skinny_supports(const QView &b) {
 struct SkinnyLaunch {
     const GemmArgs &g;
     hipStream_t st;
-    int classes;
-    template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED, int RJ>
-    int go_class() {
-        auto kern = qgemm_skinny_kernel<Fmt, GATE_UP, FACTORED, PACKED, RJ>;
+    template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED>
+    int go() {
+        auto kern = qgemm_skinny_kernel<Fmt, GATE_UP, FACTORED, PACKED>;
         const size_t lds = skinny_lds_bytes(g.b0);
         static thread_local size_t allowed = 0; // per instantiation: raise the dynamic LDS limit once
         if (lds > allowed) {
@@ -386,17 +398,9 @@ struct SkinnyLaunch {
             allowed = 150 * 1024;
         }
         dim3 grid((unsigned)ceil_div(g.b0.rows, kSkinnyWaves * 32), (unsigned)g.max_tiles);
-        dim3 block((GATE_UP && RJ == 1 ? 2 : 1) * kSkinnyWaves * 64);
+        dim3 block((GATE_UP ? 2 : 1) * kSkinnyWaves * 64);
         hipLaunchKernelGGL(kern, grid, block, lds, st, g);
         DMOE_LAUNCH_CHECK();
-        return DMOE_OK;
-    }
-    template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED>
-    int go() {
-        if (classes & kSkinnySmallTiles) DMOE_TRY((go_class<Fmt, GATE_UP, FACTORED, PACKED, 1>()));
-        // tile lists built with one row block per tile hold no larger tile
-        if ((classes & kSkinnyBigTiles) && g.tile_m > kSkinnyRowBlock)
-            DMOE_TRY((go_class<Fmt, GATE_UP, FACTORED, PACKED, kSkinnyBigRowBlocks>()));
         return DMOE_OK;
     }
     template <typename Fmt>
@@ -413,9 +417,7 @@ struct SkinnyLaunch {
     }
 };
 
-bool qgemm_skinny_has_big_tiles(const GemmArgs &g) { return g.tile_m > kSkinnyRowBlock; }
-
-int launch_qgemm_skinny(const GemmArgs &g, hipStream_t st, int classes) {
+int launch_qgemm_skinny(const GemmArgs &g, hipStream_t st) {
     DMOE_REQUIRE(qgemm_skinny_supports(g.b0), "skinny GEMM: unsupported weight shape (cols=%d)", g.b0.cols);
     DMOE_REQUIRE(g.max_tiles >= 0 && g.max_tiles <= 65535, "skinny GEMM: %d tiles exceed the grid limit", g.max_tiles);
     DMOE_REQUIRE(g.a && g.out && g.ldo > 0 && ((uintptr_t)g.a % 16) == 0, "skinny GEMM: bad pointer");
@@ -426,7 +428,7 @@ int launch_qgemm_skinny(const GemmArgs &g, hipStream_t st, int classes) {
                          g.b1.bits == g.b0.bits && g.b1.group == g.b0.group && g.b1.packed == g.b0.packed,
                      "skinny GEMM: gate and up projections differ in shape or format");
     if (g.max_tiles == 0) return DMOE_OK;
-    return dispatch_format(g.b0, SkinnyLaunch{g, st, classes});
+    return dispatch_format(g.b0, SkinnyLaunch{g, st});
 }
 
 } // namespace dmoe

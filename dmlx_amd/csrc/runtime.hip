@@ -46,14 +46,6 @@ int side_stream_ready(Workspace *w) {
     return DMOE_OK;
 }
 
-int side2_stream_ready(Workspace *w) {
-    if (w->side2) return DMOE_OK;
-    DMOE_HIP(hipStreamCreateWithFlags(&w->side2, hipStreamNonBlocking));
-    DMOE_HIP(hipEventCreateWithFlags(&w->packed, hipEventDisableTiming));
-    DMOE_HIP(hipEventCreateWithFlags(&w->small_done, hipEventDisableTiming));
-    return DMOE_OK;
-}
-
 int stage_flush(Workspace *w) {
     StageTimer &t = w->timer;
     for (int i = 0; i < DMOE_STAGE_COUNT; ++i) {
@@ -236,10 +228,6 @@ int dmoe_workspace_destroy(dmoe_workspace ws) {
     if (w->fork) (void)hipEventDestroy(w->fork);
     if (w->join) (void)hipEventDestroy(w->join);
     if (w->side) (void)hipStreamDestroy(w->side);
-    if (w->side2) (void)hipStreamSynchronize(w->side2);
-    if (w->packed) (void)hipEventDestroy(w->packed);
-    if (w->small_done) (void)hipEventDestroy(w->small_done);
-    if (w->side2) (void)hipStreamDestroy(w->side2);
     hipError_t e = w->base ? hipFree(w->base) : hipSuccess;
     delete w;
     if (e != hipSuccess) return hip_fail(e, "hipFree(workspace)");
