@@ -73,6 +73,9 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
     constexpr int KSTEP = 2 * KV;    // reduction elements per step (both lane halves)
     constexpr int NJ = KV / 8;       // MFMAs (K = 16) per step
     constexpr bool SPLIT = GATE_UP;                 // gate and up rows on separate wavefronts
+    // depth of the weight ring: the large-tile copy keeps 16 accumulators per lane and takes a shallower ring to
+    // stay inside the same register budget (span boundaries stay whole ring rounds either way)
+    constexpr int STAGES = RJT == 1 ? kSkinnyStages : kSkinnyStages / 2;
     constexpr int NM = GATE_UP && !SPLIT ? 2 : 1;   // projections per wavefront
     constexpr int WAVES = (SPLIT ? 2 : 1) * kSkinnyWaves;
     const int tid = (int)threadIdx.x, lane = tid & 63, ln = lane & 31, h = lane >> 5;
@@ -162,14 +165,14 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
     // Loads return in issue order: the first span is requested ahead of the first stages of the weight ring, and
     // the wait below lets the ring stay in flight.
     issue_x(0);
-    SkinnyStage<NM> ring[kSkinnyStages];
+    SkinnyStage<NM> ring[STAGES];
 #pragma unroll
     for (int mi = 0; mi < NM; ++mi) cs[mi].pin(); // keeps the weight loads behind the requests above
 #pragma unroll
-    for (int j = 0; j < kSkinnyStages - 1; ++j)
+    for (int j = 0; j < STAGES - 1; ++j)
         if (j < n_steps) load_stage(j, ring[j]);
     // every ring stage holds at least NM loads younger than the activation requests
-    if (n_steps >= kSkinnyStages - 1) __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt((kSkinnyStages - 1) * NM));
+    if (n_steps >= STAGES - 1) __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt((STAGES - 1) * NM));
     else __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt(0));
     __syncthreads();
     if (FACTORED) {
@@ -264,10 +267,10 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
 
         // whole rounds of the ring run without guards (the look-ahead is clamped onto the last step: a few repeated
         // loads at the very end instead of a branch per step); a partial last round runs the guarded copy
-        const int full = n_steps / kSkinnyStages * kSkinnyStages;
+        const int full = n_steps / STAGES * STAGES;
         int x0 = 0, next_span = span_steps; // first step of the span in LDS, first step of the next one
 #pragma unroll 1
-        for (int s0 = 0; s0 < full; s0 += kSkinnyStages) {
+        for (int s0 = 0; s0 < full; s0 += STAGES) {
             if (RJT > 1 && s0 == next_span) {
                 // the next span of the activations replaces the one in LDS (the weight ring stays in flight; its
                 // loads are older than these requests, so the wait covers nothing that was not due anyway)
@@ -283,17 +286,17 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
                 next_span += span_steps;
             }
 #pragma unroll
-            for (int j = 0; j < kSkinnyStages; ++j) {
-                const int step = s0 + j, ahead = step + kSkinnyStages - 1;
-                load_stage(ahead < n_steps ? ahead : n_steps - 1, ring[(j + kSkinnyStages - 1) % kSkinnyStages]);
+            for (int j = 0; j < STAGES; ++j) {
+                const int step = s0 + j, ahead = step + STAGES - 1;
+                load_stage(ahead < n_steps ? ahead : n_steps - 1, ring[(j + STAGES - 1) % STAGES]);
                 consume(step - x0, ring[j]);
             }
         }
         if (RJT == 1 && full < n_steps) { // only tiles of one row block get here (larger ones need whole rounds per span)
 #pragma unroll
-            for (int j = 0; j < kSkinnyStages; ++j) {
+            for (int j = 0; j < STAGES; ++j) {
                 const int step = full + j;
-                if (step + kSkinnyStages - 1 < n_steps) load_stage(step + kSkinnyStages - 1, ring[(j + kSkinnyStages - 1) % kSkinnyStages]);
+                if (step + STAGES - 1 < n_steps) load_stage(step + STAGES - 1, ring[(j + STAGES - 1) % STAGES]);
                 if (step < n_steps) consume(step, ring[j]);
             }
         }
@@ -343,7 +346,7 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
 }
 
 template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED>
-__global__ __launch_bounds__((GATE_UP ? 2 : 1) * kSkinnyWaves * 64, GATE_UP ? 4 : 1) void qgemm_skinny_kernel(GemmArgs g) {
+__global__ __launch_bounds__((GATE_UP ? 2 : 1) * kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArgs g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t skinny_lds[];
     Tile t;
     const uint32_t slot = blockIdx.y;
