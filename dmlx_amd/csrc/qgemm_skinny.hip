@@ -77,7 +77,8 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
     // stay inside the same register budget (span boundaries stay whole ring rounds either way)
     constexpr int STAGES = RJT == 1 ? kSkinnyStages : kSkinnyStages / 2;
     constexpr int NM = GATE_UP && !SPLIT ? 2 : 1;   // projections per wavefront
-    constexpr int WAVES = (SPLIT ? 2 : 1) * kSkinnyWaves;
+    constexpr int WAVES = 2 * kSkinnyWaves;         // eight wavefronts share one staging of the tile's activations
+    constexpr int CG = SPLIT ? kSkinnyWaves : WAVES; // 32-row blocks of weight rows per workgroup
     const int tid = (int)threadIdx.x, lane = tid & 63, ln = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int cols = g.b0.cols, n_out = g.b0.rows;
@@ -88,7 +89,7 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
     // A wavefront past the last block of weight rows repeats that block (and stores nothing): every wavefront
     // of the workgroup then runs the same control flow, which the barriers below rely on.
     const int proj = SPLIT ? (wave & 1) : 0;        // split: even wavefronts take gate rows, odd ones up rows
-    const int col_raw = ((int)blockIdx.x * kSkinnyWaves + (SPLIT ? wave >> 1 : wave)) * 32;
+    const int col_raw = ((int)blockIdx.x * CG + (SPLIT ? wave >> 1 : wave)) * 32;
     const int col_last = ((n_out - 1) >> 5) << 5;
     const int col0 = col_raw < n_out ? col_raw : col_last;
     const bool store_on = col_raw + ln < n_out;
@@ -346,7 +347,7 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
 }
 
 template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED>
-__global__ __launch_bounds__((GATE_UP ? 2 : 1) * kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArgs g) {
+__global__ __launch_bounds__(2 * kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArgs g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t skinny_lds[];
     Tile t;
     const uint32_t slot = blockIdx.y;
@@ -400,8 +401,9 @@ struct SkinnyLaunch {
             DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(150 * 1024)));
             allowed = 150 * 1024;
         }
-        dim3 grid((unsigned)ceil_div(g.b0.rows, kSkinnyWaves * 32), (unsigned)g.max_tiles);
-        dim3 block((GATE_UP ? 2 : 1) * kSkinnyWaves * 64);
+        // 8 wavefronts per workgroup: 128 output columns of gate AND up, or 256 of a single projection
+        dim3 grid((unsigned)ceil_div(g.b0.rows, (GATE_UP ? 1 : 2) * kSkinnyWaves * 32), (unsigned)g.max_tiles);
+        dim3 block(2 * kSkinnyWaves * 64);
         hipLaunchKernelGGL(kern, grid, block, lds, st, g);
         DMOE_LAUNCH_CHECK();
         return DMOE_OK;
