@@ -27,7 +27,7 @@ COPY_PROBE_BYTES = 256 << 20  # --copy-probe: bytes read (and written) by each c
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
 # (scaled by the same counters' reading for the --copy-probe copies; profiles/hbm_traffic_gemm_kernels.txt).
 # A counter cannot be read from inside the timed run, so these are the recorded values for the default workloads.
-MEASURED_TRAFFIC = {(1, "gate_up"): 1051430000, (1, "down"): 538685000,
+MEASURED_TRAFFIC = {(1, "gate_up"): 997250000, (1, "down"): 511455000,
                     (3, "gate_up"): 5182157000, (3, "down"): 2804555000}
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
@@ -161,12 +161,19 @@ def main():
     down_w = wl.down.nbytes() // wl.E
     kern = "gate_up" if stages["gate_up"] >= stages["down"] else "down"
     decode = rows <= 8 * wl.E   # the library's own rule for the small-M path (8 rows per resident expert on average)
+    # At decode sizes a shared expert of the routed experts' format rides in the routed launches as one more expert
+    # with T rows (the library's rule: small-M path, same shape / mode / bits / group): its weights and rows count.
+    sh = wl.shared
+    folded = decode and sh is not None and all(
+        (a.rows, a.cols, a.mode, a.bits, a.group_size) == (b.rows, b.cols, b.mode, b.bits, b.group_size)
+        for a, b in ((sh[0], wl.gate), (sh[1], wl.up), (sh[2], wl.down)))
+    k_experts, k_rows = U + (1 if folded else 0), rows + (wl.T if folded else 0)
     if kern == "gate_up":
-        k_bytes = U * gate_up_w + wl.T * wl.D * 2 + rows * wl.F * 2
-        k_flops = 2.0 * rows * 2 * wl.D * wl.F
+        k_bytes = k_experts * gate_up_w + wl.T * wl.D * 2 + k_rows * wl.F * 2
+        k_flops = 2.0 * k_rows * 2 * wl.D * wl.F
     else:
-        k_bytes = U * down_w + rows * wl.F * 2 + rows * wl.D * 2
-        k_flops = 2.0 * rows * wl.D * wl.F
+        k_bytes = k_experts * down_w + k_rows * wl.F * 2 + k_rows * wl.D * 2
+        k_flops = 2.0 * k_rows * wl.D * wl.F
     k_ms = stages[kern]
     if decode:
         achieved = k_bytes / (k_ms * 1e-3) / 1e9
@@ -179,7 +186,8 @@ def main():
     roof["traffic"] = MEASURED_TRAFFIC.get((args.config, kern))
     roof["measured_peaks"] = measured_peaks(torch)
     roof.update({"kernel": f"grouped {kern} GEMM ({'small-M' if decode else 'MFMA'} path)", "kernel_ms": k_ms,
-                 "algorithmic_bytes": k_bytes, "algorithmic_flops": k_flops, "live_experts": U})
+                 "algorithmic_bytes": k_bytes, "algorithmic_flops": k_flops, "live_experts": U,
+                 "shared_expert_in_launch": bool(folded)})
 
     step_bytes = U * wl.expert_bytes() + wl.shared_bytes() + 2 * wl.T * wl.D * 2 + wl.T * wl.E_total * 4 + rows * 8
     step_flops = wl.routed_flops() + wl.shared_flops()
