@@ -154,6 +154,9 @@ struct GemmArgs {
     int tile_m = 0;               // rows per tile the tile list (or the dense split) was built with
     int dense_rows = 0;
     float swiglu_limit = 0.0f;
+    // a launch serves the tiles with min_rows <= nrows <= max_rows of the list (prefill: the matrix-core kernels take the
+    // large tiles, the weight-streaming kernel the small ones)
+    int min_rows = 0, max_rows = 0x7fffffff;
     float swiglu_limit_dense = 0.0f;    // the limit for tiles flagged kTileDense
     uint32_t row_scale_rows = 0xffffffffu; // row_scale applies to sorted rows below this
 };

@@ -199,10 +199,18 @@ __global__ __launch_bounds__(kPackThreads) void pack_scan_kernel(PackOut o, uint
     const int tid = (int)threadIdx.x;
     uint32_t count = 0;
     if (tid < E) {
-        for (int sidx = 0; sidx < n_sub; ++sidx) {
-            uint32_t c = cnt[(size_t)sidx * E + tid];
-            cnt[(size_t)sidx * E + tid] = count;
-            count += c;
+        // exclusive scan down this expert's column of sub-chunk counts, eight independent loads at a time (one
+        // dependent load per sub-chunk made this loop the longest part of packing a prefill batch)
+        constexpr int kBatch = 8;
+        for (int s0 = 0; s0 < n_sub; s0 += kBatch) {
+            uint32_t c[kBatch];
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j) c[j] = s0 + j < n_sub ? cnt[(size_t)(s0 + j) * E + tid] : 0u;
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j) {
+                if (s0 + j < n_sub) cnt[(size_t)(s0 + j) * E + tid] = count;
+                count += c[j];
+            }
         }
     }
     uint32_t off = emit_segments(count, tid, E, n, tile_m, o, scan_sm);

@@ -355,6 +355,7 @@ __global__ __launch_bounds__(2 * kSkinnyWaves * 64) void qgemm_skinny_kernel(Gem
         const uint32_t n_tiles = *g.n_tiles; // both loads are issued before either is needed
         t = g.tiles[slot];                   // the list has room for every launched slot
         if (slot >= n_tiles) return;
+        if ((int)t.nrows > g.max_rows) return; // a list built for the matrix-core kernels: those take the larger tiles
     } else {
         t.expert = 0;
         t.flags = 0;
@@ -426,8 +427,8 @@ int launch_qgemm_skinny(const GemmArgs &g, hipStream_t st) {
     DMOE_REQUIRE(qgemm_skinny_supports(g.b0), "skinny GEMM: unsupported weight shape (cols=%d)", g.b0.cols);
     DMOE_REQUIRE(g.max_tiles >= 0 && g.max_tiles <= 65535, "skinny GEMM: %d tiles exceed the grid limit", g.max_tiles);
     DMOE_REQUIRE(g.a && g.out && g.ldo > 0 && ((uintptr_t)g.a % 16) == 0, "skinny GEMM: bad pointer");
-    DMOE_REQUIRE(g.tile_m > 0 && g.tile_m <= qgemm_skinny_tile_m(g.b0), "skinny GEMM: tiles of %d rows, this shape takes %d",
-                 g.tile_m, qgemm_skinny_tile_m(g.b0));
+    DMOE_REQUIRE(g.tile_m > 0 && std::min(g.tile_m, g.max_rows) <= qgemm_skinny_tile_m(g.b0),
+                 "skinny GEMM: tiles of %d rows, this shape takes %d", std::min(g.tile_m, g.max_rows), qgemm_skinny_tile_m(g.b0));
     if (g.gate_up)
         DMOE_REQUIRE(g.b1.rows == g.b0.rows && g.b1.cols == g.b0.cols && g.b1.mode == g.b0.mode &&
                          g.b1.bits == g.b0.bits && g.b1.group == g.b0.group && g.b1.packed == g.b0.packed,

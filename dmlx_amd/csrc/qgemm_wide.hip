@@ -278,6 +278,7 @@ __global__ __launch_bounds__(kWideWaves * 64) void qgemm_wide_kernel(GemmArgs g)
         const uint32_t n_tiles = *g.n_tiles;
         t = g.tiles[slot];
         if (slot >= n_tiles) return;
+        if ((int)t.nrows < g.min_rows) return; // left to the weight-streaming kernel
     } else {
         t.expert = 0;
         t.row0 = slot * (uint32_t)g.tile_m;

@@ -63,6 +63,7 @@ def test_dequantize_bit_exact(dmoe, orc, fmt):
                                                 (130, 1, 128, 2048),    # single expert, MFMA, partial tile
                                                 (700, 4, 256, 384),     # reduction not a multiple of the pipeline depth
                                                 (1200, 2, 192, 640),    # 256-row tiles, idle wavefronts in the last strip
+                                                (900, 12, 256, 2048),   # MFMA path for the large tiles + weight-streaming kernel for the small ones
                                                 (60, 8, 256, 2048),     # small-M path, some experts above 8 rows (restaged tiles)
                                                 (30, 4, 192, 2048)])    # same, weight rows not a multiple of the workgroup's
 def test_gather_qmm_matches_oracle(dmoe, orc, ws, fmt, R, n_mats, rows, cols):
