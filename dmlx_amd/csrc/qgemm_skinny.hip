@@ -66,19 +66,20 @@ struct SkinnyStage {
 // tiles (16 accumulators; a tile of two row blocks computes four, the surplus rows are never stored). The kernel
 // calls one or the other right after fetching the tile, so the two share nothing but the arguments and each keeps
 // its own register allocation.
-template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED, int RJT>
-__device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, uint8_t *skinny_lds) {
+// `gate_up` (workgroup-uniform) is the role of the launch: gate and up projections with SwiGLU (their rows on
+// separate wavefronts, paired through LDS at the end), or a single projection.
+template <typename Fmt, bool FACTORED, bool PACKED, int RJT>
+__device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, uint8_t *skinny_lds, const bool gate_up) {
     using CS = ChunkStream<Fmt, PACKED>;
     constexpr int KV = Fmt::kVals;   // values per 16-byte chunk
     constexpr int KSTEP = 2 * KV;    // reduction elements per step (both lane halves)
     constexpr int NJ = KV / 8;       // MFMAs (K = 16) per step
-    constexpr bool SPLIT = GATE_UP;                 // gate and up rows on separate wavefronts
     // depth of the weight ring: the large-tile copy keeps 16 accumulators per lane and takes a shallower ring to
     // stay inside the same register budget (span boundaries stay whole ring rounds either way)
     constexpr int STAGES = RJT == 1 ? kSkinnyStages : kSkinnyStages / 2;
-    constexpr int NM = GATE_UP && !SPLIT ? 2 : 1;   // projections per wavefront
+    constexpr int NM = 1;                           // projections per wavefront
     constexpr int WAVES = 2 * kSkinnyWaves;         // eight wavefronts share one staging of the tile's activations
-    constexpr int CG = SPLIT ? kSkinnyWaves : WAVES; // 32-row blocks of weight rows per workgroup
+    const int cg = gate_up ? kSkinnyWaves : WAVES;  // 32-row blocks of weight rows per workgroup
     const int tid = (int)threadIdx.x, lane = tid & 63, ln = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int cols = g.b0.cols, n_out = g.b0.rows;
@@ -88,8 +89,9 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
     // ---- this lane's weight row ------------------------------------------------------------------------
     // A wavefront past the last block of weight rows repeats that block (and stores nothing): every wavefront
     // of the workgroup then runs the same control flow, which the barriers below rely on.
-    const int proj = SPLIT ? (wave & 1) : 0;        // split: even wavefronts take gate rows, odd ones up rows
-    const int col_raw = ((int)blockIdx.x * CG + (SPLIT ? wave >> 1 : wave)) * 32;
+    const int proj = gate_up ? (wave & 1) : 0;      // gate/up: even wavefronts take gate rows, odd ones up rows
+    const int col_raw = ((int)blockIdx.x * cg + (gate_up ? wave >> 1 : wave)) * 32;
+    const QView &qv = proj ? g.b1 : g.b0;           // this wavefront's matrix stack
     const int col_last = ((n_out - 1) >> 5) << 5;
     const int col0 = col_raw < n_out ? col_raw : col_last;
     const bool store_on = col_raw + ln < n_out;
@@ -97,12 +99,12 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
     if (n >= n_out) n = n_out - 1; // stay inside the matrix; such rows are never stored
     CS cs[NM];
 #pragma unroll
-    for (int mi = 0; mi < NM; ++mi) cs[mi].init((mi + proj) == 0 ? g.b0 : g.b1, e, col0 >> 5, ln, h, n);
+    for (int mi = 0; mi < NM; ++mi) cs[mi].init(qv, e, col0 >> 5, ln, h, n);
     auto load_stage = [&](int step, SkinnyStage<NM> &s) {
 #pragma unroll
         for (int mi = 0; mi < NM; ++mi) {
             s.raw[mi] = cs[mi].load_chunk_stream(step);
-            cs[mi].load_meta((mi + proj) == 0 ? g.b0 : g.b1, step, s.sb[mi]);
+            cs[mi].load_meta(qv, step, s.sb[mi]);
         }
     };
 
@@ -306,12 +308,11 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
         float v[2][4 * RJT];
 #pragma unroll
         for (int mi = 0; mi < NM; ++mi) {
-            const QView &q = (mi + proj) == 0 ? g.b0 : g.b1;
-            const float rs = Fmt::kRowScale ? *(const float *)(q.scales + e * q.s_mat + (size_t)n * q.s_row) : 1.0f;
+            const float rs = Fmt::kRowScale ? *(const float *)(qv.scales + e * qv.s_mat + (size_t)n * qv.s_row) : 1.0f;
 #pragma unroll
             for (int r = 0; r < 4 * RJT; ++r) v[mi][r] = (FACTORED ? facc[mi][r] : acc[mi][r]) * rs;
         }
-        if (SPLIT) {
+        if (gate_up) {
             // the up wavefront hands its values to the gate wavefront of the same weight rows, through the
             // activation window (free once every wavefront has left the main loop)
             float4 *xch = (float4 *)xs_lds + ((wave >> 1) * 64 + lane) * RJT;
@@ -337,7 +338,7 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
                 const int i = 8 * j + 4 * h + r;
                 if (i >= nrows) continue;
                 const uint32_t p = t.row0 + (uint32_t)i;
-                float val = GATE_UP ? limited_swiglu(v[0][4 * j + r], v[1][4 * j + r], swiglu_limit) : v[0][4 * j + r];
+                float val = gate_up ? limited_swiglu(v[0][4 * j + r], v[1][4 * j + r], swiglu_limit) : v[0][4 * j + r];
                 if (g.row_scale && p < g.row_scale_rows) val *= g.row_scale[g.row_scale_idx ? g.row_scale_idx[p] : p];
                 const size_t dst = g.out_rows ? g.out_rows[p] : p;
                 g.out[dst * (size_t)g.ldo + n] = f32_to_bf16_bits(val);
@@ -346,7 +347,7 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
     }
 }
 
-template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED>
+template <typename Fmt, bool FACTORED, bool PACKED>
 __global__ __launch_bounds__(2 * kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArgs g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t skinny_lds[];
     Tile t;
@@ -364,8 +365,8 @@ __global__ __launch_bounds__(2 * kSkinnyWaves * 64) void qgemm_skinny_kernel(Gem
         uint32_t left = (uint32_t)g.dense_rows - t.row0;
         t.nrows = left < (uint32_t)g.tile_m ? left : (uint32_t)g.tile_m;
     }
-    if (__builtin_amdgcn_readfirstlane((int)t.nrows) <= kSkinnyRowBlock) skinny_tile<Fmt, GATE_UP, FACTORED, PACKED, 1>(g, t, skinny_lds);
-    else skinny_tile<Fmt, GATE_UP, FACTORED, PACKED, kSkinnyTileM / kSkinnyRowBlock>(g, t, skinny_lds);
+    if (__builtin_amdgcn_readfirstlane((int)t.nrows) <= kSkinnyRowBlock) skinny_tile<Fmt, FACTORED, PACKED, 1>(g, t, skinny_lds, g.gate_up);
+    else skinny_tile<Fmt, FACTORED, PACKED, kSkinnyTileM / kSkinnyRowBlock>(g, t, skinny_lds, g.gate_up);
 }
 
 static int skinny_vals(const QView &b) {
@@ -393,9 +394,9 @@ bool qgemm_skinny_supports(const QView &b) {
 struct SkinnyLaunch {
     const GemmArgs &g;
     hipStream_t st;
-    template <typename Fmt, bool GATE_UP, bool FACTORED, bool PACKED>
+    template <typename Fmt, bool FACTORED, bool PACKED>
     int go() {
-        auto kern = qgemm_skinny_kernel<Fmt, GATE_UP, FACTORED, PACKED>;
+        auto kern = qgemm_skinny_kernel<Fmt, FACTORED, PACKED>;
         const size_t lds = skinny_lds_bytes(g.b0);
         static thread_local size_t allowed = 0; // per instantiation: raise the dynamic LDS limit once
         if (lds > allowed) {
@@ -403,7 +404,7 @@ struct SkinnyLaunch {
             allowed = 150 * 1024;
         }
         // 8 wavefronts per workgroup: 128 output columns of gate AND up, or 256 of a single projection
-        dim3 grid((unsigned)ceil_div(g.b0.rows, (GATE_UP ? 1 : 2) * kSkinnyWaves * 32), (unsigned)g.max_tiles);
+        dim3 grid((unsigned)ceil_div(g.b0.rows, (g.gate_up ? 1 : 2) * kSkinnyWaves * 32), (unsigned)g.max_tiles);
         dim3 block(2 * kSkinnyWaves * 64);
         hipLaunchKernelGGL(kern, grid, block, lds, st, g);
         DMOE_LAUNCH_CHECK();
@@ -414,12 +415,8 @@ struct SkinnyLaunch {
         // the scale can be factored out of the matrix product when both halves of a step share a group
         constexpr bool can_factor = std::is_same<Fmt, FmtAffine4>::value;
         const bool factor = can_factor && g.b0.group >= 64;
-        if (g.b0.packed) {
-            if (factor) return g.gate_up ? go<Fmt, true, can_factor, true>() : go<Fmt, false, can_factor, true>();
-            return g.gate_up ? go<Fmt, true, false, true>() : go<Fmt, false, false, true>();
-        }
-        if (factor) return g.gate_up ? go<Fmt, true, can_factor, false>() : go<Fmt, false, can_factor, false>();
-        return g.gate_up ? go<Fmt, true, false, false>() : go<Fmt, false, false, false>();
+        if (g.b0.packed) return factor ? go<Fmt, can_factor, true>() : go<Fmt, false, true>();
+        return factor ? go<Fmt, can_factor, false>() : go<Fmt, false, false>();
     }
 };
 
