@@ -27,7 +27,7 @@ COPY_PROBE_BYTES = 256 << 20  # --copy-probe: bytes read (and written) by each c
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
 # (scaled by the same counters' reading for the --copy-probe copies; profiles/hbm_traffic_gemm_kernels.txt).
 # A counter cannot be read from inside the timed run, so these are the recorded values for the default workloads.
-MEASURED_TRAFFIC = {(1, "gate_up"): 997250000, (1, "down"): 511455000,
+MEASURED_TRAFFIC = {(1, "gate_up+down"): 1509859000,
                     (3, "gate_up"): 5204994000, (3, "down"): 2859303000}
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
@@ -168,13 +168,20 @@ def main():
         (a.rows, a.cols, a.mode, a.bits, a.group_size) == (b.rows, b.cols, b.mode, b.bits, b.group_size)
         for a, b in ((sh[0], wl.gate), (sh[1], wl.up), (sh[2], wl.down)))
     k_experts, k_rows = U + (1 if folded else 0), rows + (wl.T if folded else 0)
-    if kern == "gate_up":
-        k_bytes = k_experts * gate_up_w + wl.T * wl.D * 2 + k_rows * wl.F * 2
-        k_flops = 2.0 * k_rows * 2 * wl.D * wl.F
+    gu_bytes = k_experts * gate_up_w + wl.T * wl.D * 2 + k_rows * wl.F * 2
+    dn_bytes = k_experts * down_w + k_rows * wl.F * 2 + k_rows * wl.D * 2
+    gu_flops, dn_flops = 2.0 * k_rows * 2 * wl.D * wl.F, 2.0 * k_rows * wl.D * wl.F
+    # decode steps run both GEMMs as ONE launch (a down workgroup waits for its own tile's gate/up workgroups): the
+    # library then reports the launch under the gate/up stage and nothing under down
+    paired = decode and stages["down"] == 0.0
+    if paired:
+        # the intermediate h ([rows, F], written by one half of the launch and read by the other) is not algorithmic traffic
+        kern, k_bytes, k_flops = "gate_up+down", gu_bytes + dn_bytes - 2 * k_rows * wl.F * 2, gu_flops + dn_flops
+    elif kern == "gate_up":
+        k_bytes, k_flops = gu_bytes, gu_flops
     else:
-        k_bytes = k_experts * down_w + k_rows * wl.F * 2 + k_rows * wl.D * 2
-        k_flops = 2.0 * k_rows * wl.D * wl.F
-    k_ms = stages[kern]
+        k_bytes, k_flops = dn_bytes, dn_flops
+    k_ms = stages["gate_up"] if paired else stages[kern]
     if decode:
         achieved = k_bytes / (k_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -187,7 +194,7 @@ def main():
     roof["measured_peaks"] = measured_peaks(torch)
     # prefill with packed 4-bit weights: the stage is two launches on one tile list (matrix-core kernel for the tiles
     # above 32 rows, weight-streaming kernel for the rest); kernel_ms is the stage, the sum of the two
-    launches = (["qgemm_skinny_kernel"] if decode else
+    launches = (["qgemm_skinny_kernel (gate/up and down tiles in one launch)"] if paired else ["qgemm_skinny_kernel"] if decode else
                 ["qgemm_wide_kernel", "qgemm_skinny_kernel"] if wl.gate.mode in (0, 1) and wl.gate.bits == 4 else ["qgemm_mfma_kernel"])
     roof.update({"kernel": f"grouped {kern} GEMM ({'small-M' if decode else 'MFMA'} path)", "launches": launches, "kernel_ms": k_ms,
                  "algorithmic_bytes": k_bytes, "algorithmic_flops": k_flops, "live_experts": U,

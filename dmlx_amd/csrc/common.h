@@ -102,6 +102,9 @@ struct PackOut {
     // (row n+t = token t) of matrix `dense_expert`, cut into tiles of `tile_m` rows that come FIRST in the list,
     // flagged kTileDense. order / token / sorted_e then hold n + dense_rows entries.
     uint32_t dense_rows = 0, dense_expert = 0;
+    // optional per-tile completion counters (n_done of them), zeroed by the pack kernels: see GemmArgs::tile_done
+    uint32_t *tile_done = nullptr;
+    uint32_t n_done = 0;
 };
 
 inline int pack_max_tiles(size_t n, int E, int tile_m) {
@@ -157,6 +160,10 @@ struct GemmArgs {
     // a launch serves the tiles with min_rows <= nrows <= max_rows of the list (prefill: the matrix-core kernels take the
     // large tiles, the weight-streaming kernel the small ones)
     int min_rows = 0, max_rows = 0x7fffffff;
+    // Paired launch (gate/up and down of a decode step in ONE launch): the workgroups of a gate/up tile add 1 to
+    // tile_done[tile] after their stores, a down workgroup of that tile waits for tile_done_target before it reads h.
+    uint32_t *tile_done = nullptr;
+    uint32_t tile_done_target = 0;
     float swiglu_limit_dense = 0.0f;    // the limit for tiles flagged kTileDense
     uint32_t row_scale_rows = 0xffffffffu; // row_scale applies to sorted rows below this
 };
@@ -166,6 +173,9 @@ constexpr int kSkinnyDenseTileM = 8;      // dense (one matrix) launches: small 
 constexpr int kMfmaTileM = 128;
 constexpr int kMfmaWideTileM = 256;
 int launch_qgemm_skinny(const GemmArgs &g, hipStream_t st);
+// gate/up + down of one tile list in one launch (down waits per tile for gate/up); gu.tile_done must be zeroed
+bool qgemm_skinny_pair_supports(const GemmArgs &gu, const GemmArgs &dn);
+int launch_qgemm_skinny_pair(const GemmArgs &gu, const GemmArgs &dn, hipStream_t st);
 int launch_qgemm_mfma(const GemmArgs &g, hipStream_t st); // picks the wide kernel when the format allows it
 int launch_qgemm_wide(const GemmArgs &g, hipStream_t st);
 bool qgemm_skinny_supports(const QView &b);

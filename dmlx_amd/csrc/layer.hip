@@ -180,7 +180,7 @@ static bool use_small_path(size_t rows, int n_experts, const QView &b) {
     return qgemm_skinny_supports(b) && rows <= (size_t)kSkinnyAvgRows * (size_t)n_experts;
 }
 struct FwdLayout {
-    size_t slot_idx, order, inv, token, sorted_e, counts, offsets, live, n_live, tiles, n_tiles, scratch;
+    size_t slot_idx, order, inv, token, sorted_e, counts, offsets, live, n_live, tiles, n_tiles, tile_done, scratch;
     size_t h, y, sh_h, sh_y, total;
     int max_tiles, tile_m;
     bool small;
@@ -209,6 +209,7 @@ static FwdLayout forward_layout(const Layer *L, int T, bool with_shared = true) 
     f.n_live = b.take(4);
     f.tiles = b.take((size_t)(f.max_tiles > 0 ? f.max_tiles : 1) * sizeof(Tile));
     f.n_tiles = b.take(4);
+    f.tile_done = b.take(f.small ? (size_t)(f.max_tiles > 0 ? f.max_tiles : 1) * 4 : 0);
     f.scratch = b.take(pack_scratch_bytes(n, L->E));
     f.h = b.take(rows * (size_t)L->F * 2);
     f.y = b.take(rows * (size_t)L->D * 2);
@@ -257,6 +258,10 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
         po.dense_rows = (uint32_t)T;
         po.dense_expert = (uint32_t)L->E;
     }
+    if (f.small) { // per-tile completion counters of the paired gate/up + down launch, zeroed with the tile list
+        po.tile_done = at<uint32_t>(w, f.tile_done);
+        po.n_done = (uint32_t)f.max_tiles;
+    }
     DMOE_TRY(launch_pack(po, d_slots, n, L->K, L->E, f.tile_m, at<void>(w, f.scratch), st));
     DMOE_TRY(stage_end(w, DMOE_STAGE_PACK, st));
 
@@ -279,11 +284,6 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
         gu.row_scale_idx = po.order;
         gu.row_scale_rows = (uint32_t)n; // the folded shared expert's rows carry no routing weight
     }
-    const int small_rows = f.small ? 0 : prefill_small_rows(L->gate.view, L->down.view);
-    DMOE_TRY(stage_begin(w, DMOE_STAGE_GATE_UP, st));
-    DMOE_TRY(run_gemm(gu, f.small, st, small_rows));
-    DMOE_TRY(stage_end(w, DMOE_STAGE_GATE_UP, st));
-
     GemmArgs dn;
     dn.b0 = L->down.view;
     dn.a = at<uint16_t>(w, f.h);
@@ -294,6 +294,20 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     dn.n_tiles = po.n_tiles;
     dn.max_tiles = f.max_tiles;
     dn.tile_m = f.tile_m;
+
+    // Decode sizes: both GEMMs in one launch; a down workgroup waits for its own tile's gate/up workgroups only, so
+    // the down projection fills the chip while the last gate/up workgroups drain (timed as the gate/up stage).
+    gu.tile_done = po.tile_done;
+    if (f.small && qgemm_skinny_pair_supports(gu, dn)) {
+        DMOE_TRY(stage_begin(w, DMOE_STAGE_GATE_UP, st));
+        DMOE_TRY(launch_qgemm_skinny_pair(gu, dn, st));
+        DMOE_TRY(stage_end(w, DMOE_STAGE_GATE_UP, st));
+        return DMOE_OK;
+    }
+    const int small_rows = f.small ? 0 : prefill_small_rows(L->gate.view, L->down.view);
+    DMOE_TRY(stage_begin(w, DMOE_STAGE_GATE_UP, st));
+    DMOE_TRY(run_gemm(gu, f.small, st, small_rows));
+    DMOE_TRY(stage_end(w, DMOE_STAGE_GATE_UP, st));
     DMOE_TRY(stage_begin(w, DMOE_STAGE_DOWN, st));
     DMOE_TRY(run_gemm(dn, f.small, st, small_rows));
     DMOE_TRY(stage_end(w, DMOE_STAGE_DOWN, st));

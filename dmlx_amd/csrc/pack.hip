@@ -79,6 +79,7 @@ __device__ uint32_t emit_segments(uint32_t count, int e, int E, size_t n, int ti
         if (count > 0 && o.live) o.live[lb] = (uint32_t)e;
         if (e == 0 && o.n_live) *o.n_live = lt;
     }
+    for (uint32_t i = threadIdx.x; i < o.n_done; i += blockDim.x) o.tile_done[i] = 0;
     // the folded always-on expert: identity rows behind the routed ones, its tiles ahead of the routed tiles
     const uint32_t dense_m = tile_m > 0 ? (uint32_t)tile_m : 1u;
     const uint32_t nt_dense = (o.dense_rows + dense_m - 1) / dense_m;

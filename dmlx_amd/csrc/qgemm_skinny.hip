@@ -68,8 +68,15 @@ struct SkinnyStage {
 // its own register allocation.
 // `gate_up` (workgroup-uniform) is the role of the launch: gate and up projections with SwiGLU (their rows on
 // separate wavefronts, paired through LDS at the end), or a single projection.
+// `sync` (paired launch, workgroup-uniform): kSkinnySyncSignal = every workgroup of the tile adds 1 to
+// g.tile_done[slot] once its stores have reached memory; kSkinnySyncWait = the workgroup waits for g.tile_done[slot] to
+// reach g.tile_done_target before it reads its activations (the other role's output), its weight ring already in flight.
+constexpr int kSkinnySyncNone = 0, kSkinnySyncSignal = 1, kSkinnySyncWait = 2;
+constexpr uint32_t kSkinnySpinLimit = 1u << 16; // polls of ~0.25 us: the wait ends after ~16 ms whatever happens
+
 template <typename Fmt, bool FACTORED, bool PACKED, int RJT>
-__device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, uint8_t *skinny_lds, const bool gate_up) {
+__device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, uint8_t *skinny_lds, const bool gate_up,
+                                            const int sync, const uint32_t slot) {
     using CS = ChunkStream<Fmt, PACKED>;
     constexpr int KV = Fmt::kVals;   // values per 16-byte chunk
     constexpr int KSTEP = 2 * KV;    // reduction elements per step (both lane halves)
@@ -136,8 +143,14 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
             const size_t src = (uint32_t)__builtin_amdgcn_readlane((int)src_of_lane, r);
             const uint8_t *gp = (const uint8_t *)(g.a + src * (size_t)cols) + (size_t)span * span_bytes + c + lane * 16;
             const uint32_t la = lds_addr + (uint32_t)(r * pitch + c); // uniform; lane i lands at la + 16 i
-            if (c + lane * 16 < span_bytes)
-                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gp), "s"(la) : "memory"); // nothing else in this kernel uses M0
+            if (c + lane * 16 < span_bytes) {
+                // nothing else in this kernel uses M0. A waiting consumer reads rows that workgroups on other XCDs
+                // have just written with device-scope stores: its loads go past this XCD's L2 (sc1), no fence needed.
+                if (sync == kSkinnySyncWait)
+                    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off sc1" : : "v"(gp), "s"(la) : "memory");
+                else
+                    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gp), "s"(la) : "memory");
+            }
         }
     };
     // factored form: per 16-byte piece (x0..x7) -> (x0,x4,x1,x5,x2,x6,x3,x7), the order the code pairs come out
@@ -165,18 +178,39 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
         }
     };
 
-    // Loads return in issue order: the first span is requested ahead of the first stages of the weight ring, and
-    // the wait below lets the ring stay in flight.
-    issue_x(0);
     SkinnyStage<NM> ring[STAGES];
+    if (sync == kSkinnySyncWait) {
+        // the activations are still being written: start the weight ring, then wait for the tile's producers (one
+        // wavefront polls, the barrier holds the others), then fetch the rows
 #pragma unroll
-    for (int mi = 0; mi < NM; ++mi) cs[mi].pin(); // keeps the weight loads behind the requests above
+        for (int j = 0; j < STAGES - 1; ++j)
+            if (j < n_steps) load_stage(j, ring[j]);
+        if (wave == 0) {
+            uint32_t polls = 0;
+            while (__hip_atomic_load(&g.tile_done[slot], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < g.tile_done_target &&
+                   polls < kSkinnySpinLimit) {
+                __builtin_amdgcn_s_sleep(8);
+                ++polls;
+            }
+        }
+        __syncthreads();
 #pragma unroll
-    for (int j = 0; j < STAGES - 1; ++j)
-        if (j < n_steps) load_stage(j, ring[j]);
-    // every ring stage holds at least NM loads younger than the activation requests
-    if (n_steps >= STAGES - 1) __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt((STAGES - 1) * NM));
-    else __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt(0));
+        for (int mi = 0; mi < NM; ++mi) cs[mi].pin();
+        issue_x(0);
+        __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt(0));
+    } else {
+        // Loads return in issue order: the first span is requested ahead of the first stages of the weight ring, and
+        // the wait below lets the ring stay in flight.
+        issue_x(0);
+#pragma unroll
+        for (int mi = 0; mi < NM; ++mi) cs[mi].pin(); // keeps the weight loads behind the requests above
+#pragma unroll
+        for (int j = 0; j < STAGES - 1; ++j)
+            if (j < n_steps) load_stage(j, ring[j]);
+        // every ring stage holds at least NM loads younger than the activation requests
+        if (n_steps >= STAGES - 1) __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt((STAGES - 1) * NM));
+        else __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt(0));
+    }
     __syncthreads();
     if (FACTORED) {
         fix_x();
@@ -322,36 +356,63 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
                 for (int j = 0; j < RJT; ++j) xch[j] = make_float4(v[0][4 * j], v[0][4 * j + 1], v[0][4 * j + 2], v[0][4 * j + 3]);
             }
             __syncthreads();
-            if (proj == 1) return;
+            if (proj == 0) {
 #pragma unroll
-            for (int j = 0; j < RJT; ++j) {
-                const float4 u = xch[j];
-                v[1][4 * j] = u.x, v[1][4 * j + 1] = u.y, v[1][4 * j + 2] = u.z, v[1][4 * j + 3] = u.w;
+                for (int j = 0; j < RJT; ++j) {
+                    const float4 u = xch[j];
+                    v[1][4 * j] = u.x, v[1][4 * j + 1] = u.y, v[1][4 * j + 2] = u.z, v[1][4 * j + 3] = u.w;
+                }
             }
         }
-        if (!store_on) return;
+        const bool storer = store_on && proj == 0;
         const float swiglu_limit = (t.flags & kTileDense) ? g.swiglu_limit_dense : g.swiglu_limit;
 #pragma unroll
         for (int j = 0; j < RJT; ++j) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int i = 8 * j + 4 * h + r;
-                if (i >= nrows) continue;
+                if (!storer || i >= nrows) continue;
                 const uint32_t p = t.row0 + (uint32_t)i;
                 float val = gate_up ? limited_swiglu(v[0][4 * j + r], v[1][4 * j + r], swiglu_limit) : v[0][4 * j + r];
                 if (g.row_scale && p < g.row_scale_rows) val *= g.row_scale[g.row_scale_idx ? g.row_scale_idx[p] : p];
                 const size_t dst = g.out_rows ? g.out_rows[p] : p;
-                g.out[dst * (size_t)g.ldo + n] = f32_to_bf16_bits(val);
+                // a producer's rows are read by workgroups on other XCDs within the same launch: device-scope
+                // stores (written through this XCD's L2), so no cache-wide write-back is needed before the signal
+                if (sync == kSkinnySyncSignal)
+                    __hip_atomic_store(&g.out[dst * (size_t)g.ldo + n], f32_to_bf16_bits(val), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                else
+                    g.out[dst * (size_t)g.ldo + n] = f32_to_bf16_bits(val);
             }
+        }
+        if (sync == kSkinnySyncSignal) {
+            __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt(0)); // this wavefront's stores have reached memory ...
+            __syncthreads();                                   // ... and every other wavefront's of the workgroup ...
+            if (tid == 0) __hip_atomic_fetch_add(&g.tile_done[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); // ... before this
         }
     }
 }
 
+// `paired` = 0: one GEMM (`a`). `paired` = 1: gate/up (`a`) and down (`b`) of one tile list in one launch: workgroups
+// y < a.max_tiles are the gate/up tiles, the next a.max_tiles the down tiles of the same list. The hardware starts
+// workgroups in index order, so every producer of a tile is running or done by the time a consumer of it starts to
+// wait; the down workgroups that become resident while the last gate/up workgroups drain stream their weights meanwhile.
 template <typename Fmt, bool FACTORED, bool PACKED>
-__global__ __launch_bounds__(2 * kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArgs g) {
+__global__ __launch_bounds__(2 * kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArgs a, GemmArgs b, int paired) {
     extern __shared__ __attribute__((aligned(16))) uint8_t skinny_lds[];
+    const bool second = paired && blockIdx.y >= (uint32_t)a.max_tiles; // workgroup-uniform
+    // The role's arguments, read from the kernel-argument segment with a uniform index (`a` sits at offset 0 and `b`
+    // right behind it): taking the address of `a` or `b` instead would move both structs to scratch memory.
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef const __attribute__((address_space(4))) GemmArgs *KernArgs;
+    const GemmArgs g = ((KernArgs)__builtin_amdgcn_kernarg_segment_ptr())[second ? 1 : 0];
+#else
+    const GemmArgs g = a; // host pass of the compiler: never runs
+#endif
+    (void)b;
+    const uint32_t slot = blockIdx.y - (second ? (uint32_t)a.max_tiles : 0u);
+    const int sync = !paired ? kSkinnySyncNone : second ? kSkinnySyncWait : kSkinnySyncSignal;
+    if ((int)blockIdx.x * (g.gate_up ? 1 : 2) * kSkinnyWaves * 32 >= g.b0.rows) return; // the grid is sized for the wider role
     Tile t;
-    const uint32_t slot = blockIdx.y;
     if (g.tiles) {
         const uint32_t n_tiles = *g.n_tiles; // both loads are issued before either is needed
         t = g.tiles[slot];                   // the list has room for every launched slot
@@ -365,8 +426,10 @@ __global__ __launch_bounds__(2 * kSkinnyWaves * 64) void qgemm_skinny_kernel(Gem
         uint32_t left = (uint32_t)g.dense_rows - t.row0;
         t.nrows = left < (uint32_t)g.tile_m ? left : (uint32_t)g.tile_m;
     }
-    if (__builtin_amdgcn_readfirstlane((int)t.nrows) <= kSkinnyRowBlock) skinny_tile<Fmt, FACTORED, PACKED, 1>(g, t, skinny_lds, g.gate_up);
-    else skinny_tile<Fmt, FACTORED, PACKED, kSkinnyTileM / kSkinnyRowBlock>(g, t, skinny_lds, g.gate_up);
+    if (__builtin_amdgcn_readfirstlane((int)t.nrows) <= kSkinnyRowBlock)
+        skinny_tile<Fmt, FACTORED, PACKED, 1>(g, t, skinny_lds, g.gate_up, sync, slot);
+    else
+        skinny_tile<Fmt, FACTORED, PACKED, kSkinnyTileM / kSkinnyRowBlock>(g, t, skinny_lds, g.gate_up, sync, slot);
 }
 
 static int skinny_vals(const QView &b) {
@@ -394,6 +457,7 @@ bool qgemm_skinny_supports(const QView &b) {
 struct SkinnyLaunch {
     const GemmArgs &g;
     hipStream_t st;
+    const GemmArgs *second = nullptr; // paired launch: the down projection behind the gate/up GEMM `g`
     template <typename Fmt, bool FACTORED, bool PACKED>
     int go() {
         auto kern = qgemm_skinny_kernel<Fmt, FACTORED, PACKED>;
@@ -404,9 +468,19 @@ struct SkinnyLaunch {
             allowed = 150 * 1024;
         }
         // 8 wavefronts per workgroup: 128 output columns of gate AND up, or 256 of a single projection
-        dim3 grid((unsigned)ceil_div(g.b0.rows, (g.gate_up ? 1 : 2) * kSkinnyWaves * 32), (unsigned)g.max_tiles);
+        auto blocks_x = [](const GemmArgs &a) { return ceil_div(a.b0.rows, (a.gate_up ? 1 : 2) * kSkinnyWaves * 32); };
         dim3 block(2 * kSkinnyWaves * 64);
-        hipLaunchKernelGGL(kern, grid, block, lds, st, g);
+        if (second) {
+            GemmArgs a = g, b = *second;
+            a.tile_done_target = b.tile_done_target = (uint32_t)blocks_x(g);
+            b.tile_done = a.tile_done;
+            const size_t lds2 = std::max(lds, skinny_lds_bytes(second->b0));
+            dim3 grid((unsigned)std::max(blocks_x(a), blocks_x(b)), (unsigned)(2 * g.max_tiles));
+            hipLaunchKernelGGL(kern, grid, block, lds2, st, a, b, 1);
+        } else {
+            dim3 grid((unsigned)blocks_x(g), (unsigned)g.max_tiles);
+            hipLaunchKernelGGL(kern, grid, block, lds, st, g, g, 0);
+        }
         DMOE_LAUNCH_CHECK();
         return DMOE_OK;
     }
@@ -419,6 +493,28 @@ struct SkinnyLaunch {
         return factor ? go<Fmt, can_factor, false>() : go<Fmt, false, false>();
     }
 };
+
+static bool skinny_factored(const QView &b) { return b.mode == DMOE_QUANT_AFFINE && b.bits == 4 && b.group >= 64; }
+
+bool qgemm_skinny_pair_supports(const GemmArgs &gu, const GemmArgs &dn) {
+    const QView &a = gu.b0, &b = dn.b0;
+    return gu.gate_up && !dn.gate_up && gu.tiles && gu.tiles == dn.tiles && gu.n_tiles == dn.n_tiles &&
+           gu.max_tiles == dn.max_tiles && gu.max_tiles > 0 && 2 * (long)gu.max_tiles <= 65535 &&
+           a.packed == b.packed && a.mode == b.mode && a.bits == b.bits && skinny_factored(a) == skinny_factored(b) &&
+           qgemm_skinny_supports(a) && qgemm_skinny_supports(b) && gu.tile_m <= qgemm_skinny_tile_m(a) &&
+           dn.tile_m <= qgemm_skinny_tile_m(b) && gu.tile_done != nullptr && dn.a == gu.out;
+}
+
+int launch_qgemm_skinny_pair(const GemmArgs &gu, const GemmArgs &dn, hipStream_t st) {
+    DMOE_REQUIRE(qgemm_skinny_pair_supports(gu, dn), "skinny GEMM pair: arguments do not form a gate/up + down pair");
+    DMOE_REQUIRE(gu.a && gu.out && dn.out && ((uintptr_t)gu.a % 16) == 0 && ((uintptr_t)dn.a % 16) == 0, "skinny GEMM pair: bad pointer");
+    DMOE_REQUIRE(gu.b1.rows == gu.b0.rows && gu.b1.cols == gu.b0.cols && gu.b1.mode == gu.b0.mode && gu.b1.bits == gu.b0.bits &&
+                     gu.b1.group == gu.b0.group && gu.b1.packed == gu.b0.packed,
+                 "skinny GEMM pair: gate and up projections differ in shape or format");
+    SkinnyLaunch l{gu, st};
+    l.second = &dn;
+    return dispatch_format(gu.b0, l);
+}
 
 int launch_qgemm_skinny(const GemmArgs &g, hipStream_t st) {
     DMOE_REQUIRE(qgemm_skinny_supports(g.b0), "skinny GEMM: unsupported weight shape (cols=%d)", g.b0.cols);

@@ -42,3 +42,23 @@ def test_layer_step_replays_bit_identically(dmoe, ws, config, scale):
         eager = step(x)                                      # eager work between the replays
         torch.cuda.synchronize()
         assert torch.equal(eager, want)
+
+
+@pytest.mark.parametrize("config", [1, 2])
+def test_decode_step_is_reproducible_call_after_call(dmoe, ws, config):
+    """The decode step runs gate/up and down tiles in one launch, the down tiles waiting on per-tile counters for the
+    gate/up tiles. 200 calls in a row, with other work queued between them, give the same bits every time."""
+    wl = workloads.make(config)
+    layer = dmoe.Layer(wl.D, wl.F, wl.K, wl.gate, wl.up, wl.down, swiglu_limit=wl.swiglu_limit,
+                       score_before_down=wl.score_before_down, shared=wl.shared,
+                       shared_swiglu_limit=wl.shared_swiglu_limit, remap=wl.remap, borrow=True)
+    want = layer.layer_forward(wl.x, wl.scores, wl.bias, wl.resident_mask, wl.renorm, wl.route_scale, ws).clone()
+    scratch = torch.empty(64 << 20, dtype=torch.uint8, device="cuda")
+    bad = 0
+    for i in range(200):
+        if i % 3 == 0:
+            scratch.fill_(i & 0xff)          # other traffic through the caches between the steps
+        out = layer.layer_forward(wl.x, wl.scores, wl.bias, wl.resident_mask, wl.renorm, wl.route_scale, ws)
+        bad += int(not torch.equal(out, want))
+    torch.cuda.synchronize()
+    assert bad == 0, f"{bad} of 200 calls differ from the first"
