@@ -41,7 +41,7 @@ constexpr int wait_vmcnt_lgkm0(int n) { return 0x0070 | (n & 15) | ((n >> 4) << 
 constexpr int kWaitLgkm0 = 0xc07f;
 
 template <typename Fmt, bool GATE_UP, int MT>
-__device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint8_t *lds) {
+__device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint8_t *lds, const int strip) {
     using CS = ChunkStream<Fmt, true>;
     static_assert(Fmt::kVals == 32, "one reduction step must be 64 elements = one 128-byte activation granule");
     constexpr int KV = 32, KSTEP = 64, NJ = 4, NT = 2;
@@ -55,7 +55,7 @@ __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint
     const size_t e = t.expert;
 
     // ---- this wavefront's weight rows (gate_up: tile 0 = gate, tile 1 = up rows of the same 32 columns) ----
-    const int col_base = ((int)blockIdx.x * kWideWaves + wave) * (GATE_UP ? 32 : 64);
+    const int col_base = (strip * kWideWaves + wave) * (GATE_UP ? 32 : 64);
     const bool wave_on = col_base < n_out;
     CS cs[NT];
 #pragma unroll
@@ -273,10 +273,15 @@ template <typename Fmt, bool GATE_UP>
 __global__ __launch_bounds__(kWideWaves * 64) void qgemm_wide_kernel(GemmArgs g) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t wide_lds[]; // [kWideRing][256 rows][128 bytes], swizzled
     Tile t;
-    const uint32_t slot = blockIdx.y;
+    // Workgroups go to the eight XCDs round-robin in launch order. All column strips of a tile are given to ONE XCD
+    // (tile = 8 * (k / strips) + xcd for the k-th workgroup of that XCD), so the tile's activations are fetched into one
+    // L2 instead of eight; gridDim.y is a multiple of 8, which makes this a permutation of the grid.
+    const uint32_t nx = gridDim.x, b = blockIdx.y * nx + blockIdx.x, k = b >> 3;
+    const uint32_t slot = (k / nx) * 8u + (b & 7u);
+    const int strip = (int)(k % nx);
     if (g.tiles) {
         const uint32_t n_tiles = *g.n_tiles;
-        t = g.tiles[slot];
+        t = g.tiles[slot < (uint32_t)g.max_tiles ? slot : 0u];
         if (slot >= n_tiles) return;
         if ((int)t.nrows < g.min_rows) return; // left to the weight-streaming kernel
     } else {
@@ -288,12 +293,12 @@ __global__ __launch_bounds__(kWideWaves * 64) void qgemm_wide_kernel(GemmArgs g)
     }
     // the tile is the same for the whole workgroup; saying so keeps the variants apart as scalar branches
     const int mt = __builtin_amdgcn_readfirstlane((int)((t.nrows + 31u) >> 5));
-    if (mt <= 1) wide_tile<Fmt, GATE_UP, 1>(g, t, wide_lds);
-    else if (mt == 2) wide_tile<Fmt, GATE_UP, 2>(g, t, wide_lds);
-    else if (mt == 3) wide_tile<Fmt, GATE_UP, 3>(g, t, wide_lds);
-    else if (mt == 4) wide_tile<Fmt, GATE_UP, 4>(g, t, wide_lds);
-    else if (mt <= 6) wide_tile<Fmt, GATE_UP, 6>(g, t, wide_lds);
-    else wide_tile<Fmt, GATE_UP, 8>(g, t, wide_lds);
+    if (mt <= 1) wide_tile<Fmt, GATE_UP, 1>(g, t, wide_lds, strip);
+    else if (mt == 2) wide_tile<Fmt, GATE_UP, 2>(g, t, wide_lds, strip);
+    else if (mt == 3) wide_tile<Fmt, GATE_UP, 3>(g, t, wide_lds, strip);
+    else if (mt == 4) wide_tile<Fmt, GATE_UP, 4>(g, t, wide_lds, strip);
+    else if (mt <= 6) wide_tile<Fmt, GATE_UP, 6>(g, t, wide_lds, strip);
+    else wide_tile<Fmt, GATE_UP, 8>(g, t, wide_lds, strip);
 }
 
 bool qgemm_wide_supports(const QView &b) {
@@ -310,7 +315,7 @@ static int launch_wide(const GemmArgs &g, hipStream_t st) {
         raised = true;
     }
     const int cols_per_block = kWideWaves * (GATE_UP ? 32 : 64);
-    dim3 grid((unsigned)ceil_div(g.b0.rows, cols_per_block), (unsigned)g.max_tiles), block(kWideWaves * 64);
+    dim3 grid((unsigned)ceil_div(g.b0.rows, cols_per_block), (unsigned)((g.max_tiles + 7) / 8 * 8)), block(kWideWaves * 64);
     hipLaunchKernelGGL(kern, grid, block, kWideLdsBytes, st, g);
     DMOE_LAUNCH_CHECK();
     return DMOE_OK;
