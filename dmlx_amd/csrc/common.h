@@ -55,6 +55,7 @@ struct Workspace {
     // side stream (default priority) + fork/join events for work that overlaps the main stream
     hipStream_t side = nullptr;
     hipEvent_t fork = nullptr, join = nullptr;
+    hipEvent_t packed = nullptr, small_done = nullptr; // prefill: the small tiles' GEMMs run on the side stream
     bool last_with_shared = true; // layout of the last forward on this workspace (for dmoe_debug_last_activations)
 };
 int side_stream_ready(Workspace *w);  // creates the side stream and its events on first use

@@ -209,7 +209,7 @@ static FwdLayout forward_layout(const Layer *L, int T, bool with_shared = true) 
     f.n_live = b.take(4);
     f.tiles = b.take((size_t)(f.max_tiles > 0 ? f.max_tiles : 1) * sizeof(Tile));
     f.n_tiles = b.take(4);
-    f.tile_done = b.take(f.small ? (size_t)(f.max_tiles > 0 ? f.max_tiles : 1) * 4 : 0);
+    f.tile_done = b.take((size_t)(f.max_tiles > 0 ? f.max_tiles : 1) * 4);
     f.scratch = b.take(pack_scratch_bytes(n, L->E));
     f.h = b.take(rows * (size_t)L->F * 2);
     f.y = b.take(rows * (size_t)L->D * 2);
@@ -258,10 +258,9 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
         po.dense_rows = (uint32_t)T;
         po.dense_expert = (uint32_t)L->E;
     }
-    if (f.small) { // per-tile completion counters of the paired gate/up + down launch, zeroed with the tile list
-        po.tile_done = at<uint32_t>(w, f.tile_done);
-        po.n_done = (uint32_t)f.max_tiles;
-    }
+    // per-tile completion counters of the paired gate/up + down launch, zeroed with the tile list
+    po.tile_done = at<uint32_t>(w, f.tile_done);
+    po.n_done = (uint32_t)f.max_tiles;
     DMOE_TRY(launch_pack(po, d_slots, n, L->K, L->E, f.tile_m, at<void>(w, f.scratch), st));
     DMOE_TRY(stage_end(w, DMOE_STAGE_PACK, st));
 
@@ -305,6 +304,25 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
         return DMOE_OK;
     }
     const int small_rows = f.small ? 0 : prefill_small_rows(L->gate.view, L->down.view);
+    if (small_rows > 0 && !w->timer.enabled) {
+        // Prefill: the small tiles' two GEMMs (one paired launch) depend on the tile list only. They go to the side
+        // stream and fill the tails of the two matrix-core launches, which take the large tiles on `st`. (With stage
+        // timing on, the launches stay in a row on `st` so that every stage's time covers all of its tiles.)
+        GemmArgs gu_small = gu, dn_small = dn, gu_big = gu, dn_big = dn;
+        gu_small.max_rows = dn_small.max_rows = small_rows;
+        gu_big.min_rows = dn_big.min_rows = small_rows + 1;
+        if (qgemm_skinny_pair_supports(gu_small, dn_small)) {
+            DMOE_TRY(side_stream_ready(w));
+            DMOE_HIP(hipEventRecord(w->packed, st));
+            DMOE_HIP(hipStreamWaitEvent(w->side, w->packed, 0));
+            DMOE_TRY(launch_qgemm_skinny_pair(gu_small, dn_small, w->side));
+            DMOE_HIP(hipEventRecord(w->small_done, w->side));
+            DMOE_TRY(launch_qgemm_mfma(gu_big, st));
+            DMOE_TRY(launch_qgemm_mfma(dn_big, st));
+            DMOE_HIP(hipStreamWaitEvent(st, w->small_done, 0));
+            return DMOE_OK;
+        }
+    }
     DMOE_TRY(stage_begin(w, DMOE_STAGE_GATE_UP, st));
     DMOE_TRY(run_gemm(gu, f.small, st, small_rows));
     DMOE_TRY(stage_end(w, DMOE_STAGE_GATE_UP, st));

@@ -501,8 +501,9 @@ bool qgemm_skinny_pair_supports(const GemmArgs &gu, const GemmArgs &dn) {
     return gu.gate_up && !dn.gate_up && gu.tiles && gu.tiles == dn.tiles && gu.n_tiles == dn.n_tiles &&
            gu.max_tiles == dn.max_tiles && gu.max_tiles > 0 && 2 * (long)gu.max_tiles <= 65535 &&
            a.packed == b.packed && a.mode == b.mode && a.bits == b.bits && skinny_factored(a) == skinny_factored(b) &&
-           qgemm_skinny_supports(a) && qgemm_skinny_supports(b) && gu.tile_m <= qgemm_skinny_tile_m(a) &&
-           dn.tile_m <= qgemm_skinny_tile_m(b) && gu.tile_done != nullptr && dn.a == gu.out;
+           qgemm_skinny_supports(a) && qgemm_skinny_supports(b) && std::min(gu.tile_m, gu.max_rows) <= qgemm_skinny_tile_m(a) &&
+           std::min(dn.tile_m, dn.max_rows) <= qgemm_skinny_tile_m(b) && gu.max_rows == dn.max_rows &&
+           gu.tile_done != nullptr && dn.a == gu.out;
 }
 
 int launch_qgemm_skinny_pair(const GemmArgs &gu, const GemmArgs &dn, hipStream_t st) {

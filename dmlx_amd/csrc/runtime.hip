@@ -43,6 +43,8 @@ int side_stream_ready(Workspace *w) {
     DMOE_HIP(hipStreamCreateWithFlags(&w->side, hipStreamNonBlocking));
     DMOE_HIP(hipEventCreateWithFlags(&w->fork, hipEventDisableTiming));
     DMOE_HIP(hipEventCreateWithFlags(&w->join, hipEventDisableTiming));
+    DMOE_HIP(hipEventCreateWithFlags(&w->packed, hipEventDisableTiming));
+    DMOE_HIP(hipEventCreateWithFlags(&w->small_done, hipEventDisableTiming));
     return DMOE_OK;
 }
 
@@ -227,6 +229,8 @@ int dmoe_workspace_destroy(dmoe_workspace ws) {
     if (w->side) (void)hipStreamSynchronize(w->side);
     if (w->fork) (void)hipEventDestroy(w->fork);
     if (w->join) (void)hipEventDestroy(w->join);
+    if (w->packed) (void)hipEventDestroy(w->packed);
+    if (w->small_done) (void)hipEventDestroy(w->small_done);
     if (w->side) (void)hipStreamDestroy(w->side);
     hipError_t e = w->base ? hipFree(w->base) : hipSuccess;
     delete w;
