@@ -203,6 +203,53 @@ def test_c2_decode_mxfp4_smelt_full_size(dmoe, orc, ws):
     _check_layer(dmoe, orc, ws, wl)
 
 
+@pytest.mark.parametrize("config", [3, 4])
+def test_prefill_configs_full_size(dmoe, orc, ws, config):
+    """BASELINE configs 3 (8192-token ragged prefill, Zipf routing, affine-4) and 4 (2080-token mixed batch, affine-8
+    routed + FP8 shared expert) at full size. Routing and packing are compared bit for bit with the oracle on the
+    whole batch. The oracle's FFN would take minutes on 49 152 rows, so the outputs are pinned two ways that do not
+    depend on the batch size: a sample of 64 tokens (the rows of the most and of the least loaded experts, the
+    first and last tokens, random ones) against the oracle at full D, F and E, and the same 64 tokens run alone,
+    which takes the decode kernels instead of the prefill ones and must give the same rows."""
+    import copy
+    wl = workloads.make(config)
+    layer = dmoe.Layer(wl.D, wl.F, wl.K, wl.gate, wl.up, wl.down, swiglu_limit=wl.swiglu_limit,
+                       score_before_down=wl.score_before_down, shared=wl.shared,
+                       shared_swiglu_limit=wl.shared_swiglu_limit, remap=wl.remap)
+    idx, w, want_idx, want_w = _route(dmoe, orc, wl)
+    got = dmoe.pack(idx, wl.E, ws)
+    want = orc.pack(want_idx, wl.E)
+    for name in ("order", "inv", "token", "sorted_e", "counts", "offsets"):
+        np.testing.assert_array_equal(to_np_u32(got[name]), want[name], err_msg=name)
+    counts = want["counts"].astype(np.int64)
+    assert counts.sum() == wl.T * wl.K
+    out = layer.forward(wl.x, idx, w, ws)
+    assert out.shape == (wl.T, wl.D) and bool(torch.isfinite(out.float()).all())
+
+    rng = np.random.default_rng(config)
+    live = np.nonzero(counts)[0]
+    heavy, light = live[np.argmax(counts[live])], live[np.argmin(counts[live])]
+    tok_of = lambda e: np.nonzero((want_idx == e).any(axis=1))[0]
+    pick = np.concatenate([tok_of(heavy)[:16], tok_of(light)[:8], [0, 1, wl.T - 2, wl.T - 1],
+                           rng.integers(0, wl.T, 64)])
+    sample = np.unique(pick)[:64]
+    sel = torch.from_numpy(sample).to("cuda")
+    sub = copy.copy(wl)
+    sub.x, sub.T = wl.x[sel].contiguous(), len(sample)
+    want_out = oracle_forward(sub, want_idx[sample], want_w[sample])
+    got_out = out[sel].float().cpu().numpy()
+    err = max_abs_rel(got_out, want_out)
+    assert err < OUT_TOL, (wl.name, "sample against the oracle", err)
+    alone = layer.forward(sub.x, idx[sel].contiguous(), w[sel].contiguous(), ws).float().cpu().numpy()
+    err_alone = max_abs_rel(alone, want_out)
+    assert err_alone < OUT_TOL, (wl.name, "sample run alone against the oracle", err_alone)
+    err_paths = max_abs_rel(alone, got_out)
+    assert err_paths < OUT_TOL, (wl.name, "prefill kernels against decode kernels", err_paths)
+    print(f"[parity] {wl.name}: T={wl.T} rows/expert max {counts.max()} min {counts[live].min()} "
+          f"sample err {err:.3e}, alone {err_alone:.3e}, prefill vs decode {err_paths:.3e}")
+    layer.close()
+
+
 def test_forward_edge_cases(dmoe, orc, ws):
     wl = workloads.make(1, scale=0.125)
     layer = dmoe.Layer(wl.D, wl.F, wl.K, wl.gate, wl.up, wl.down, swiglu_limit=wl.swiglu_limit, shared=wl.shared)
