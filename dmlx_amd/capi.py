@@ -63,6 +63,7 @@ EXPORTS = [
     "dmoe_stream_create", "dmoe_stream_destroy", "dmoe_stream_synchronize",
     "dmoe_malloc", "dmoe_free", "dmoe_copy_to_device", "dmoe_copy_to_host",
     "dmoe_workspace_create", "dmoe_workspace_destroy", "dmoe_workspace_reserved",
+    "dmoe_workspace_check", "dmoe_workspace_set_wait_limit",
     "dmoe_workspace_set_stage_timing", "dmoe_workspace_read_stage_times",
     "dmoe_topk_route", "dmoe_gate_route", "dmoe_remap_indices", "dmoe_expand_tokens",
     "dmoe_reduce_experts", "dmoe_smelt_build_mask", "dmoe_build_remap", "dmoe_preload_remap",
@@ -117,6 +118,13 @@ class Workspace:
         n = C.c_size_t()
         check(lib().dmoe_workspace_reserved(C.byref(n), self.h))
         return n.value
+
+    def check(self):
+        """Wait for the current stream; raises if a kernel launched with this workspace gave up a bounded wait."""
+        check(lib().dmoe_workspace_check(self.h, _stream()))
+
+    def set_wait_limit(self, polls):
+        check(lib().dmoe_workspace_set_wait_limit(self.h, C.c_uint(polls)))
 
     STAGES = ("route", "pack", "gate_up", "down", "shared", "combine")
 

@@ -57,6 +57,10 @@ struct Workspace {
     hipEvent_t fork = nullptr, join = nullptr;
     hipEvent_t packed = nullptr, small_done = nullptr; // prefill: the small tiles' GEMMs run on the side stream
     bool last_with_shared = true; // layout of the last forward on this workspace (for dmoe_debug_last_activations)
+    // Device words that outlive workspace growth: [0] counts waits inside a paired GEMM launch that gave up (see
+    // GemmArgs::wait_expired), read and cleared by dmoe_workspace_check. [1] is unused.
+    uint32_t *flags = nullptr;
+    uint32_t spin_limit = 1u << 16; // polls of ~0.25 us a waiting workgroup makes before it gives up (~16 ms)
 };
 int side_stream_ready(Workspace *w);  // creates the side stream and its events on first use
 
@@ -165,6 +169,10 @@ struct GemmArgs {
     // tile_done[tile] after their stores, a down workgroup of that tile waits for tile_done_target before it reads h.
     uint32_t *tile_done = nullptr;
     uint32_t tile_done_target = 0;
+    // a waiting workgroup polls at most spin_limit times; one that gives up adds 1 to *wait_expired (may be null)
+    // and goes on with whatever the rows hold, so the launch always ends and the host can see that it went wrong
+    uint32_t spin_limit = 1u << 16;
+    uint32_t *wait_expired = nullptr;
     float swiglu_limit_dense = 0.0f;    // the limit for tiles flagged kTileDense
     uint32_t row_scale_rows = 0xffffffffu; // row_scale applies to sorted rows below this
 };

@@ -297,6 +297,8 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     // Decode sizes: both GEMMs in one launch; a down workgroup waits for its own tile's gate/up workgroups only, so
     // the down projection fills the chip while the last gate/up workgroups drain (timed as the gate/up stage).
     gu.tile_done = po.tile_done;
+    dn.spin_limit = w->spin_limit;
+    dn.wait_expired = w->flags;
     if (f.small && qgemm_skinny_pair_supports(gu, dn)) {
         DMOE_TRY(stage_begin(w, DMOE_STAGE_GATE_UP, st));
         DMOE_TRY(launch_qgemm_skinny_pair(gu, dn, st));

@@ -72,7 +72,6 @@ struct SkinnyStage {
 // g.tile_done[slot] once its stores have reached memory; kSkinnySyncWait = the workgroup waits for g.tile_done[slot] to
 // reach g.tile_done_target before it reads its activations (the other role's output), its weight ring already in flight.
 constexpr int kSkinnySyncNone = 0, kSkinnySyncSignal = 1, kSkinnySyncWait = 2;
-constexpr uint32_t kSkinnySpinLimit = 1u << 16; // polls of ~0.25 us: the wait ends after ~16 ms whatever happens
 
 template <typename Fmt, bool FACTORED, bool PACKED, int RJT>
 __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, uint8_t *skinny_lds, const bool gate_up,
@@ -188,10 +187,14 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
         if (wave == 0) {
             uint32_t polls = 0;
             while (__hip_atomic_load(&g.tile_done[slot], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < g.tile_done_target &&
-                   polls < kSkinnySpinLimit) {
+                   polls < g.spin_limit) {
                 __builtin_amdgcn_s_sleep(8);
                 ++polls;
             }
+            // gave up: the launch still ends, the host learns about it from the workspace's counter
+            if (polls >= g.spin_limit && lane == 0 && g.wait_expired &&
+                __hip_atomic_load(&g.tile_done[slot], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < g.tile_done_target)
+                atomicAdd(g.wait_expired, 1u);
         }
         __syncthreads();
 #pragma unroll

@@ -174,11 +174,19 @@ int dmoe_workspace_create(dmoe_workspace *out, size_t initial_bytes) {
         delete w;
         return hip_fail(e, "hipGetDevice");
     }
+    e = hipMalloc((void **)&w->flags, 256);
+    if (e == hipSuccess) e = hipMemset(w->flags, 0, 256);
+    if (e != hipSuccess) {
+        if (w->flags) (void)hipFree(w->flags);
+        delete w;
+        return hip_fail(e, "hipMalloc(workspace flags)");
+    }
     out->ctx = w;
     if (initial_bytes) {
         Workspace *tmp;
         int rc = workspace_reserve(*out, initial_bytes, &tmp);
         if (rc != DMOE_OK) {
+            (void)hipFree(w->flags);
             delete w;
             out->ctx = nullptr;
             return rc;
@@ -233,8 +241,35 @@ int dmoe_workspace_destroy(dmoe_workspace ws) {
     if (w->small_done) (void)hipEventDestroy(w->small_done);
     if (w->side) (void)hipStreamDestroy(w->side);
     hipError_t e = w->base ? hipFree(w->base) : hipSuccess;
+    if (w->flags) {
+        hipError_t e2 = hipFree(w->flags);
+        if (e == hipSuccess) e = e2;
+    }
     delete w;
     if (e != hipSuccess) return hip_fail(e, "hipFree(workspace)");
+    return DMOE_OK;
+}
+
+int dmoe_workspace_check(dmoe_workspace ws, dmoe_stream s) {
+    Workspace *w = (Workspace *)ws.ctx;
+    DMOE_REQUIRE(w != nullptr, "workspace handle is null");
+    DMOE_HIP(hipStreamSynchronize(to_hip(s)));
+    if (w->side) DMOE_HIP(hipStreamSynchronize(w->side));
+    uint32_t expired = 0;
+    DMOE_HIP(hipMemcpy(&expired, w->flags, sizeof expired, hipMemcpyDeviceToHost));
+    if (expired) {
+        DMOE_HIP(hipMemset(w->flags, 0, sizeof expired));
+        set_error("%u workgroup(s) gave up waiting for their tile's gate/up results: outputs since the last check are invalid",
+                  (unsigned)expired);
+        return DMOE_ERR_TIMEOUT;
+    }
+    return DMOE_OK;
+}
+
+int dmoe_workspace_set_wait_limit(dmoe_workspace ws, unsigned polls) {
+    Workspace *w = (Workspace *)ws.ctx;
+    DMOE_REQUIRE(w != nullptr, "workspace handle is null");
+    w->spin_limit = polls;
     return DMOE_OK;
 }
 

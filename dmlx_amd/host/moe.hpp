@@ -58,7 +58,10 @@ class Context {
     Context &operator=(const Context &) = delete;
     dmoe_stream stream() const { return stream_; }
     dmoe_workspace workspace() const { return ws_; }
-    void synchronize() const { check(dmoe_stream_synchronize(stream_)); } // Array.eval()
+    // Array.eval(): the host-visible sync point, where a failed step surfaces (a bounded wait inside a kernel that
+    // gave up throws here, as a failed lazy graph throws at eval() in the reference)
+    void synchronize() const { check(dmoe_workspace_check(ws_, stream_)); }
+    void setWaitLimit(unsigned polls) const { check(dmoe_workspace_set_wait_limit(ws_, polls)); }
 
   private:
     dmoe_stream stream_{};

@@ -44,9 +44,12 @@ pub const Context = struct {
         _ = c.dmoe_workspace_destroy(self.ws);
         _ = c.dmoe_stream_destroy(self.stream);
     }
-    /// Array.eval(): the host-visible synchronisation point
+    /// Array.eval(): the host-visible synchronisation point; a step whose kernels gave up a bounded wait fails here
     pub fn eval(self: Context) Error!void {
-        try check(c.dmoe_stream_synchronize(self.stream));
+        try check(c.dmoe_workspace_check(self.ws, self.stream));
+    }
+    pub fn setWaitLimit(self: Context, polls: c_uint) Error!void {
+        try check(c.dmoe_workspace_set_wait_limit(self.ws, polls));
     }
 };
 

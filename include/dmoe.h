@@ -37,7 +37,8 @@ typedef enum {
     DMOE_ERR_INVALID = 1,     /* bad argument / unsupported shape            */
     DMOE_ERR_HIP = 2,         /* a HIP runtime call failed                   */
     DMOE_ERR_UNSUPPORTED = 3, /* valid request this build does not implement */
-    DMOE_ERR_NO_DEVICE = 4    /* no gfx950 device visible                    */
+    DMOE_ERR_NO_DEVICE = 4,   /* no gfx950 device visible                    */
+    DMOE_ERR_TIMEOUT = 5      /* a bounded wait inside a kernel gave up      */
 } dmoe_status;
 
 /* quantization mode; the reference passes it as the C strings "affine"/"mxfp4"
@@ -79,6 +80,15 @@ int dmoe_workspace_create(dmoe_workspace *out, size_t initial_bytes);
 int dmoe_workspace_destroy(dmoe_workspace ws);
 /* bytes currently reserved; growth happens inside calls (it synchronizes the device) */
 int dmoe_workspace_reserved(size_t *out_bytes, dmoe_workspace ws);
+/* Waits for stream s, then reports whether any kernel launched with this workspace since the last check gave up a
+ * bounded wait: at decode sizes the down projection's workgroups wait, inside the launch they share with the gate/up
+ * projection, for their tile's gate/up workgroups, and give up after the workspace's poll limit (~16 ms) so that the
+ * launch ends whatever happens. Returns DMOE_ERR_TIMEOUT (and clears the count) if that happened: the outputs of the
+ * calls since the last check must then be discarded. Plays the role of c.check(rc) after Array.eval() in the
+ * reference (moe_router.zig:68,74), where a failed lazy graph surfaces at the sync point. */
+int dmoe_workspace_check(dmoe_workspace ws, dmoe_stream s);
+/* polls (~0.25 us each) a waiting workgroup makes before it gives up; default 65536. For tests of the give-up path. */
+int dmoe_workspace_set_wait_limit(dmoe_workspace ws, unsigned polls);
 
 /* Per-stage device timing of the layer forward calls made with this workspace (HIP events recorded on the
  * call's stream around each stage). Off by default; while on, every forward call waits for the previous

@@ -62,3 +62,31 @@ def test_decode_step_is_reproducible_call_after_call(dmoe, ws, config):
         bad += int(not torch.equal(out, want))
     torch.cuda.synchronize()
     assert bad == 0, f"{bad} of 200 calls differ from the first"
+
+
+def test_decode_step_reports_a_wait_that_gave_up(dmoe, ws):
+    """Failure handling of the decode launch: its down-projection workgroups wait a bounded number of polls for
+    their tile's gate/up workgroups. With the bound forced to zero from the host they give up at once (every kernel
+    still runs to its end), and the workspace check at the next sync point must say so, once; with the default
+    bound back in place the same call is clean and gives the reference bits again."""
+    from dmlx_amd.capi import DmoeError
+    wl = workloads.make(1, scale=0.25)
+    layer = dmoe.Layer(wl.D, wl.F, wl.K, wl.gate, wl.up, wl.down, swiglu_limit=wl.swiglu_limit,
+                       score_before_down=wl.score_before_down, shared=wl.shared,
+                       shared_swiglu_limit=wl.shared_swiglu_limit, remap=wl.remap, borrow=True)
+    step = lambda: layer.layer_forward(wl.x, wl.scores, wl.bias, wl.resident_mask, wl.renorm, wl.route_scale, ws)
+    want = step().clone()
+    ws.check()                                   # a normal step leaves nothing behind
+    ws.set_wait_limit(0)
+    try:
+        for _ in range(3):
+            step()
+        with pytest.raises(DmoeError, match="gave up"):
+            ws.check()
+        ws.check()                               # reported once, then cleared
+    finally:
+        ws.set_wait_limit(1 << 16)
+    out = step()
+    ws.check()
+    assert torch.equal(out, want)
+    layer.close()
