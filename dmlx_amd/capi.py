@@ -12,7 +12,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libdmoe.so")
 
-QUANT_AFFINE, QUANT_MXFP4, QUANT_FP8_ROW = 0, 1, 2
+QUANT_AFFINE, QUANT_MXFP4, QUANT_FP8_ROW, QUANT_NONE = 0, 1, 2, 3
 WEIGHTS_COPY_FROM_HOST, WEIGHTS_COPY_FROM_DEVICE, WEIGHTS_BORROW_DEVICE = 0, 1, 2
 
 
@@ -154,14 +154,14 @@ class QWeight:
     """A stack [n, rows, cols] of quantized matrices held as torch tensors (any device)."""
 
     def __init__(self, w, scales, biases, rows, cols, mode, bits, group_size):
-        self.w, self.scales, self.biases = w.contiguous(), scales.contiguous(), biases
+        self.w, self.scales, self.biases = w.contiguous(), None if scales is None else scales.contiguous(), biases
         if self.biases is not None:
             self.biases = self.biases.contiguous()
         self.rows, self.cols, self.mode, self.bits, self.group_size = rows, cols, mode, bits, group_size
         self.n_mats = w.shape[0] if w.dim() == 3 else 1
 
     def to(self, device):
-        return QWeight(self.w.to(device), self.scales.to(device),
+        return QWeight(self.w.to(device), None if self.scales is None else self.scales.to(device),
                        None if self.biases is None else self.biases.to(device),
                        self.rows, self.cols, self.mode, self.bits, self.group_size)
 
@@ -170,7 +170,9 @@ class QWeight:
                         self.cols, self.mode, self.bits, self.group_size)
 
     def nbytes(self):
-        n = self.w.numel() * self.w.element_size() + self.scales.numel() * self.scales.element_size()
+        n = self.w.numel() * self.w.element_size()
+        if self.scales is not None:
+            n += self.scales.numel() * self.scales.element_size()
         if self.biases is not None:
             n += self.biases.numel() * self.biases.element_size()
         return n

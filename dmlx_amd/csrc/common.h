@@ -188,6 +188,9 @@ int launch_qgemm_skinny_pair(const GemmArgs &gu, const GemmArgs &dn, hipStream_t
 int launch_qgemm_mfma(const GemmArgs &g, hipStream_t st); // picks the wide kernel when the format allows it
 int launch_qgemm_wide(const GemmArgs &g, hipStream_t st);
 bool qgemm_skinny_supports(const QView &b);
+// unquantized bf16 weights (DMOE_QUANT_NONE): one kernel for every size
+bool gemm_bf16_supports(const QView &b);
+int launch_gemm_bf16(const GemmArgs &g, hipStream_t st);
 int qgemm_skinny_tile_m(const QView &b);  // rows per tile to build tile lists with for the skinny path
 bool qgemm_mfma_supports(const QView &b);
 bool qgemm_wide_supports(const QView &b);

@@ -5,9 +5,11 @@
 namespace dmoe {
 
 static size_t w_row_bytes(const dmoe_qweight *q) {
+    if (q->mode == DMOE_QUANT_NONE) return (size_t)q->cols * 2;
     return q->mode == DMOE_QUANT_FP8_ROW ? (size_t)q->cols : (size_t)q->cols * (size_t)q->bits / 8;
 }
 static size_t s_row_bytes(const dmoe_qweight *q) {
+    if (q->mode == DMOE_QUANT_NONE) return 0;
     if (q->mode == DMOE_QUANT_FP8_ROW) return 4;
     if (q->mode == DMOE_QUANT_MXFP4) return (size_t)q->cols / 32;
     return (size_t)(q->cols / q->group_size) * 2;
@@ -20,7 +22,7 @@ size_t qweight_b_bytes(const dmoe_qweight *q) {
 
 int make_qview(QView *v, const dmoe_qweight *q, const char *name) {
     DMOE_REQUIRE(q != nullptr, "%s: descriptor is null", name);
-    DMOE_REQUIRE(q->w && q->scales, "%s: weight / scales pointer is null", name);
+    DMOE_REQUIRE(q->w && (q->scales || q->mode == DMOE_QUANT_NONE), "%s: weight / scales pointer is null", name);
     DMOE_REQUIRE(q->n_mats >= 1 && q->rows >= 1 && q->cols >= 1, "%s: bad shape [%d,%d,%d]", name, q->n_mats,
                  q->rows, q->cols);
     switch (q->mode) {
@@ -40,6 +42,12 @@ int make_qview(QView *v, const dmoe_qweight *q, const char *name) {
         DMOE_REQUIRE(q->bits == 8, "%s: fp8 needs bits=8", name);
         DMOE_REQUIRE(q->biases == nullptr, "%s: fp8 takes no biases", name);
         DMOE_REQUIRE(q->cols % 16 == 0, "%s: cols %d not a multiple of 16", name, q->cols);
+        break;
+    case DMOE_QUANT_NONE:
+        DMOE_REQUIRE(q->bits == 16, "%s: unquantized weights are bf16 (bits=16, got %d)", name, q->bits);
+        DMOE_REQUIRE(q->scales == nullptr && q->biases == nullptr, "%s: unquantized weights take no scales / biases", name);
+        DMOE_REQUIRE(q->cols % 8 == 0 && q->rows % 4 == 0, "%s: unquantized weights need rows %% 4 == 0 and cols %% 8 == 0 (got [%d,%d])",
+                     name, q->rows, q->cols);
         break;
     default:
         set_error("%s: unknown quantization mode %d", name, q->mode);
@@ -113,6 +121,10 @@ extern "C" int dmoe_dequantize(uint16_t *d_out, const dmoe_qweight *qw, int mat_
     DMOE_REQUIRE(d_out != nullptr, "dequantize: out is null");
     DMOE_REQUIRE(mat_index >= 0 && mat_index < q.n_mats, "dequantize: mat_index %d out of [0,%d)", mat_index,
                  q.n_mats);
+    if (q.mode == DMOE_QUANT_NONE) { // nothing to decode: the matrix as it is
+        DMOE_HIP(hipMemcpyAsync(d_out, q.w + (size_t)mat_index * q.w_mat, q.w_mat, hipMemcpyDeviceToDevice, to_hip(s)));
+        return DMOE_OK;
+    }
     DMOE_REQUIRE(q.cols % 32 == 0, "dequantize: cols %d not a multiple of 32", q.cols);
     return dispatch_format(q, DequantLaunch{d_out, q, mat_index, to_hip(s)});
 }

@@ -52,7 +52,7 @@ static void free_layer(Layer *L) {
 static int adopt(QOwned *dst, const dmoe_qweight *src, int source, const char *name, hipStream_t st, int spare_mats = 0) {
     dst->q = *src;
     if (source != DMOE_WEIGHTS_BORROW_DEVICE) {
-        DMOE_REQUIRE(src->w && src->scales, "%s: weight / scales pointer is null", name);
+        DMOE_REQUIRE(src->w && (src->scales || src->mode == DMOE_QUANT_NONE), "%s: weight / scales pointer is null", name);
         // validate the shape before sizing any copy
         QView probe;
         dmoe_qweight tmp = *src;
@@ -230,6 +230,7 @@ static int prefill_small_rows(const QView &b0, const QView &b1) {
     return std::min(qgemm_skinny_tile_m(b0), qgemm_skinny_tile_m(b1));
 }
 static int run_gemm(const GemmArgs &g, bool small, hipStream_t st, int small_rows = 0) {
+    if (g.b0.mode == DMOE_QUANT_NONE) return launch_gemm_bf16(g, st);
     if (small) return launch_qgemm_skinny(g, st);
     if (small_rows <= 0 || !g.tiles) return launch_qgemm_mfma(g, st);
     GemmArgs big = g, rest = g;
@@ -576,7 +577,7 @@ int dmoe_gather_qmm(uint16_t *d_out, const uint16_t *d_x, const dmoe_qweight *qw
     DMOE_REQUIRE(v.n_mats <= 1024, "gather_qmm: more than 1024 matrices in the stack");
     hipStream_t st = to_hip(s);
     const bool small = use_small_path((size_t)R, v.n_mats, v);
-    DMOE_REQUIRE(small || qgemm_mfma_supports(v), "gather_qmm: unsupported weight shape rows=%d cols=%d", v.rows, v.cols);
+    DMOE_REQUIRE(small || qgemm_mfma_supports(v) || gemm_bf16_supports(v), "gather_qmm: unsupported weight shape rows=%d cols=%d", v.rows, v.cols);
     const int tile_m = small ? qgemm_skinny_tile_m(v) : qgemm_mfma_tile_m(v);
     const int max_tiles = pack_max_tiles((size_t)R, v.n_mats, tile_m);
     Bump b;

@@ -188,10 +188,29 @@ static int find_proj(const std::map<std::string, StTensor> &index, const std::st
                      int group, bool stacked, dmoe_qweight *q) {
     auto w = index.find(prefix + ".weight"), s = index.find(prefix + ".scales"), b = index.find(prefix + ".biases");
     DMOE_REQUIRE(w != index.end(), "safetensors: tensor %s.weight not found", prefix.c_str());
-    DMOE_REQUIRE(s != index.end(), "safetensors: tensor %s.scales not found (unquantized experts are not supported)",
+    const size_t nd = stacked ? 3 : 2;
+    if (mode == DMOE_QUANT_NONE) { // unquantized experts: the bf16 matrix as it is
+        const StTensor &tw = w->second;
+        DMOE_REQUIRE(tw.shape.size() == nd, "safetensors: %s: expected a %zu-dimensional weight", prefix.c_str(), nd);
+        DMOE_REQUIRE(tw.dtype == "BF16", "safetensors: %s.weight has dtype %s, expected BF16 (unquantized experts)",
+                     prefix.c_str(), tw.dtype.c_str());
+        const long long n = stacked ? tw.shape[0] : 1, rows = tw.shape[nd - 2], cols = tw.shape[nd - 1];
+        DMOE_REQUIRE(n >= 1 && rows >= 1 && cols >= 1 && tw.bytes == (size_t)(n * rows * cols * 2),
+                     "safetensors: %s.weight: bad shape or byte count", prefix.c_str());
+        q->w = tw.data;
+        q->scales = nullptr;
+        q->biases = nullptr;
+        q->n_mats = (int)n;
+        q->rows = (int)rows;
+        q->cols = (int)cols;
+        q->mode = mode;
+        q->bits = 16;
+        q->group_size = 0;
+        return DMOE_OK;
+    }
+    DMOE_REQUIRE(s != index.end(), "safetensors: tensor %s.scales not found (pass mode \"none\" for unquantized experts)",
                  prefix.c_str());
     const StTensor &tw = w->second, &ts = s->second;
-    const size_t nd = stacked ? 3 : 2;
     DMOE_REQUIRE(tw.shape.size() == nd && ts.shape.size() == nd, "safetensors: %s: expected %zu-dimensional weight and scales",
                  prefix.c_str(), nd);
     DMOE_REQUIRE(tw.dtype == "U32", "safetensors: %s.weight has dtype %s, expected U32 (packed codes)", prefix.c_str(),
@@ -229,8 +248,9 @@ static int find_proj(const std::map<std::string, StTensor> &index, const std::st
 struct Subset {
     std::vector<uint8_t> w, s, b;
     void take(dmoe_qweight *q, const uint8_t *mask, int n_total, int n_keep) {
-        const size_t wb = (size_t)q->rows * (q->cols * q->bits / 32) * 4;
-        const size_t sb = (size_t)q->rows * (q->cols / q->group_size) * (q->mode == DMOE_QUANT_MXFP4 ? 1 : 2);
+        const bool plain = q->mode == DMOE_QUANT_NONE;
+        const size_t wb = plain ? (size_t)q->rows * q->cols * 2 : (size_t)q->rows * (q->cols * q->bits / 32) * 4;
+        const size_t sb = plain ? 0 : (size_t)q->rows * (q->cols / q->group_size) * (q->mode == DMOE_QUANT_MXFP4 ? 1 : 2);
         w.resize(wb * n_keep);
         s.resize(sb * n_keep);
         if (q->biases) b.resize(sb * n_keep);
@@ -238,12 +258,12 @@ struct Subset {
         for (int e = 0; e < n_total; ++e) {
             if (!mask[e]) continue;
             memcpy(w.data() + wb * slot, (const uint8_t *)q->w + wb * e, wb);
-            memcpy(s.data() + sb * slot, (const uint8_t *)q->scales + sb * e, sb);
+            if (sb) memcpy(s.data() + sb * slot, (const uint8_t *)q->scales + sb * e, sb);
             if (q->biases) memcpy(b.data() + sb * slot, (const uint8_t *)q->biases + sb * e, sb);
             ++slot;
         }
         q->w = w.data();
-        q->scales = s.data();
+        if (sb) q->scales = s.data();
         if (q->biases) q->biases = b.data();
         q->n_mats = n_keep;
     }
@@ -259,7 +279,8 @@ extern "C" int dmoe_layer_create_from_safetensors(dmoe_layer *out, const char *c
     out->ctx = nullptr;
     DMOE_REQUIRE(n_paths >= 1 && layer_idx >= 0, "layer_create_from_safetensors: need at least one file and a layer index >= 0");
     const int mode = dmoe_quant_mode_from_string(o->mode ? o->mode : "");
-    DMOE_REQUIRE(mode == DMOE_QUANT_AFFINE || mode == DMOE_QUANT_MXFP4, "layer_create_from_safetensors: mode must be \"affine\" or \"mxfp4\"");
+    DMOE_REQUIRE(mode == DMOE_QUANT_AFFINE || mode == DMOE_QUANT_MXFP4 || mode == DMOE_QUANT_NONE,
+                 "layer_create_from_safetensors: mode must be \"affine\", \"mxfp4\" or \"none\"");
     std::vector<StFile> files((size_t)n_paths);
     std::map<std::string, StTensor> index;
     for (int i = 0; i < n_paths; ++i) {
@@ -280,7 +301,8 @@ extern "C" int dmoe_layer_create_from_safetensors(dmoe_layer *out, const char *c
     d.weight_source = DMOE_WEIGHTS_COPY_FROM_HOST;
     if (o->load_shared && index.count(base + "shared_experts.gate_proj.weight")) {
         const int smode = dmoe_quant_mode_from_string(o->shared_mode ? o->shared_mode : o->mode);
-        DMOE_REQUIRE(smode == DMOE_QUANT_AFFINE || smode == DMOE_QUANT_MXFP4, "layer_create_from_safetensors: bad shared_mode");
+        DMOE_REQUIRE(smode == DMOE_QUANT_AFFINE || smode == DMOE_QUANT_MXFP4 || smode == DMOE_QUANT_NONE,
+                     "layer_create_from_safetensors: bad shared_mode");
         const int sbits = o->shared_bits ? o->shared_bits : o->bits, sgroup = o->shared_group_size ? o->shared_group_size : o->group_size;
         DMOE_TRY(find_proj(index, base + "shared_experts.gate_proj", smode, sbits, sgroup, false, &d.shared_gate));
         DMOE_TRY(find_proj(index, base + "shared_experts.up_proj", smode, sbits, sgroup, false, &d.shared_up));

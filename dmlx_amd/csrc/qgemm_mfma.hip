@@ -321,7 +321,8 @@ __global__ __launch_bounds__(kMfmaWaves * 64) void qgemm_mfma_kernel(GemmArgs g)
 
 bool qgemm_mfma_supports(const QView &b) {
     int vals = (b.mode == DMOE_QUANT_AFFINE && b.bits == 4) || b.mode == DMOE_QUANT_MXFP4 ? 32 : 16;
-    return b.cols % (2 * vals) == 0 && b.cols % 64 == 0 && b.rows % 4 == 0; // activation rows are staged in 128-byte granules
+    // activation rows are staged in 128-byte granules; unquantized weights have their own kernel
+    return b.mode != DMOE_QUANT_NONE && b.cols % (2 * vals) == 0 && b.cols % 64 == 0 && b.rows % 4 == 0;
 }
 
 struct MfmaLaunch {

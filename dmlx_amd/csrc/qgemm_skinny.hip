@@ -454,7 +454,7 @@ int qgemm_skinny_tile_m(const QView &b) {
 }
 
 bool qgemm_skinny_supports(const QView &b) {
-    return b.cols % (2 * skinny_vals(b)) == 0 && skinny_lds_bytes(b) <= 150 * 1024;
+    return b.mode != DMOE_QUANT_NONE && b.cols % (2 * skinny_vals(b)) == 0 && skinny_lds_bytes(b) <= 150 * 1024;
 }
 
 struct SkinnyLaunch {

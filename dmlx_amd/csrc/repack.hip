@@ -5,6 +5,7 @@
 namespace dmoe {
 
 static int chunk_vals(const QView &v) {
+    if (v.mode == DMOE_QUANT_NONE) return 8; // a 16-byte piece holds 8 bf16; a step of two pieces is one MFMA (K = 16)
     return (v.mode == DMOE_QUANT_AFFINE && v.bits == 4) || v.mode == DMOE_QUANT_MXFP4 ? 32 : 16;
 }
 

@@ -93,6 +93,7 @@ int dmoe_quant_mode_from_string(const char *name) {
     if (!strcmp(name, "affine")) return DMOE_QUANT_AFFINE;
     if (!strcmp(name, "mxfp4")) return DMOE_QUANT_MXFP4;
     if (!strcmp(name, "fp8")) return DMOE_QUANT_FP8_ROW;
+    if (!strcmp(name, "none") || !strcmp(name, "bf16")) return DMOE_QUANT_NONE;
     return -1;
 }
 

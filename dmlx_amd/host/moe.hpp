@@ -275,7 +275,20 @@ struct QuantizedWeight {
     const void *data = nullptr, *scales = nullptr, *biases = nullptr; // host or device memory, see weight_source
     int n_mats = 1, rows = 0, cols = 0;
     int group_size = 64, bits = 4;
-    std::string mode = "affine"; // "affine" | "mxfp4" | "fp8"
+    // "affine" | "mxfp4" | "fp8" | "none": unquantized bf16 [n_mats, rows, cols] (bits 16, no scales), the
+    // is_quantized == false arm of DSV4SwitchGLU (deepseek_v4.zig:969-979, ops.gatherMm)
+    std::string mode = "affine";
+    static QuantizedWeight unquantized(const void *bf16_data, int n_mats, int rows, int cols) {
+        QuantizedWeight q;
+        q.data = bf16_data;
+        q.n_mats = n_mats;
+        q.rows = rows;
+        q.cols = cols;
+        q.group_size = 0;
+        q.bits = 16;
+        q.mode = "none";
+        return q;
+    }
     dmoe_qweight c() const {
         dmoe_qweight q{};
         q.w = data;
@@ -534,6 +547,45 @@ inline DeviceBatch buildOnDevice(const Context &ctx, const std::vector<const Req
     return out;
 }
 } // namespace batch_builder
+
+// ---- quantize_mod / ops leaf calls (mlx-zig; call shapes at deepseek_v4.zig:976-978, expert_preload.zig:265) ------
+namespace quantize_mod {
+// gatherQmm(ctx, x, w, scales, biases, lhs_indices?, rhs_indices, transpose=true, config, sorted): row r of the
+// result is x[lhs[r] or r] times the transposed matrix rhs[r] of the stack. `w` describes DEVICE memory here.
+inline Array gatherQmm(const Context &ctx, const Array &x, const QuantizedWeight &w, const Array *lhs_indices,
+                       const Array &rhs_indices, bool sorted) {
+    if (x.dtype() != DType::bfloat16 || x.shape().size() != 2 || x.shape()[1] != w.cols)
+        throw Error(DMOE_ERR_INVALID, "gatherQmm: x must be bfloat16 [rows, cols of the weights]");
+    if (rhs_indices.dtype() != DType::uint32 || (lhs_indices && (lhs_indices->dtype() != DType::uint32 ||
+                                                                 lhs_indices->size() != rhs_indices.size())))
+        throw Error(DMOE_ERR_INVALID, "gatherQmm: indices must be uint32 and of equal length");
+    const int R = (int)rhs_indices.size();
+    Array out(ctx, DType::bfloat16, {R, w.rows});
+    dmoe_qweight q = w.c();
+    check(dmoe_gather_qmm((uint16_t *)out.data(), (const uint16_t *)x.data(), &q,
+                          lhs_indices ? (const uint32_t *)lhs_indices->data() : nullptr,
+                          (const uint32_t *)rhs_indices.data(), R, sorted ? 1 : 0, ctx.workspace(), ctx.stream()));
+    return out;
+}
+// mlx_dequantize of one matrix of the stack -> bf16 [rows, cols]
+inline Array dequantize(const Context &ctx, const QuantizedWeight &w, int mat_index) {
+    Array out(ctx, DType::bfloat16, {w.rows, w.cols});
+    dmoe_qweight q = w.c();
+    check(dmoe_dequantize((uint16_t *)out.data(), &q, mat_index, ctx.stream()));
+    return out;
+}
+} // namespace quantize_mod
+namespace ops {
+// gatherMm(ctx, a, b, lhs?, rhs, sorted) with unquantized experts (deepseek_v4.zig:978). The reference hands over
+// the transposed view [E, in, out] of its [E, out, in] weights; this takes the [E, out, in] array itself (bf16).
+inline Array gatherMm(const Context &ctx, const Array &a, const Array &weight, const Array *lhs_indices,
+                      const Array &rhs_indices, bool sorted) {
+    if (weight.dtype() != DType::bfloat16 || weight.shape().size() != 3)
+        throw Error(DMOE_ERR_INVALID, "gatherMm: weight must be bfloat16 [n_experts, out, in]");
+    const QuantizedWeight q = QuantizedWeight::unquantized(weight.data(), weight.shape()[0], weight.shape()[1], weight.shape()[2]);
+    return quantize_mod::gatherQmm(ctx, a, q, lhs_indices, rhs_indices, sorted);
+}
+} // namespace ops
 
 // ---- the step after the layer (deepseek_v4.zig:2450-2499, 2652-2654, 2674) ---------------------------------
 // mhcPost(x, residual, post_mix, comb_mix): x [T,H] bf16, residual [T,hc_mult,H] bf16, post_mix [T,hc_mult(,1)]

@@ -10,7 +10,7 @@ from typing import Optional
 import torch
 
 from . import quantize as Q
-from .capi import QUANT_AFFINE, QUANT_FP8_ROW, QUANT_MXFP4, QWeight
+from .capi import QUANT_AFFINE, QUANT_FP8_ROW, QUANT_MXFP4, QUANT_NONE, QWeight
 
 
 @dataclass
@@ -69,6 +69,8 @@ def _quant_stack(n, rows, cols, fmt, gen, device, chunk=16):
         elif fmt == "fp8row":
             a, s = Q.quantize_fp8_row(w)
             b = None
+        elif fmt == "bf16":   # unquantized experts
+            a, s, b = w.to(torch.bfloat16), None, None
         else:
             raise ValueError(fmt)
         ws.append(a)
@@ -76,10 +78,11 @@ def _quant_stack(n, rows, cols, fmt, gen, device, chunk=16):
         bs.append(b)
         del w
     w = torch.cat(ws)
-    s = torch.cat(ss)
+    s = None if ss[0] is None else torch.cat(ss)
     b = None if bs[0] is None else torch.cat(bs)
     mode, bits, group = {"affine4": (QUANT_AFFINE, 4, 64), "affine8": (QUANT_AFFINE, 8, 64),
-                         "mxfp4": (QUANT_MXFP4, 4, 32), "fp8row": (QUANT_FP8_ROW, 8, 0)}[fmt]
+                         "mxfp4": (QUANT_MXFP4, 4, 32), "fp8row": (QUANT_FP8_ROW, 8, 0),
+                         "bf16": (QUANT_NONE, 16, 0)}[fmt]
     return QWeight(w, s, b, rows, cols, mode, bits, group)
 
 

@@ -187,6 +187,16 @@ pub fn batchBuild(ctx: Context, tokens: []const u32, seq_lens: []const i32, base
     try check(c.dmoe_batch_build(@ptrCast(@alignCast(out_tokens.ptr)), @ptrCast(@alignCast(out_positions.ptr)), if (out_mask) |m| @ptrCast(@alignCast(m.ptr)) else null, null, tokens.ptr, seq_lens.ptr, base_pos.ptr, @intCast(seq_lens.len), @intCast(tokens.len), ctx.ws, ctx.stream));
 }
 
+/// quantize_mod.gatherQmm (call shape at src/models/deepseek_v4.zig:976): row r of the result is x[lhs[r] or r]
+/// times the transposed matrix rhs[r] of the stack `q` (device memory). With `q.mode = c.DMOE_QUANT_NONE`, `q.bits = 16`
+/// and no scales this is ops.gatherMm on the untransposed [E, out, in] bf16 weights (:978).
+pub fn gatherQmm(ctx: Context, x: DeviceArray(u16), q: *const c.dmoe_qweight, lhs_indices: ?DeviceArray(u32), rhs_indices: DeviceArray(u32), sorted: bool) Error!DeviceArray(u16) {
+    const out = try DeviceArray(u16).alloc(rhs_indices.len * @as(usize, @intCast(q.rows)));
+    errdefer out.deinit();
+    try check(c.dmoe_gather_qmm(@ptrCast(@alignCast(out.ptr)), @ptrCast(@alignCast(x.ptr)), q, if (lhs_indices) |l| @ptrCast(@alignCast(l.ptr)) else null, @ptrCast(@alignCast(rhs_indices.ptr)), @intCast(rhs_indices.len), @intFromBool(sorted), ctx.ws, ctx.stream));
+    return out;
+}
+
 /// DSV4HyperConn.post / mhcPost (src/models/deepseek_v4.zig:2450-2499) when `hc_mult` > 0, the plain residual add
 /// of the block (:2674) when it is 0 (mixes null).
 pub fn blockPost(ctx: Context, out: DeviceArray(u16), ffn_out: DeviceArray(u16), residual: DeviceArray(u16), post_mix: ?DeviceArray(f32), comb_mix: ?DeviceArray(f32), n_tokens: usize, dim: usize, hc_mult: usize) Error!void {

@@ -46,7 +46,9 @@ typedef enum {
 typedef enum {
     DMOE_QUANT_AFFINE = 0, /* bits 4|8, group 32|64|128, bf16 scales + bf16 biases (biases nullable = 0) */
     DMOE_QUANT_MXFP4 = 1,  /* E2M1 nibbles, one E8M0 byte per 32 values, no biases                      */
-    DMOE_QUANT_FP8_ROW = 2 /* E4M3FN bytes, one f32 scale per output row, no biases                     */
+    DMOE_QUANT_FP8_ROW = 2, /* E4M3FN bytes, one f32 scale per output row, no biases                    */
+    DMOE_QUANT_NONE = 3     /* unquantized bf16 [n_mats, rows, cols]; bits 16, no scales, no biases: the float
+                               arm of dispatchGatherMm / ops.gatherMm (deepseek_v4.zig:969-979)           */
 } dmoe_quant_mode;
 
 typedef struct dmoe_stream_ { void *ctx; } dmoe_stream;           /* ctx = hipStream_t */
@@ -54,7 +56,8 @@ typedef struct dmoe_workspace_ { void *ctx; } dmoe_workspace;     /* grow-only d
 typedef struct dmoe_layer_ { void *ctx; } dmoe_layer;             /* resident expert weights of one MoE layer */
 typedef struct dmoe_gate_ { void *ctx; } dmoe_gate;               /* resident router of one MoE layer */
 
-/* "affine" -> DMOE_QUANT_AFFINE, "mxfp4" -> DMOE_QUANT_MXFP4, "fp8" -> DMOE_QUANT_FP8_ROW; -1 if unknown */
+/* "affine" -> DMOE_QUANT_AFFINE, "mxfp4" -> DMOE_QUANT_MXFP4, "fp8" -> DMOE_QUANT_FP8_ROW,
+ * "none" | "bf16" -> DMOE_QUANT_NONE; -1 if unknown */
 int dmoe_quant_mode_from_string(const char *name);
 
 /* ---- runtime ------------------------------------------------------------------ */
@@ -174,15 +177,16 @@ int dmoe_pack(uint32_t *d_out_order, uint32_t *d_out_inv_order, uint32_t *d_out_
  *   affine : w u32 [n, rows, cols*bits/32]; scales, biases bf16 [n, rows, cols/group_size]
  *   mxfp4  : w u32 [n, rows, cols/8];       scales u8 [n, rows, cols/32]; biases NULL
  *   fp8row : w u8  [n, rows, cols];         scales f32 [n, rows];         biases NULL
+ *   none   : w bf16 [n, rows, cols] (rows % 4 == 0, cols % 8 == 0); scales, biases NULL
  * (QuantizedWeight / QuantConfig of mlx-zig as used at deepseek_v4.zig:474-481, :971-976) */
 typedef struct {
     const void *w;
-    const void *scales;
+    const void *scales; /* NULL for DMOE_QUANT_NONE */
     const void *biases; /* nullable */
     int n_mats, rows, cols;
     int mode;           /* dmoe_quant_mode */
-    int bits;           /* 4 | 8 (affine), 4 (mxfp4), 8 (fp8row) */
-    int group_size;     /* 32 | 64 | 128 (affine), 32 (mxfp4), ignored (fp8row) */
+    int bits;           /* 4 | 8 (affine), 4 (mxfp4), 8 (fp8row), 16 (none) */
+    int group_size;     /* 32 | 64 | 128 (affine), 32 (mxfp4), ignored (fp8row, none) */
 } dmoe_qweight;
 
 /* mlx_dequantize(..., dtype = bf16) (deepseek_v4_loader.zig:129): d_out bf16 [rows, cols] of matrix
@@ -194,7 +198,10 @@ int dmoe_dequantize(uint16_t *d_out, const dmoe_qweight *qw, int mat_index, dmoe
  * (call shape deepseek_v4.zig:976, expert_preload.zig:265; mlx.core.gather_qmm):
  *   out[r, :] = x[lhs ? lhs[r] : r, :] . dequant(W[rhs[r]])^T     r < R
  * x bf16 [*, cols], out bf16 [R, rows], f32 accumulation. d_lhs_indices nullable. `sorted` != 0 promises
- * non-decreasing rhs_indices (as the reference's sorted=true); the result is the same either way. */
+ * non-decreasing rhs_indices (as the reference's sorted=true); the result is the same either way.
+ * With qw->mode == DMOE_QUANT_NONE (bf16 weights [n_mats, rows, cols], bits 16, no scales) this is
+ * ops.gatherMm(x, w^T, null, rhs_indices, sorted) of the unquantized arm (deepseek_v4.zig:978): pass the
+ * [E, out, in] weight itself, not its transposed view. */
 int dmoe_gather_qmm(uint16_t *d_out, const uint16_t *d_x, const dmoe_qweight *qw,
                     const uint32_t *d_lhs_indices, const uint32_t *d_rhs_indices, int R, int sorted,
                     dmoe_workspace ws, dmoe_stream s);

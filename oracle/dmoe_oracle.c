@@ -488,6 +488,8 @@ static inline size_t qmat_words_per_row(const orc_qmat *m) {
  * fp8row: e4m3(byte) * row_scale in f32. */
 float orc_dequant_value(const orc_qmat *m, int mi, int row, int col) {
     size_t r = (size_t)mi * m->rows + row;
+    if (m->mode == ORC_NONE) /* unquantized bf16 weights: dispatchGatherMm's float arm, deepseek_v4.zig:978 */
+        return orc_bf16_to_f32(((const uint16_t *)m->w)[r * m->cols + col]);
     if (m->mode == ORC_FP8_ROW) {
         const uint8_t *w = (const uint8_t *)m->w;
         const float *sc = (const float *)m->scales;

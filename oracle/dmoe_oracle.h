@@ -42,14 +42,15 @@
 extern "C" {
 #endif
 
-enum { ORC_AFFINE = 0, ORC_MXFP4 = 1, ORC_FP8_ROW = 2 };
+enum { ORC_AFFINE = 0, ORC_MXFP4 = 1, ORC_FP8_ROW = 2, ORC_NONE = 3 };
 enum { ORC_SCORE_SOFTMAX = 0, ORC_SCORE_SIGMOID = 1, ORC_SCORE_SQRTSOFTPLUS = 2 };
 enum { ORC_SMELT_UNIFORM = 0, ORC_SMELT_FIRST = 1 };
 
 /* One quantized matrix stack [n_mats, rows, cols] in MLX layout.
  * affine : w u32 [n, rows, cols*bits/32], scales/biases bf16 [n, rows, cols/group]
  * mxfp4  : w u32 [n, rows, cols/8], scales u8 (E8M0) [n, rows, cols/32], biases NULL
- * fp8row : w u8  [n, rows, cols] (E4M3FN), scales f32 [n, rows], biases NULL */
+ * fp8row : w u8  [n, rows, cols] (E4M3FN), scales f32 [n, rows], biases NULL
+ * none   : w bf16 [n, rows, cols] as it is (the unquantized arm, ops.gatherMm), scales/biases NULL */
 typedef struct {
     const void *w;
     const void *scales;

@@ -14,7 +14,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "_build", "libdmoe_oracle.so")
 
-AFFINE, MXFP4, FP8_ROW = 0, 1, 2
+AFFINE, MXFP4, FP8_ROW, NONE = 0, 1, 2, 3
 SCORE_SOFTMAX, SCORE_SIGMOID, SCORE_SQRTSOFTPLUS = 0, 1, 2
 SMELT_UNIFORM, SMELT_FIRST = 0, 1
 
@@ -87,7 +87,11 @@ class QMat:
 
     def __init__(self, w, scales, biases, rows, cols, mode, bits, group):
         self.mode, self.bits, self.group, self.rows, self.cols = mode, bits, group, rows, cols
-        if mode == FP8_ROW:
+        if mode == NONE:
+            self.w = _c(w, np.uint16)
+            self.scales = None
+            self.biases = None
+        elif mode == FP8_ROW:
             self.w = _c(w, np.uint8)
             self.scales = _c(scales, np.float32)
             self.biases = None

@@ -22,6 +22,8 @@ def bf16_to_f32(t):
 def qmat(qw):
     """capi.QWeight (torch, any device) -> oracle.QMat (numpy)"""
     w = qw.w.detach().cpu().contiguous()
+    if qw.mode == capi.QUANT_NONE:
+        return oracle.QMat(bf16_bits(w), None, None, qw.rows, qw.cols, oracle.NONE, 16, 0)
     s = qw.scales.detach().cpu().contiguous()
     b = None if qw.biases is None else qw.biases.detach().cpu().contiguous()
     if qw.mode == capi.QUANT_FP8_ROW:

@@ -301,6 +301,31 @@ static void test_block_post(Context &ctx) {
     for (int d = 0; d < H; ++d) EXPECT(sv[d] == bf16(2.0f * (d + 1)));
 }
 
+// ops.gatherMm on unquantized experts with values exact in bf16: expert e is (e + 1) * [identity rows | zeros],
+// so row r of the result is (rhs[r] + 1) * x[lhs[r]][0..rows)
+static void test_gather_mm(Context &ctx) {
+    const int E = 3, rows = 8, cols = 16, R = 5;
+    std::vector<uint16_t> w((size_t)E * rows * cols, bf16(0.0f)), x((size_t)R * cols);
+    for (int e = 0; e < E; ++e)
+        for (int n = 0; n < rows; ++n) w[((size_t)e * rows + n) * cols + n] = bf16((float)(e + 1));
+    for (int r = 0; r < R; ++r)
+        for (int k = 0; k < cols; ++k) x[(size_t)r * cols + k] = bf16((float)(r * 16 + k));
+    const uint32_t rhs[R] = {2, 0, 1, 1, 2}, lhs[R] = {4, 3, 2, 1, 0};
+    Array wa = Array::fromData(ctx, w.data(), {E, rows, cols}, DType::bfloat16);
+    Array xa = Array::fromData(ctx, x.data(), {R, cols}, DType::bfloat16);
+    Array ra = Array::fromData(ctx, rhs, {R}, DType::uint32), la = Array::fromData(ctx, lhs, {R}, DType::uint32);
+    auto plain = ops::gatherMm(ctx, xa, wa, nullptr, ra, false).dataSlice<uint16_t>();
+    auto gathered = ops::gatherMm(ctx, xa, wa, &la, ra, false).dataSlice<uint16_t>();
+    for (int r = 0; r < R; ++r)
+        for (int n = 0; n < rows; ++n) {
+            EXPECT(from_bf16(plain[(size_t)r * rows + n]) == (float)((rhs[r] + 1) * (r * 16 + n)));
+            EXPECT(from_bf16(gathered[(size_t)r * rows + n]) == (float)((rhs[r] + 1) * (lhs[r] * 16 + n)));
+        }
+    const QuantizedWeight q = QuantizedWeight::unquantized(wa.data(), E, rows, cols);
+    auto back = quantize_mod::dequantize(ctx, q, 1).dataSlice<uint16_t>();
+    for (int i = 0; i < rows * cols; ++i) EXPECT(back[i] == w[(size_t)rows * cols + i]);
+}
+
 int main() {
     try {
         Context ctx(0);
@@ -311,6 +336,7 @@ int main() {
         test_layer_closed_form(ctx);
         test_gate_from_hidden(ctx);
         test_block_post(ctx);
+        test_gather_mm(ctx);
         ctx.synchronize();
     } catch (const Error &e) {
         std::printf("dmoe::Error %d: %s\n", e.code, e.what());

@@ -7,7 +7,7 @@ import torch
 
 from dmlx_amd import quantize as Q
 from dmlx_amd import workloads
-from dmlx_amd.capi import QUANT_AFFINE, QUANT_FP8_ROW, QUANT_MXFP4, QWeight
+from dmlx_amd.capi import QUANT_AFFINE, QUANT_FP8_ROW, QUANT_MXFP4, QUANT_NONE, QWeight
 from tests.helpers import bf16_bits, max_abs_rel, oracle_forward, qmat, to_np_u32
 
 pytestmark = pytest.mark.gpu
@@ -33,11 +33,13 @@ def _stack(fmt, n, rows, cols, seed):
     if fmt == "mxfp4":
         a, s = Q.quantize_mxfp4(w)
         return QWeight(a, s, None, rows, cols, QUANT_MXFP4, 4, 32)
+    if fmt == "bf16":     # unquantized experts (the float arm of dispatchGatherMm)
+        return QWeight(w.to(torch.bfloat16), None, None, rows, cols, QUANT_NONE, 16, 0)
     a, s = Q.quantize_fp8_row(w)
     return QWeight(a, s, None, rows, cols, QUANT_FP8_ROW, 8, 0)
 
 
-FORMATS = ["affine4", "affine4g32", "affine4g128", "affine8", "mxfp4", "fp8row"]
+FORMATS = ["affine4", "affine4g32", "affine4g128", "affine8", "mxfp4", "fp8row", "bf16"]
 
 
 @pytest.mark.parametrize("fmt", FORMATS)
@@ -247,6 +249,42 @@ def test_prefill_configs_full_size(dmoe, orc, ws, config):
     assert err_paths < OUT_TOL, (wl.name, "prefill kernels against decode kernels", err_paths)
     print(f"[parity] {wl.name}: T={wl.T} rows/expert max {counts.max()} min {counts[live].min()} "
           f"sample err {err:.3e}, alone {err_alone:.3e}, prefill vs decode {err_paths:.3e}")
+    layer.close()
+
+
+@pytest.mark.parametrize("config,scale", [(1, 0.25), (3, 0.125), (4, 0.25)])
+def test_unquantized_experts_layer(dmoe, orc, ws, config, scale):
+    """A layer whose experts (and shared expert) are plain bf16 matrices: the float arm of dispatchGatherMm
+    (deepseek_v4.zig:978, ops.gatherMm) and of DSV4Expert.expertMatmul, at a decode and at two prefill sizes."""
+    wl = workloads.make(config, scale=scale)
+    wl.gate, wl.up = _stack("bf16", wl.E, wl.F, wl.D, 21), _stack("bf16", wl.E, wl.F, wl.D, 22)
+    wl.down = _stack("bf16", wl.E, wl.D, wl.F, 23)
+    if wl.shared is not None:
+        wl.shared = (_stack("bf16", 1, wl.F, wl.D, 24), _stack("bf16", 1, wl.F, wl.D, 25), _stack("bf16", 1, wl.D, wl.F, 26))
+    _check_layer(dmoe, orc, ws, wl)
+
+
+def test_unquantized_tiny_model_shape(dmoe, orc, ws):
+    """The shape of the reference's own DSV4 smoke tests (src/tests/deepseek_v4_tests.zig:398-610): 2 experts, top-2,
+    D=16, F=8, float weights. All-zero weights must give zeros (finite); random ones must match the oracle. F=8 makes
+    the down projection's reduction half an MFMA step, D=16 keeps the weights in their row-major layout."""
+    E, K, D, F, T = 2, 2, 16, 8, 5
+    g = torch.Generator(device="cuda").manual_seed(4)
+    x = torch.randn((T, D), generator=g, device="cuda").to(torch.bfloat16)
+    idx = torch.tensor([[0, 1], [1, 0], [0, 1], [1, 0], [0, 1]], dtype=torch.int32, device="cuda")
+    w = torch.full((T, K), 0.5, dtype=torch.float32, device="cuda")
+    zeros = lambda r, c: QWeight(torch.zeros((E, r, c), dtype=torch.bfloat16, device="cuda"), None, None, r, c, QUANT_NONE, 16, 0)
+    layer = dmoe.Layer(D, F, K, zeros(F, D), zeros(F, D), zeros(D, F))
+    out = layer.forward(x, idx, w, ws)
+    assert out.shape == (T, D) and bool((out == 0).all())
+    layer.close()
+    gate, up, down = _stack("bf16", E, F, D, 31), _stack("bf16", E, F, D, 32), _stack("bf16", E, D, F, 33)
+    for q in (gate, up, down):
+        q.w *= 40.0  # N(0, 0.8): outputs well above the bf16 rounding of a 16-term sum
+    layer = dmoe.Layer(D, F, K, gate, up, down)
+    out = layer.forward(x, idx, w, ws).float().cpu().numpy()
+    want = orc.moe_forward(bf16_bits(x), to_np_u32(idx), w.cpu().numpy(), qmat(gate), qmat(up), qmat(down))
+    assert max_abs_rel(out, want) < OUT_TOL, max_abs_rel(out, want)
     layer.close()
 
 

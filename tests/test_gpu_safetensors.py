@@ -43,13 +43,15 @@ def _layer_tensors(wl, layer_idx, with_shared):
     out = {}
     for proj, q in (("gate_proj", wl.gate), ("up_proj", wl.up), ("down_proj", wl.down)):
         out[base + f"switch_mlp.{proj}.weight"] = q.w
-        out[base + f"switch_mlp.{proj}.scales"] = q.scales
+        if q.scales is not None:
+            out[base + f"switch_mlp.{proj}.scales"] = q.scales
         if q.biases is not None:
             out[base + f"switch_mlp.{proj}.biases"] = q.biases
     if with_shared:
         for proj, q in zip(("gate_proj", "up_proj", "down_proj"), wl.shared):
             out[base + f"shared_experts.{proj}.weight"] = q.w[0]
-            out[base + f"shared_experts.{proj}.scales"] = q.scales[0]
+            if q.scales is not None:
+                out[base + f"shared_experts.{proj}.scales"] = q.scales[0]
             if q.biases is not None:
                 out[base + f"shared_experts.{proj}.biases"] = q.biases[0]
     return out
@@ -100,6 +102,41 @@ def test_smelt_subset_from_safetensors(dmoe, ws, tmp_path):
     assert disk.n_slots == int(mask.sum())
     idx, w = dmoe.gate_route(wl.scores, wl.bias, torch.from_numpy(mask).cuda(), wl.K, wl.renorm, wl.route_scale)
     assert mask[to_np_u32(idx)].all()
+    assert torch.equal(mem.forward(wl.x, idx, w, ws), disk.forward(wl.x, idx, w, ws))
+    mem.close()
+    disk.close()
+
+
+def test_unquantized_experts_from_safetensors(dmoe, ws, tmp_path):
+    """A float checkpoint: `switch_mlp.*.weight` are bf16 [E, rows, cols] and there are no scales (mode "none").
+    Whole layer with its shared expert, then a Smelt subset of the same file."""
+    wl = workloads.make(1, scale=0.125)
+    g = torch.Generator(device="cuda").manual_seed(8)
+    bf = lambda n, r, c: dmoe.QWeight((torch.randn((n, r, c), generator=g, device="cuda") * 0.02).to(torch.bfloat16),
+                                      None, None, r, c, dmoe.QUANT_NONE, 16, 0)
+    wl.gate, wl.up, wl.down = bf(wl.E, wl.F, wl.D), bf(wl.E, wl.F, wl.D), bf(wl.E, wl.D, wl.F)
+    wl.shared = (bf(1, wl.F, wl.D), bf(1, wl.F, wl.D), bf(1, wl.D, wl.F))
+    path = str(tmp_path / "float.safetensors")
+    write_safetensors(path, _layer_tensors(wl, 2, with_shared=True))
+    idx, w = dmoe.gate_route(wl.scores, wl.bias, None, wl.K, wl.renorm, wl.route_scale)
+    mem = dmoe.Layer(wl.D, wl.F, wl.K, wl.gate, wl.up, wl.down, swiglu_limit=wl.swiglu_limit, shared=wl.shared)
+    disk = dmoe.Layer.from_safetensors([path], 2, wl.K, "none", 0, 16, swiglu_limit=wl.swiglu_limit)
+    assert (disk.hidden, disk.ffn, disk.n_slots) == (wl.D, wl.F, wl.E)
+    assert torch.equal(mem.forward(wl.x, idx, w, ws), disk.forward(wl.x, idx, w, ws))
+    mem.close()
+    disk.close()
+    with pytest.raises(dmoe.DmoeError, match="scales not found"):
+        dmoe.Layer.from_safetensors([path], 2, wl.K, "affine", 64, 4)   # a float file is not an affine one
+    mask = np.zeros(wl.E, np.uint8)
+    mask[1::2] = 1
+    keep = torch.from_numpy(np.nonzero(mask)[0]).cuda()
+    sub = lambda q: dmoe.QWeight(q.w[keep].contiguous(), None, None, q.rows, q.cols, q.mode, q.bits, q.group_size)
+    mem = dmoe.Layer(wl.D, wl.F, wl.K, sub(wl.gate), sub(wl.up), sub(wl.down), swiglu_limit=wl.swiglu_limit,
+                     remap=list(dmoe.build_remap(mask)))
+    disk = dmoe.Layer.from_safetensors([path], 2, wl.K, "none", 0, 16, swiglu_limit=wl.swiglu_limit,
+                                       load_shared=False, resident_mask=mask.tolist())
+    assert disk.n_slots == int(mask.sum())
+    idx, w = dmoe.gate_route(wl.scores, wl.bias, torch.from_numpy(mask).cuda(), wl.K, wl.renorm, wl.route_scale)
     assert torch.equal(mem.forward(wl.x, idx, w, ws), disk.forward(wl.x, idx, w, ws))
     mem.close()
     disk.close()

@@ -7,8 +7,8 @@ import pytest
 import torch
 
 from dmlx_amd import quantize as Q
-from dmlx_amd.capi import QUANT_AFFINE, QUANT_FP8_ROW, QUANT_MXFP4, QWeight
-from tests.helpers import max_abs_rel, qmat
+from dmlx_amd.capi import QUANT_AFFINE, QUANT_FP8_ROW, QUANT_MXFP4, QUANT_NONE, QWeight
+from tests.helpers import bf16_bits, max_abs_rel, qmat
 
 
 # ---------------------------------------------------------------- router (moe_router.zig tests) ----
@@ -284,9 +284,11 @@ def test_affine_dequant_layout_and_rounding(orc, bits, group):
 def _small_layer(fmt, E=4, D=256, F=128, seed=11):
     g = torch.Generator().manual_seed(seed)
     mk = {"affine4": lambda w: Q.quantize_affine(w, 64, 4), "affine8": lambda w: Q.quantize_affine(w, 64, 8),
-          "mxfp4": lambda w: Q.quantize_mxfp4(w) + (None,), "fp8row": lambda w: Q.quantize_fp8_row(w) + (None,)}[fmt]
+          "mxfp4": lambda w: Q.quantize_mxfp4(w) + (None,), "fp8row": lambda w: Q.quantize_fp8_row(w) + (None,),
+          "bf16": lambda w: (w.to(torch.bfloat16), None, None)}[fmt]
     mode, bits, group = {"affine4": (QUANT_AFFINE, 4, 64), "affine8": (QUANT_AFFINE, 8, 64),
-                         "mxfp4": (QUANT_MXFP4, 4, 32), "fp8row": (QUANT_FP8_ROW, 8, 0)}[fmt]
+                         "mxfp4": (QUANT_MXFP4, 4, 32), "fp8row": (QUANT_FP8_ROW, 8, 0),
+                         "bf16": (QUANT_NONE, 16, 0)}[fmt]
     out = []
     for rows, cols in ((F, D), (F, D), (D, F)):
         w = torch.randn(E, rows, cols, generator=g) * 0.02
@@ -295,10 +297,12 @@ def _small_layer(fmt, E=4, D=256, F=128, seed=11):
     return out
 
 
-@pytest.mark.parametrize("fmt", ["affine4", "affine8", "mxfp4", "fp8row"])
+@pytest.mark.parametrize("fmt", ["affine4", "affine8", "mxfp4", "fp8row", "bf16"])
 def test_gather_qmm_reduces_to_dense_matmul(orc, fmt):
     gate, _, _ = _small_layer(fmt)
     qm = qmat(gate)
+    if fmt == "bf16":   # unquantized: the "dequantized" matrix is the matrix itself
+        np.testing.assert_array_equal(orc.dequantize(qm, 2), bf16_bits(gate.w[2]))
     rng = np.random.default_rng(2)
     R = 10
     x = rng.standard_normal((R, 256)).astype(np.float32)
