@@ -300,10 +300,17 @@ extern "C" int dmoe_layer_create_from_safetensors(dmoe_layer *out, const char *c
     d.score_before_down = o->score_before_down;
     d.weight_source = DMOE_WEIGHTS_COPY_FROM_HOST;
     if (o->load_shared && index.count(base + "shared_experts.gate_proj.weight")) {
-        const int smode = dmoe_quant_mode_from_string(o->shared_mode ? o->shared_mode : o->mode);
+        // Without an explicit shared_mode the file decides, by the reference's rule (deepseek_v4_loader.zig:1890-1892):
+        // biases present -> affine with the model's group size, scales only -> mxfp4 (group 32), neither -> float
+        int smode;
+        if (o->shared_mode) smode = dmoe_quant_mode_from_string(o->shared_mode);
+        else if (!index.count(base + "shared_experts.gate_proj.scales")) smode = DMOE_QUANT_NONE;
+        else smode = index.count(base + "shared_experts.gate_proj.biases") ? DMOE_QUANT_AFFINE : DMOE_QUANT_MXFP4;
         DMOE_REQUIRE(smode == DMOE_QUANT_AFFINE || smode == DMOE_QUANT_MXFP4 || smode == DMOE_QUANT_NONE,
                      "layer_create_from_safetensors: bad shared_mode");
-        const int sbits = o->shared_bits ? o->shared_bits : o->bits, sgroup = o->shared_group_size ? o->shared_group_size : o->group_size;
+        const int dbits = mode == DMOE_QUANT_NONE ? 4 : o->bits, dgroup = mode == DMOE_QUANT_NONE ? 64 : o->group_size;
+        const int sbits = smode == DMOE_QUANT_NONE ? 16 : o->shared_bits ? o->shared_bits : dbits;
+        const int sgroup = smode == DMOE_QUANT_MXFP4 ? 32 : o->shared_group_size ? o->shared_group_size : dgroup;
         DMOE_TRY(find_proj(index, base + "shared_experts.gate_proj", smode, sbits, sgroup, false, &d.shared_gate));
         DMOE_TRY(find_proj(index, base + "shared_experts.up_proj", smode, sbits, sgroup, false, &d.shared_up));
         DMOE_TRY(find_proj(index, base + "shared_experts.down_proj", smode, sbits, sgroup, false, &d.shared_down));

@@ -245,13 +245,16 @@ int dmoe_layer_destroy(dmoe_layer layer);
  * Shapes [E, rows, cols*bits/32] and [E, rows, cols/group]; D, F and E are read from them. */
 typedef struct {
     int top_k;
-    const char *mode;            /* "affine" | "mxfp4" (the reference passes "mxfp4", 32, 4; :318-321) */
+    const char *mode;            /* "affine" | "mxfp4" (the reference passes "mxfp4", 32, 4; :318-321) | "none":
+                                    float checkpoint, weights BF16 [E, rows, cols], no scales */
     int group_size, bits;
     float swiglu_limit;
     int score_before_down;
     int load_shared;             /* also load the shared expert when the files hold one */
-    const char *shared_mode;     /* NULL / 0 below: same as the routed experts */
-    int shared_group_size, shared_bits;
+    const char *shared_mode;     /* NULL: decided by the file as the reference's loader does
+                                    (deepseek_v4_loader.zig:1890-1892): biases present -> "affine", scales only ->
+                                    "mxfp4" with group 32, neither -> "none" */
+    int shared_group_size, shared_bits; /* 0: the routed experts' values */
     float shared_swiglu_limit;
     const uint8_t *resident_mask;/* nullable HOST u8 [n_experts_total]: Smelt, only experts with 1 are uploaded, in
                                     increasing id order; the router-id -> slot remap is built like
