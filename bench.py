@@ -210,8 +210,13 @@ def main():
         "config": {"workload": wl.name, "baseline_config": args.config, "tokens": wl.T, "hidden": wl.D,
                    "ffn": wl.F, "experts": wl.E_total, "resident_experts": wl.E, "top_k": wl.K,
                    "shared_expert": wl.shared is not None,
-                   "weights": {0: "affine", 1: "mxfp4", 2: "fp8row"}[wl.gate.mode] + f"-{wl.gate.bits}bit",
-                   "max_rows_per_expert": int(counts.max()), "request_lengths": wl.seg_lens},
+                   "weights": {0: "affine", 1: "mxfp4", 2: "fp8row", 3: "unquantized"}[wl.gate.mode] + f"-{wl.gate.bits}bit",
+                   "max_rows_per_expert": int(counts.max()),
+                   "experts_by_rows": {"0": int((counts == 0).sum()), "1-9": int(((counts >= 1) & (counts < 10)).sum()),
+                                       "10-99": int(((counts >= 10) & (counts < 100)).sum()),
+                                       "100-499": int(((counts >= 100) & (counts < 500)).sum()),
+                                       "500+": int((counts >= 500).sum())},
+                   "request_lengths": wl.seg_lens},
         "roofline": roof,
         "step": {"algorithmic_bytes": step_bytes, "algorithmic_flops": step_flops,
                  "hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
