@@ -8,7 +8,7 @@ GEMM + limited SwiGLU -> grouped down GEMM -> weighted combine + shared expert, 
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1]
 
---config selects the BASELINE configuration (default 1: the 64-sequence decode step the headline metric is
+--config selects the benchmark configuration (0..4, as listed in BASELINE.json) (default 1: the 64-sequence decode step the headline metric is
 quoted on; 3 = the 8k-token ragged prefill). `roofline` describes the dominant kernel of the step, timed
 with HIP events recorded inside the library on the launch stream; `cpu_baseline` is the CPU restatement of
 the dmlx/MLX op sequence (the oracle) timed on this box's host cores on a bounded sample.

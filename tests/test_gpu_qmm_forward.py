@@ -137,7 +137,7 @@ def _check_layer(dmoe, orc, ws, wl, check_h=True):
 
 
 def test_c0_small_layer_full_size(dmoe, orc, ws):
-    """BASELINE config 0 at its real size: 16 tokens, D=1024, E=8, top-2, F=2048, affine-4 g64, softmax scores
+    """Benchmark configuration 0 at its real size: 16 tokens, D=1024, E=8, top-2, F=2048, affine-4 g64, softmax scores
     renormalised over the top-k (MoERouter.topkRoute)."""
     wl = workloads.make(0)
     idx, w = dmoe.topk_route(wl.scores, wl.K, True)
@@ -194,7 +194,7 @@ def test_prefill_sized_batch_with_4bit_shared_expert(dmoe, orc, ws, config, T):
 
 
 def test_c1_decode_full_size(dmoe, orc, ws):
-    """BASELINE config 1 at full size (64 x 1 tokens, D=4096, 256 experts top-6 + shared, F=2048, affine-4)."""
+    """Benchmark configuration 1 at full size (64 x 1 tokens, D=4096, 256 experts top-6 + shared, F=2048, affine-4)."""
     wl = workloads.make(1)
     _check_layer(dmoe, orc, ws, wl, check_h=True)
 
@@ -207,7 +207,7 @@ def test_c2_decode_mxfp4_smelt_full_size(dmoe, orc, ws):
 
 @pytest.mark.parametrize("config", [3, 4])
 def test_prefill_configs_full_size(dmoe, orc, ws, config):
-    """BASELINE configs 3 (8192-token ragged prefill, Zipf routing, affine-4) and 4 (2080-token mixed batch, affine-8
+    """Benchmark configurations 3 (8192-token ragged prefill, Zipf routing, affine-4) and 4 (2080-token mixed batch, affine-8
     routed + FP8 shared expert) at full size. Routing and packing are compared bit for bit with the oracle on the
     whole batch. The oracle's FFN would take minutes on 49 152 rows, so the outputs are pinned two ways that do not
     depend on the batch size: a sample of 64 tokens (the rows of the most and of the least loaded experts, the
