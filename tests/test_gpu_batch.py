@@ -16,6 +16,23 @@ def _requests(seed, lens):
     return toks, base
 
 
+def test_batch_build_reference_cases(dmoe, ws, golden):
+    """The literal cases of the reference's batch builder tests (src/tests/batch_builder_tests.zig:61-316)."""
+    for case in golden["batch_builder"]["cases"]:
+        lens = [len(r["tokens"]) for r in case["requests"]]
+        flat = [t for r in case["requests"] for t in r["tokens"]]
+        d_tok, d_pos, d_mask, d_req = dmoe.batch_build(flat, lens, [r["base"] for r in case["requests"]], ws)
+        assert d_tok.numel() == case.get("total_tokens", sum(lens)) and int(d_req.max()) + 1 == case["num_requests"]
+        if case["tokens"] is not None:
+            np.testing.assert_array_equal(to_np_u32(d_tok), case["tokens"], err_msg=case["name"])
+        if case["positions"] is not None:
+            np.testing.assert_array_equal(d_pos.cpu().numpy(), case["positions"], err_msg=case["name"])
+        m = d_mask.cpu().numpy()
+        assert m.shape == (len(flat), len(flat))
+        for r, c, att in case["attending"]:
+            assert (m[r, c] == 0.0) == bool(att), (case["name"], r, c)
+
+
 @pytest.mark.parametrize("lens", [[5, 3, 1, 1], [512, 512, 1, 1, 1, 7], [1], [3, 0, 4], [129, 2]])
 def test_batch_build_matches_oracle(dmoe, orc, ws, lens):
     toks, base = _requests(3, lens)

@@ -375,6 +375,26 @@ def test_moe_forward_against_dense_float64(orc, fmt, before):
 
 # ---------------------------------------------------------------- batch builder --------------------------------
 
+def test_batch_builder_reference_cases(orc, golden):
+    """The literal expectations of src/tests/batch_builder_tests.zig: token order (prefill requests first), positions,
+    request count and the isAttending assertions (mask value 0 = attends, batch_builder.zig:253-256)."""
+    for case in golden["batch_builder"]["cases"]:
+        toks = [np.array(r["tokens"], np.uint32) for r in case["requests"]]
+        base = np.array([r["base"] for r in case["requests"]], np.int32)
+        flat, pos, offs = orc.batch_concat(toks, base)
+        lens = [len(t) for t in toks]
+        assert len(offs) - 1 == case["num_requests"], case["name"]
+        assert flat.size == case.get("total_tokens", sum(lens))
+        if case["tokens"] is not None:
+            np.testing.assert_array_equal(flat, case["tokens"], err_msg=case["name"])
+        if case["positions"] is not None:
+            np.testing.assert_array_equal(pos, case["positions"], err_msg=case["name"])
+        m = orc.batch_mask(lens)
+        assert m.shape == (flat.size, flat.size)
+        for r, c, att in case["attending"]:
+            assert (m[r, c] == 0.0) == bool(att), (case["name"], r, c)
+
+
 def test_batch_concat_and_mask_properties(orc):
     """batch_builder.zig:90-214 and Property 11 of src/tests/batch_builder_tests.zig: total_tokens is the
     sum of the request lengths, positions restart per request, requests never attend to each other."""
