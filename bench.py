@@ -28,7 +28,7 @@ COPY_PROBE_BYTES = 256 << 20  # --copy-probe: bytes read (and written) by each c
 # (scaled by the same counters' reading for the --copy-probe copies; profiles/hbm_traffic_gemm_kernels.txt).
 # A counter cannot be read from inside the timed run, so these are the recorded values for the default workloads.
 MEASURED_TRAFFIC = {(1, "gate_up+down"): 1509859000,
-                    (3, "gate_up"): 3520760000, (3, "down"): 2035244000}
+                    (3, "gate_up"): 4762998000, (3, "down"): 2571839000}
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 

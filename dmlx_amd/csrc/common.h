@@ -180,7 +180,7 @@ struct GemmArgs {
 constexpr int kSkinnyTileM = 32;          // most rows a skinny tile can hold (see qgemm_skinny_tile_m)
 constexpr int kSkinnyDenseTileM = 8;      // dense (one matrix) launches: small tiles, many workgroups per row block
 constexpr int kMfmaTileM = 128;
-constexpr int kMfmaWideTileM = 256;
+constexpr int kMfmaWideTileM = 128;
 int launch_qgemm_skinny(const GemmArgs &g, hipStream_t st);
 // gate/up + down of one tile list in one launch (down waits per tile for gate/up); gu.tile_done must be zeroed
 bool qgemm_skinny_pair_supports(const GemmArgs &gu, const GemmArgs &dn);

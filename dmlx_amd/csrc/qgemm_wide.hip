@@ -1,28 +1,33 @@
 // Grouped quantized GEMM, wide MFMA path (prefill, 4-bit formats in the packed resident layout).
 //
-// Same decomposition as the 128-row MFMA kernel (one workgroup = one tile of ONE expert segment against a strip
-// of output columns, each wavefront dequantizes its own 64 weight rows straight into the A operand of
-// v_mfma_f32_32x32x16_bf16), but with tiles of up to 256 rows: every decoded weight fragment then feeds eight
-// matrix instructions instead of four, which halves the decode arithmetic per MFMA -- the vector ALU, not the
-// matrix core, is what bounds the 128-row kernel. 256 rows x 64 columns of f32 accumulators fill all 256
-// accumulation registers of a wavefront, so everything else has to be lean:
+// One workgroup (4 wavefronts) = one tile of up to 128 rows of ONE expert segment against a strip of output columns;
+// each wavefront dequantizes its own 64 weight rows straight into the A operand of v_mfma_f32_32x32x16_bf16 and
+// holds 128 x 64 f32 accumulators. The kernel is built so that TWO workgroups fit a compute unit (at most 256
+// registers per wavefront, 64 KiB of LDS): a lone wavefront on a SIMD issues a vector instruction only every ~5
+// cycles, two wavefronts every ~2.8, and the 4-bit decode (2.9 vector instructions per weight) is what this kernel
+// is bound by. A variant with 256-row tiles (every decoded fragment feeds eight MFMAs instead of four, but one
+// wavefront per SIMD: all 512 registers, 128 KiB of LDS) measured 5 % slower on the 8k-token ragged prefill.
+// Differences from the 8-bit / MLX-layout kernel in qgemm_mfma.hip:
 //
 //  * Activations go from global memory into LDS without passing through registers (global_load_lds_dwordx4).
 //    One such instruction moves 1 KiB: 8 rows x 128 bytes (one reduction step of 64 bf16). Inside that KiB the
 //    16-byte pieces of row r are stored at position piece ^ r, so that the MFMA operand reads (32 rows at the
 //    same reduction offset) hit 32 different banks; the swizzle costs nothing because each lane picks its
 //    global source address freely.
-//  * Four LDS buffers of one reduction step each (4 x 32 KiB): while step s computes, the loads of step s+2
+//  * Four LDS buffers of one reduction step each (4 x 16 KiB): while step s computes, the loads of step s+2
 //    are in flight. The compiler does not know about these loads (they are issued from inline assembly), so
 //    their completion is tracked by hand: VMEM operations return in order, hence "at most MT operations
 //    outstanding" three quarters into step s implies that everything issued before this step's own MT loads
 //    -- in particular the loads of step s+1 -- has landed. One s_barrier per step then publishes the buffer.
+//  * The same in-order rule means a deep register ring of weight loads buys nothing (any wait for a staging request
+//    also waits for every older weight load), so the weights of only two steps are in flight, which is what
+//    keeps the wavefront under 256 registers.
 //  * Activation fragments are single-buffered (except for tiles of at most 64 rows): the fragment of row tile mt
 //    is reloaded for the next MFMA group right after its last use in this one, 2*MT-1 units before it is needed
 //    again.
 //
-// The reduction loop is software-pipelined exactly like the 128-row kernel: units of [one MFMA | a slice of the
-// decode of the next step's weights] separated by scheduling barriers.
+// The reduction loop is software-pipelined like the other MFMA kernel: units of [one MFMA | a slice of the decode
+// of the next step's weights] separated by scheduling barriers.
 #include <type_traits>
 
 #include "common.h"
@@ -31,7 +36,8 @@
 namespace dmoe {
 
 constexpr int kWideWaves = 4;
-constexpr int kWideRing = 4;                              // weight steps in registers = LDS activation buffers
+constexpr int kWideRing = 4;                              // LDS activation buffers = steps per unrolled trip
+constexpr int kWideWRing = 2;                             // weight steps held in registers (see the header)
 constexpr int kWideBufBytes = kMfmaWideTileM * 128;       // one reduction step (64 bf16) of every row of the tile
 constexpr size_t kWideLdsBytes = (size_t)kWideRing * kWideBufBytes;
 
@@ -67,8 +73,8 @@ __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint
         if (n >= n_out) n = n_out - 1;
         cs[nt].init(b, e, (on ? base : 0) >> 5, ln, h, n); // a switched-off tile aliases valid memory, never stored
     }
-    uint4 ring_raw[kWideRing][NT];
-    uint32_t ring_sb[kWideRing][NT][2];
+    uint4 ring_raw[kWideWRing][NT];
+    uint32_t ring_sb[kWideWRing][NT][2];
     auto load_b = [&](int step, int slot_) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
@@ -78,7 +84,7 @@ __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint
         }
     };
 #pragma unroll
-    for (int j = 0; j < kWideRing; ++j) load_b(j < n_steps ? j : n_steps - 1, j);
+    for (int j = 0; j < kWideWRing; ++j) load_b(j < n_steps ? j : n_steps - 1, j);
 
     // ---- activation staging -------------------------------------------------------------------------------
     // operation i of this wavefront moves rows (wave + 4 i) * 8 .. + 7; lane = (row r8 of the eight, position c),
@@ -164,9 +170,9 @@ __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint
 #pragma unroll
         for (int j = 0; j < kWideRing; ++j) {
             const int s = s0 + j;
-            const int s_ahead = s + kWideRing < n_steps ? s + kWideRing : n_steps - 1;
-            load_b(s_ahead, j); // slot j was decoded one step ago
-            const int slot_next = (j + 1) % kWideRing, which = j & 1, buf_next = (j + 1) % kWideRing;
+            const int s_ahead = s + kWideWRing < n_steps ? s + kWideWRing : n_steps - 1;
+            load_b(s_ahead, j % kWideWRing); // this slot was decoded one step ago
+            const int slot_next = (j + 1) % kWideWRing, which = j & 1, buf_next = (j + 1) % kWideRing;
             const bool stage = s + AHEAD < n_steps; // uniform
             Meta meta_next[NT];
 #pragma unroll
@@ -270,8 +276,8 @@ __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint
 }
 
 template <typename Fmt, bool GATE_UP>
-__global__ __launch_bounds__(kWideWaves * 64) void qgemm_wide_kernel(GemmArgs g) {
-    extern __shared__ __attribute__((aligned(1024))) uint8_t wide_lds[]; // [kWideRing][256 rows][128 bytes], swizzled
+__global__ __launch_bounds__(kWideWaves * 64, 2) void qgemm_wide_kernel(GemmArgs g) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t wide_lds[]; // [kWideRing][128 rows][128 bytes], swizzled
     Tile t;
     // Workgroups go to the eight XCDs round-robin in launch order. All column strips of a tile are given to ONE XCD
     // (tile = 8 * (k / strips) + xcd for the k-th workgroup of that XCD), so the tile's activations are fetched into one
@@ -297,8 +303,6 @@ __global__ __launch_bounds__(kWideWaves * 64) void qgemm_wide_kernel(GemmArgs g)
     else if (mt == 2) wide_tile<Fmt, GATE_UP, 2>(g, t, wide_lds, strip);
     else if (mt == 3) wide_tile<Fmt, GATE_UP, 3>(g, t, wide_lds, strip);
     else if (mt == 4) wide_tile<Fmt, GATE_UP, 4>(g, t, wide_lds, strip);
-    else if (mt <= 6) wide_tile<Fmt, GATE_UP, 6>(g, t, wide_lds, strip);
-    else wide_tile<Fmt, GATE_UP, 8>(g, t, wide_lds, strip);
 }
 
 bool qgemm_wide_supports(const QView &b) {
