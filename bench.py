@@ -28,7 +28,7 @@ COPY_PROBE_BYTES = 256 << 20  # --copy-probe: bytes read (and written) by each c
 # (scaled by the same counters' reading for the --copy-probe copies; profiles/hbm_traffic_gemm_kernels.txt).
 # A counter cannot be read from inside the timed run, so these are the recorded values for the default workloads.
 MEASURED_TRAFFIC = {(1, "gate_up+down"): 1509859000,
-                    (3, "gate_up"): 4762998000, (3, "down"): 2571839000}
+                    (3, "gate_up"): 3667158000, (3, "down"): 2016777000}
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 
@@ -168,7 +168,16 @@ def main():
         (a.rows, a.cols, a.mode, a.bits, a.group_size) == (b.rows, b.cols, b.mode, b.bits, b.group_size)
         for a, b in ((sh[0], wl.gate), (sh[1], wl.up), (sh[2], wl.down)))
     k_experts, k_rows = U + (1 if folded else 0), rows + (wl.T if folded else 0)
-    gu_bytes = k_experts * gate_up_w + wl.T * wl.D * 2 + k_rows * wl.F * 2
+    # Prefill on packed 4-bit weights: each grouped GEMM is two launches on one tile list. The matrix-core kernel (the
+    # dominant one, timed as the gate_up / down stage) takes the tiles above 32 rows; an expert's rows are cut into
+    # tiles of 128, so only a remainder of at most 32 rows goes to the weight-streaming kernel (stages *_small).
+    split = (not decode) and stages.get("gate_up_small", 0.0) > 0.0
+    if split:
+        c = counts.to(torch.int64)
+        rem = c % 128
+        wide = c - torch.where(rem <= 32, rem, torch.zeros_like(rem))
+        k_experts, k_rows = int((wide > 0).sum()), int(wide.sum())
+    gu_bytes = k_experts * gate_up_w + min(wl.T, k_rows) * wl.D * 2 + k_rows * wl.F * 2
     dn_bytes = k_experts * down_w + k_rows * wl.F * 2 + k_rows * wl.D * 2
     gu_flops, dn_flops = 2.0 * k_rows * 2 * wl.D * wl.F, 2.0 * k_rows * wl.D * wl.F
     # decode steps run both GEMMs as ONE launch (a down workgroup waits for its own tile's gate/up workgroups): the
@@ -192,10 +201,11 @@ def main():
                 "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None}
     roof["traffic"] = MEASURED_TRAFFIC.get((args.config, kern))
     roof["measured_peaks"] = measured_peaks(torch)
-    # prefill with packed 4-bit weights: the stage is two launches on one tile list (matrix-core kernel for the tiles
-    # above 32 rows, weight-streaming kernel for the rest); kernel_ms is the stage, the sum of the two
     launches = (["qgemm_skinny_kernel (gate/up and down tiles in one launch)"] if paired else ["qgemm_skinny_kernel"] if decode else
-                ["qgemm_wide_kernel", "qgemm_skinny_kernel"] if wl.gate.mode in (0, 1) and wl.gate.bits == 4 else ["qgemm_mfma_kernel"])
+                ["qgemm_wide_kernel"] if split else ["qgemm_mfma_kernel"])
+    if split:
+        roof["rows_in_launch"] = k_rows
+        roof["small_tile_launch_ms"] = stages[kern + "_small"]
     roof.update({"kernel": f"grouped {kern} GEMM ({'small-M' if decode else 'MFMA'} path)", "launches": launches, "kernel_ms": k_ms,
                  "algorithmic_bytes": k_bytes, "algorithmic_flops": k_flops, "live_experts": U,
                  "shared_expert_in_launch": bool(folded)})

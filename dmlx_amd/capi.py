@@ -126,7 +126,7 @@ class Workspace:
     def set_wait_limit(self, polls):
         check(lib().dmoe_workspace_set_wait_limit(self.h, C.c_uint(polls)))
 
-    STAGES = ("route", "pack", "gate_up", "down", "shared", "combine")
+    STAGES = ("route", "pack", "gate_up", "down", "shared", "combine", "gate_up_small", "down_small")
 
     def set_stage_timing(self, enabled):
         check(lib().dmoe_workspace_set_stage_timing(self.h, int(enabled)))

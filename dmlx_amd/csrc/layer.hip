@@ -326,11 +326,29 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
             return DMOE_OK;
         }
     }
+    if (small_rows > 0) { // stage timing on: the four launches in a row, each its own stage
+        GemmArgs gu_small = gu, dn_small = dn, gu_big = gu, dn_big = dn;
+        gu_small.max_rows = dn_small.max_rows = small_rows;
+        gu_big.min_rows = dn_big.min_rows = small_rows + 1;
+        DMOE_TRY(stage_begin(w, DMOE_STAGE_GATE_UP, st));
+        DMOE_TRY(launch_qgemm_mfma(gu_big, st));
+        DMOE_TRY(stage_end(w, DMOE_STAGE_GATE_UP, st));
+        DMOE_TRY(stage_begin(w, DMOE_STAGE_GATE_UP_SMALL, st));
+        DMOE_TRY(launch_qgemm_skinny(gu_small, st));
+        DMOE_TRY(stage_end(w, DMOE_STAGE_GATE_UP_SMALL, st));
+        DMOE_TRY(stage_begin(w, DMOE_STAGE_DOWN, st));
+        DMOE_TRY(launch_qgemm_mfma(dn_big, st));
+        DMOE_TRY(stage_end(w, DMOE_STAGE_DOWN, st));
+        DMOE_TRY(stage_begin(w, DMOE_STAGE_DOWN_SMALL, st));
+        DMOE_TRY(launch_qgemm_skinny(dn_small, st));
+        DMOE_TRY(stage_end(w, DMOE_STAGE_DOWN_SMALL, st));
+        return DMOE_OK;
+    }
     DMOE_TRY(stage_begin(w, DMOE_STAGE_GATE_UP, st));
-    DMOE_TRY(run_gemm(gu, f.small, st, small_rows));
+    DMOE_TRY(run_gemm(gu, f.small, st));
     DMOE_TRY(stage_end(w, DMOE_STAGE_GATE_UP, st));
     DMOE_TRY(stage_begin(w, DMOE_STAGE_DOWN, st));
-    DMOE_TRY(run_gemm(dn, f.small, st, small_rows));
+    DMOE_TRY(run_gemm(dn, f.small, st));
     DMOE_TRY(stage_end(w, DMOE_STAGE_DOWN, st));
     return DMOE_OK;
 }

@@ -63,7 +63,7 @@ struct Meta {
 
 struct FmtAffine4 {
     static constexpr int kVals = 32;
-    static constexpr int kDecodeOps = 116; // vector instructions to decode one chunk (scheduling hint only)
+    static constexpr int kDecodeOps = 96; // vector instructions to decode one chunk (scheduling hint only)
     static constexpr bool kRowScale = false;
     __device__ static __forceinline__ void load_meta_raw(const QView &q, const uint8_t *row_s, const uint8_t *row_b,
                                                          int k0, uint32_t *sb) {
@@ -117,18 +117,36 @@ struct FmtAffine4 {
         decode_word(raw.w, m, out + 12);
     }
     __device__ static __forceinline__ void decode_fast(const uint4 &raw, Meta m, uint32_t *out) { decode(raw, m, out); }
-    // values (2q, 2q+1) of the chunk only, for callers that spread the decode between other instructions; q must
-    // run upwards through a chunk, `st` carries the two nibble planes of the current word between calls. The planes
-    // are made opaque so that the byte picks compile to v_cvt_f32_ubyteN instead of a bit-field extract each.
+    // Values (2q, 2q+1) of the chunk only, for callers that spread the decode between other instructions; q must
+    // run upwards through a chunk. `m` must come from pair_meta() and `st` from pair_state(): code c becomes the f16
+    // number 1024 + c by OR-ing it into 0x6400, v_fma_mix_f32 takes that half-word straight into an f32 fma, and
+    // (1024 + c) * s + (b - 1024 s) is c * s + b rounded once, as decode() computes it. Per word of 8 codes: four
+    // masked pairs (codes i and i + 4 share a register; 7 instructions with v_and_or_b32, the magic held in a
+    // register because the instruction takes one literal), 8 fmas, 4 packs = 19 instructions, against 23 with byte
+    // planes and v_cvt_f32_ubyteN.
+    static constexpr int kPairState = 5;
+    __device__ static __forceinline__ Meta pair_meta(Meta m) {
+        m.b = fmaf(-1024.0f, m.s, m.b);
+        return m;
+    }
+    __device__ static __forceinline__ void pair_state(uint32_t *st) {
+        uint32_t magic = 0x64006400u;
+        asm volatile("" : "+v"(magic)); // opaque, so that it stays a register operand of v_and_or_b32
+        st[4] = magic;
+    }
     __device__ static __forceinline__ void decode_pair(const uint4 &raw, Meta m, int q, uint32_t *out, uint32_t *st) {
+        typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+        const uint32_t w = (q / 4) == 0 ? raw.x : (q / 4) == 1 ? raw.y : (q / 4) == 2 ? raw.z : raw.w;
         if (q % 4 == 0) {
-            const uint32_t w = (q / 4) == 0 ? raw.x : (q / 4) == 1 ? raw.y : (q / 4) == 2 ? raw.z : raw.w;
-            st[0] = w & 0x0f0f0f0fu;
-            st[1] = (w >> 4) & 0x0f0f0f0fu;
-            asm("" : "+v"(st[0]), "+v"(st[1]));
+            st[0] = (w & 0x000f000fu) | st[4];
+            st[1] = ((w >> 4) & 0x000f000fu) | st[4];
+        } else if (q % 4 == 1) {
+            st[2] = ((w >> 8) & 0x000f000fu) | st[4];
+            st[3] = ((w >> 12) & 0x000f000fu) | st[4];
         }
-        const uint32_t lo = (st[0] >> (8 * (q % 4))) & 0xffu, hi = (st[1] >> (8 * (q % 4))) & 0xffu;
-        out[q] = pack_bf16x2(fmaf((float)lo, m.s, m.b), fmaf((float)hi, m.s, m.b));
+        const f16x2_t a = __builtin_bit_cast(f16x2_t, st[(q % 2) * 2]), b = __builtin_bit_cast(f16x2_t, st[(q % 2) * 2 + 1]);
+        const float va = (q % 4) < 2 ? (float)a.x : (float)a.y, vb = (q % 4) < 2 ? (float)b.x : (float)b.y;
+        out[q] = pack_bf16x2(fmaf(va, m.s, m.b), fmaf(vb, m.s, m.b));
     }
 };
 
@@ -171,6 +189,9 @@ struct FmtAffine8 {
         decode_word(raw.w, m, out + 6);
     }
     __device__ static __forceinline__ void decode_fast(const uint4 &raw, Meta m, uint32_t *out) { decode(raw, m, out); }
+    static constexpr int kPairState = 1;
+    __device__ static __forceinline__ Meta pair_meta(Meta m) { return m; }
+    __device__ static __forceinline__ void pair_state(uint32_t *) {}
     __device__ static __forceinline__ void decode_pair(const uint4 &raw, Meta m, int q, uint32_t *out, uint32_t *) {
         const uint32_t w = (q / 2) == 0 ? raw.x : (q / 2) == 1 ? raw.y : (q / 2) == 2 ? raw.z : raw.w;
         const uint32_t v = w >> (16 * (q % 2));
@@ -234,6 +255,9 @@ struct FmtMxfp4 {
         fast_word(raw.z, m.s, out + 8);
         fast_word(raw.w, m.s, out + 12);
     }
+    static constexpr int kPairState = 1;
+    __device__ static __forceinline__ Meta pair_meta(Meta m) { return m; }
+    __device__ static __forceinline__ void pair_state(uint32_t *) {}
     __device__ static __forceinline__ void decode_pair(const uint4 &raw, Meta m, int q, uint32_t *out, uint32_t *) {
         const uint32_t w = (q / 4) == 0 ? raw.x : (q / 4) == 1 ? raw.y : (q / 4) == 2 ? raw.z : raw.w;
         switch (q % 4) { // the byte selector is an immediate
@@ -288,6 +312,9 @@ struct FmtFp8Row {
         fast_word(raw.z, out + 4);
         fast_word(raw.w, out + 6);
     }
+    static constexpr int kPairState = 1;
+    __device__ static __forceinline__ Meta pair_meta(Meta m) { return m; }
+    __device__ static __forceinline__ void pair_state(uint32_t *) {}
     __device__ static __forceinline__ void decode_pair(const uint4 &raw, Meta, int q, uint32_t *out, uint32_t *) {
         const uint32_t w = (q / 2) == 0 ? raw.x : (q / 2) == 1 ? raw.y : (q / 2) == 2 ? raw.z : raw.w;
         if (q % 2 == 0) out[q] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false));

@@ -153,8 +153,9 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
         constexpr int NP = NT * (KV / 2); // packed pairs to decode for the next step
         Meta meta_next[NT];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) meta_next[nt] = CS::meta(ring_sb[slot_next][nt]);
-        uint32_t dstate[2] = {0, 0};
+        for (int nt = 0; nt < NT; ++nt) meta_next[nt] = Fmt::pair_meta(CS::meta(ring_sb[slot_next][nt]));
+        uint32_t dstate[Fmt::kPairState] = {};
+        Fmt::pair_state(dstate);
         if (sb == 0) {
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) read_x(buf_off, 0, 0, mt, 0);

@@ -176,8 +176,9 @@ __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint
             const bool stage = s + AHEAD < n_steps; // uniform
             Meta meta_next[NT];
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) meta_next[nt] = CS::meta(ring_sb[slot_next][nt]);
-            uint32_t dstate[2] = {0, 0};
+            for (int nt = 0; nt < NT; ++nt) meta_next[nt] = Fmt::pair_meta(CS::meta(ring_sb[slot_next][nt]));
+            uint32_t dstate[Fmt::kPairState] = {};
+            Fmt::pair_state(dstate);
 #pragma unroll
             for (int jj = 0; jj < NJ; ++jj) {
                 if (jj == NJ - 1) {
