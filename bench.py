@@ -28,7 +28,7 @@ COPY_PROBE_BYTES = 256 << 20  # --copy-probe: bytes read (and written) by each c
 # (scaled by the same counters' reading for the --copy-probe copies; profiles/hbm_traffic_gemm_kernels.txt).
 # A counter cannot be read from inside the timed run, so these are the recorded values for the default workloads.
 MEASURED_TRAFFIC = {(1, "gate_up+down"): 1509859000,
-                    (3, "gate_up"): 3667158000, (3, "down"): 2016777000}
+                    (3, "gate_up"): 4045122000, (3, "down"): 2207021000}
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 
@@ -169,13 +169,13 @@ def main():
         for a, b in ((sh[0], wl.gate), (sh[1], wl.up), (sh[2], wl.down)))
     k_experts, k_rows = U + (1 if folded else 0), rows + (wl.T if folded else 0)
     # Prefill on packed 4-bit weights: each grouped GEMM is two launches on one tile list. The matrix-core kernel (the
-    # dominant one, timed as the gate_up / down stage) takes the tiles above 32 rows; an expert's rows are cut into
-    # tiles of 128, so only a remainder of at most 32 rows goes to the weight-streaming kernel (stages *_small).
+    # dominant one, timed as the gate_up / down stage) takes the tiles above 8 rows; an expert's rows are cut into
+    # tiles of 128, so only a remainder of at most 8 rows goes to the weight-streaming kernel (stages *_small).
     split = (not decode) and stages.get("gate_up_small", 0.0) > 0.0
     if split:
         c = counts.to(torch.int64)
         rem = c % 128
-        wide = c - torch.where(rem <= 32, rem, torch.zeros_like(rem))
+        wide = c - torch.where(rem <= 8, rem, torch.zeros_like(rem))
         k_experts, k_rows = int((wide > 0).sum()), int(wide.sum())
     gu_bytes = k_experts * gate_up_w + min(wl.T, k_rows) * wl.D * 2 + k_rows * wl.F * 2
     dn_bytes = k_experts * down_w + k_rows * wl.F * 2 + k_rows * wl.D * 2

@@ -222,12 +222,14 @@ static FwdLayout forward_layout(const Layer *L, int T, bool with_shared = true) 
 // Prefill-sized calls: the matrix-core kernel takes the tiles above `small_rows` rows, and the weight-streaming kernel
 // the rest of the same list right behind it (a tile of a few rows is bound by reading its expert's weights, and the
 // large-tile kernel spends a whole pass of its LDS pipeline on it). small_rows = 0: everything on the matrix-core kernel.
+constexpr int kPrefillSmallRows = 8;
 static int prefill_small_rows(const QView &b0, const QView &b1) {
     if (!qgemm_skinny_supports(b0) || !qgemm_skinny_supports(b1)) return 0;
     // measured: pays with the kernel of the packed 4-bit formats (8k-token ragged prefill: gate/up 1.757 -> 1.715 ms, down
     // unchanged), not with the 8-bit kernel (2080-token mixed batch: +1 %)
     if (!qgemm_wide_supports(b0) || !qgemm_wide_supports(b1)) return 0;
-    return std::min(qgemm_skinny_tile_m(b0), qgemm_skinny_tile_m(b1));
+    // threshold measured on the same prefill: 8 rows 2.62 ms, 16 rows 2.63, 32 rows 2.64, 4 rows 2.67, no split 2.70
+    return std::min(kPrefillSmallRows, std::min(qgemm_skinny_tile_m(b0), qgemm_skinny_tile_m(b1)));
 }
 static int run_gemm(const GemmArgs &g, bool small, hipStream_t st, int small_rows = 0) {
     if (g.b0.mode == DMOE_QUANT_NONE) return launch_gemm_bf16(g, st);

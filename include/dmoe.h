@@ -105,7 +105,7 @@ enum {
     DMOE_STAGE_SHARED = 4,       /* shared expert (both GEMMs)                    */
     DMOE_STAGE_COMBINE = 5,      /* weighted sum over k + shared add              */
     /* prefill-sized calls on packed 4-bit weights split each grouped GEMM into two launches on one tile list: the
-     * matrix-core kernel takes the tiles above 32 rows (stages 2 and 3), the weight-streaming kernel the rest: */
+     * matrix-core kernel takes the tiles above 8 rows (stages 2 and 3), the weight-streaming kernel the rest: */
     DMOE_STAGE_GATE_UP_SMALL = 6,
     DMOE_STAGE_DOWN_SMALL = 7,
     DMOE_STAGE_COUNT = 8
