@@ -21,6 +21,7 @@
 #include <new>
 
 #include "common.h"
+#include "route_device.h"
 
 namespace dmoe {
 
@@ -183,20 +184,28 @@ __device__ __forceinline__ float det_logf(float x) {
     return fmaf(fe, 0.693359375f, r);
 }
 
-// one wavefront per token: adds the segment sums left to right, rounds the logit to bf16, applies the scoring
-// function. Lane l owns experts l, l + 64, ... (E <= 1024). Softmax: the sum is taken as one partial per lane
-// (its experts in increasing order), folded by halves (lane i += lane i + 32, 16, .. 1).
+// One wavefront per token: adds the segment sums left to right, rounds the logit to bf16, applies the scoring
+// function and, with ROUTE, goes straight on to the selection (bias, Smelt mask, top-k, weights from the unbiased
+// scores, renormalisation, route scale: deepseek_v4.zig:589-678) with the scores still in registers, so they make no
+// round trip through memory; `scores` is written only when the caller wants them. Lane l owns experts l, l + 64, ...
+// (EPL of them). Softmax: the sum is taken as one partial per lane (its experts in increasing order), folded by
+// halves (lane i += lane i + 32, 16, .. 1).
+template <int EPL, bool ROUTE>
 __global__ __launch_bounds__(kGateWaves * 64) void gate_scores_kernel(float *__restrict__ scores,
                                                                       const float *__restrict__ partial, int T,
-                                                                      int E, int n_seg, int scoring) {
+                                                                      int E, int n_seg, int scoring,
+                                                                      uint32_t *__restrict__ out_idx,
+                                                                      float *__restrict__ out_w,
+                                                                      const float *__restrict__ bias,
+                                                                      const uint8_t *__restrict__ resident, int K,
+                                                                      int normalize, float route_scale) {
     const int lane = (int)threadIdx.x & 63;
     const int t = (int)blockIdx.x * kGateWaves + ((int)threadIdx.x >> 6);
     if (t >= T) return;
-    constexpr int kMaxPerLane = 16;
-    float v[kMaxPerLane];
+    float v[EPL];
     float mx = -__builtin_inff();
 #pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i) {
+    for (int i = 0; i < EPL; ++i) {
         const int e = lane + 64 * i;
         v[i] = 0.0f;
         if (e < E) {
@@ -222,7 +231,7 @@ __global__ __launch_bounds__(kGateWaves * 64) void gate_scores_kernel(float *__r
         }
         float part = 0.0f;
 #pragma unroll
-        for (int i = 0; i < kMaxPerLane; ++i)
+        for (int i = 0; i < EPL; ++i)
             if (lane + 64 * i < E) {
                 v[i] = det_expf(v[i] - mx);
                 part = part + v[i];
@@ -231,17 +240,28 @@ __global__ __launch_bounds__(kGateWaves * 64) void gate_scores_kernel(float *__r
         for (int off = 32; off >= 1; off >>= 1) part = part + __shfl_down(part, off, 64);
         const float sum = __shfl(part, 0, 64);
 #pragma unroll
-        for (int i = 0; i < kMaxPerLane; ++i)
-            if (lane + 64 * i < E) scores[(size_t)t * E + lane + 64 * i] = v[i] / sum;
+        for (int i = 0; i < EPL; ++i)
+            if (lane + 64 * i < E) v[i] = v[i] / sum;
     } else {
 #pragma unroll
-        for (int i = 0; i < kMaxPerLane; ++i) {
-            const int e = lane + 64 * i;
-            if (e >= E) continue;
-            float s;
-            if (scoring == DMOE_SCORE_SIGMOID) s = 1.0f / (1.0f + det_expf(-v[i]));
-            else s = sqrtf(det_logf(1.0f + det_expf(v[i]))); // the reference's literal form (:575-583)
-            scores[(size_t)t * E + e] = s;
+        for (int i = 0; i < EPL; ++i) {
+            if (lane + 64 * i >= E) continue;
+            if (scoring == DMOE_SCORE_SIGMOID) v[i] = 1.0f / (1.0f + det_expf(-v[i]));
+            else v[i] = sqrtf(det_logf(1.0f + det_expf(v[i]))); // the reference's literal form (:575-583)
+        }
+    }
+    if (scores) {
+#pragma unroll
+        for (int i = 0; i < EPL; ++i)
+            if (lane + 64 * i < E) scores[(size_t)t * E + lane + 64 * i] = v[i];
+    }
+    if (ROUTE) {
+        uint32_t my_idx;
+        float w;
+        route_from_registers<EPL>(v, bias, resident, E, K, normalize, 1, route_scale, lane, my_idx, w);
+        if (lane < K) {
+            out_idx[(size_t)t * K + lane] = my_idx;
+            out_w[(size_t)t * K + lane] = w;
         }
     }
 }
@@ -371,7 +391,8 @@ int dmoe_gate_forward(uint32_t *d_out_indices, float *d_out_weights, float *d_ou
     const int n_out_seg = split ? n_seg : 1;
     Bump b;
     const size_t o_part = b.take(sizeof(float) * (size_t)T * G->E * n_out_seg);
-    const size_t o_scores = b.take(d_out_scores ? 0 : sizeof(float) * (size_t)T * G->E);
+    const bool hash = G->tid2eid && d_input_ids; // only the table lookup reads the scores back from memory
+    const size_t o_scores = b.take(d_out_scores || !hash ? 0 : sizeof(float) * (size_t)T * G->E);
     Workspace *w = nullptr;
     DMOE_TRY(workspace_reserve(ws, b.off, &w));
     float *partial = at<float>(w, o_part);
@@ -382,19 +403,32 @@ int dmoe_gate_forward(uint32_t *d_out_indices, float *d_out_weights, float *d_ou
     if (split) hipLaunchKernelGGL(gate_logits_kernel<true>, grid, block, 0, st, partial, d_x, (const uint4 *)G->wgp, T, G->D, G->E, n_seg, segs_per_wave);
     else hipLaunchKernelGGL(gate_logits_kernel<false>, grid, block, 0, st, partial, d_x, (const uint4 *)G->wgp, T, G->D, G->E, n_seg, segs_per_wave);
     DMOE_LAUNCH_CHECK();
-    hipLaunchKernelGGL(gate_scores_kernel, dim3((unsigned)ceil_div(T, kGateWaves)), block, 0, st, scores, partial, T, G->E,
-                       n_out_seg, G->scoring);
-    DMOE_LAUNCH_CHECK();
     // the reference renormalises for every scoring function except softmax (:663)
-    if (G->tid2eid && d_input_ids) { // hash layer with token ids: the table replaces the top-k (:619-636)
+    const int normalize = G->scoring != DMOE_SCORE_SOFTMAX ? 1 : 0;
+    const dim3 sgrid((unsigned)ceil_div(T, kGateWaves));
+    if (hash) { // hash layer with token ids: the table replaces the top-k (:619-636)
+        if (G->E <= 256)
+            hipLaunchKernelGGL((gate_scores_kernel<4, false>), sgrid, block, 0, st, scores, partial, T, G->E, n_out_seg, G->scoring,
+                               nullptr, nullptr, nullptr, nullptr, 0, 0, 1.0f);
+        else
+            hipLaunchKernelGGL((gate_scores_kernel<16, false>), sgrid, block, 0, st, scores, partial, T, G->E, n_out_seg, G->scoring,
+                               nullptr, nullptr, nullptr, nullptr, 0, 0, 1.0f);
+        DMOE_LAUNCH_CHECK();
         hipLaunchKernelGGL(gate_hash_route_kernel, dim3((unsigned)ceil_div(T, 256)), dim3(256), 0, st, d_out_indices,
-                           d_out_weights, scores, G->tid2eid, d_input_ids, T, G->E, G->K, G->vocab,
-                           G->scoring != DMOE_SCORE_SOFTMAX ? 1 : 0, G->route_scale);
+                           d_out_weights, scores, G->tid2eid, d_input_ids, T, G->E, G->K, G->vocab, normalize, G->route_scale);
         DMOE_LAUNCH_CHECK();
         return DMOE_OK;
     }
-    return dmoe_gate_route(d_out_indices, d_out_weights, scores, G->bias, G->mask, T, G->E, G->K,
-                           G->scoring != DMOE_SCORE_SOFTMAX, G->route_scale, s);
+    // scoring and selection in one launch; the scores leave the registers only if the caller asked for them
+    DMOE_REQUIRE(G->K >= 1 && G->K <= G->E && G->K <= 64, "gate_forward: K=%d must satisfy 1 <= K <= min(E,64)", G->K);
+    if (G->E <= 256)
+        hipLaunchKernelGGL((gate_scores_kernel<4, true>), sgrid, block, 0, st, d_out_scores, partial, T, G->E, n_out_seg, G->scoring,
+                           d_out_indices, d_out_weights, G->bias, G->mask, G->K, normalize, G->route_scale);
+    else
+        hipLaunchKernelGGL((gate_scores_kernel<16, true>), sgrid, block, 0, st, d_out_scores, partial, T, G->E, n_out_seg, G->scoring,
+                           d_out_indices, d_out_weights, G->bias, G->mask, G->K, normalize, G->route_scale);
+    DMOE_LAUNCH_CHECK();
+    return DMOE_OK;
 }
 
 } // extern "C"

@@ -105,4 +105,67 @@ __device__ __forceinline__ void route_tokens(const float *const (&s)[NT], const 
     }
 }
 
+// The same selection for ONE token whose E scores are already in registers (lane l holds experts l, l + 64, ... in
+// `sc`), for kernels that have just computed the scores: no round trip through memory. Same arithmetic, same tie rule
+// and same summation order as route_tokens, so both give the same bits. Lane j < K returns column j.
+template <int EPL>
+__device__ __forceinline__ void route_from_registers(const float (&sc)[EPL], const float *__restrict__ bias,
+                                                     const uint8_t *__restrict__ resident, int E, int K, int normalize,
+                                                     int apply_scale, float route_scale, int lane, uint32_t &my_idx,
+                                                     float &w) {
+    uint32_t key[EPL];
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+        const int e = lane + 64 * i;
+        const bool in = e < E;
+        const int ec = in ? e : 0;
+        float c = sc[i];
+        if (bias) c = c + bias[ec];
+        if (resident) c = c + (resident[ec] ? 0.0f : -1e9f);
+        key[i] = in ? f32_sort_key(c) : 0u;
+    }
+    my_idx = 0;
+    float my_score = 0.0f;
+    for (int it = 0; it < K; ++it) {
+        uint64_t best = 0;
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) {
+            const uint64_t p = route_pair(key[i], (uint32_t)(lane + 64 * i));
+            best = p > best ? p : best;
+        }
+        route_pair_step<0xB1>(best);
+        route_pair_step<0x4E>(best);
+        route_pair_step<0x141>(best);
+        route_pair_step<0x140>(best);
+        uint64_t top = 0;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)best, 16 * r);
+            const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(best >> 32), 16 * r);
+            const uint64_t p = ((uint64_t)hi << 32) | lo;
+            top = p > top ? p : top;
+        }
+        const uint32_t bi = (uint32_t)top; // the winner's expert index, uniform
+        // the winner's unbiased score sits in register bi / 64 of lane bi % 64
+        float mine = 0.0f;
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) {
+            const bool hit = bi == (uint32_t)(lane + 64 * i);
+            mine = hit ? sc[i] : mine;
+            key[i] = hit ? 0u : key[i]; // taken
+        }
+        const float won = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mine), (int)(bi & 63u)));
+        const bool col = lane == K - 1 - it;
+        my_idx = col ? bi : my_idx;
+        my_score = col ? won : my_score;
+    }
+    const float my_w = (lane < K) ? my_score : 0.0f;
+    float sum = 0.0f;
+    for (int c = 0; c < K; ++c) sum += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_w), c)); // left to right
+    float v = my_w;
+    if (normalize) v = v / (sum + 1e-20f);
+    if (apply_scale) v = v * route_scale;
+    w = v;
+}
+
 } // namespace dmoe
