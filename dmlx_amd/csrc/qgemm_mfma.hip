@@ -27,7 +27,8 @@
 namespace dmoe {
 
 constexpr int kMfmaWaves = 4;
-constexpr int kMfmaRing = 4; // weight steps held in registers = reduction steps per LDS activation block
+constexpr int kMfmaRing = 4;  // reduction steps per LDS activation block
+constexpr int kMfmaWRing = 2; // weight steps held in registers
 
 template <typename Fmt>
 struct MfmaGeom {
@@ -69,8 +70,8 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
         if (n >= n_out) n = n_out - 1; // keep addresses valid; such rows are never stored
         cs[nt].init(b, e, (on ? base : 0) >> 5, ln, h, n);
     }
-    uint4 ring_raw[kMfmaRing][NT];
-    uint32_t ring_sb[kMfmaRing][NT][2];
+    uint4 ring_raw[kMfmaWRing][NT];
+    uint32_t ring_sb[kMfmaWRing][NT][2];
     auto load_b = [&](int step, int slot_) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
@@ -81,7 +82,7 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
     };
     // weight loads depend on the tile only: start them first (steps past the end are clamped, their data unused)
 #pragma unroll
-    for (int j = 0; j < kMfmaRing; ++j) load_b(j < n_steps ? j : n_steps - 1, j);
+    for (int j = 0; j < kMfmaWRing; ++j) load_b(j < n_steps ? j : n_steps - 1, j);
 
     // ---- activation staging ------------------------------------------------------------------------------
     // thread -> (row a_row + 32 * p, 16-byte piece a_piece of each 128-byte granule): eight lanes cover one full
@@ -221,10 +222,10 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
 #pragma unroll
         for (int j = 0; j < kMfmaRing; ++j) {
             const int s = s0 + j;
-            const int s_ahead = s + kMfmaRing < n_steps ? s + kMfmaRing : n_steps - 1;
-            load_b(s_ahead, j); // slot j was decoded one step ago
+            const int s_ahead = s + kMfmaWRing < n_steps ? s + kMfmaWRing : n_steps - 1;
+            load_b(s_ahead, j % kMfmaWRing); // this slot was decoded one step ago
             // steps 0, 1: fetch the two halves of the next block; steps 2, 3: store them into the other buffer
-            step_body((j + 1) % kMfmaRing, j & 1, rd_off, j, [&](int u) {
+            step_body((j + 1) % kMfmaWRing, j & 1, rd_off, j, [&](int u) {
                 constexpr int NU = NJ * MT * NT, every = NU / kOpsPerHalf;
                 static_assert(NU % kOpsPerHalf == 0, "staging operations must spread evenly over the units");
                 if (u % every != 0) return;
@@ -294,7 +295,9 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
 }
 
 template <typename Fmt, bool GATE_UP, bool PACKED>
-__global__ __launch_bounds__(kMfmaWaves * 64) void qgemm_mfma_kernel(GemmArgs g) {
+// 8-bit formats: 70 KiB of LDS per workgroup, so two workgroups share a compute unit if a wavefront stays under 256
+// registers; the 4-bit formats stage twice the reduction length per block (135 KiB) and run one workgroup per unit
+__global__ __launch_bounds__(kMfmaWaves * 64, Fmt::kVals == 16 ? 2 : 1) void qgemm_mfma_kernel(GemmArgs g) {
     extern __shared__ __attribute__((aligned(16))) uint8_t mfma_lds[]; // bf16 As[2][kMfmaTileM][LDA]
     Tile t;
     const uint32_t slot = blockIdx.y;
