@@ -81,10 +81,14 @@ def test_hash_gate_takes_experts_from_the_table(dmoe, orc, ws, func):
     np.testing.assert_array_equal(w.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
     # the table decides, not the scores: the indices are exactly the rows of the table
     np.testing.assert_array_equal(to_np_u32(idx), tid2eid.cpu().numpy()[to_np_u32(ids).astype(np.int64)].astype(np.uint32))
+    # the same call without a scores output (the scores then live in the workspace only)
+    idx3, w3 = gate.forward(x, ws, input_ids=ids)
+    assert torch.equal(idx3, idx) and torch.equal(w3, w)
     # without token ids a hash gate falls back to score-based top-k, like the reference
     idx2, w2 = gate.forward(x, ws)
     ref_idx, ref_w = orc.gate_route(want_scores, bias.cpu().numpy(), None, K, func != 0, 2.5)
     np.testing.assert_array_equal(to_np_u32(idx2), ref_idx)
+    np.testing.assert_array_equal(w2.cpu().numpy().view(np.uint32), ref_w.view(np.uint32))
     gate.close()
 
 
