@@ -68,6 +68,7 @@ EXPORTS = [
     "dmoe_topk_route", "dmoe_gate_route", "dmoe_remap_indices", "dmoe_expand_tokens",
     "dmoe_reduce_experts", "dmoe_smelt_build_mask", "dmoe_build_remap", "dmoe_preload_remap",
     "dmoe_pack", "dmoe_dequantize", "dmoe_gather_qmm",
+    "dmoe_resident_weight_create", "dmoe_resident_weight_destroy", "dmoe_gather_qmm_resident",
     "dmoe_layer_create", "dmoe_layer_destroy", "dmoe_moe_forward",
     "dmoe_switch_glu_forward_no_scores", "dmoe_moe_layer_forward", "dmoe_debug_last_activations",
     "dmoe_gate_create", "dmoe_gate_destroy", "dmoe_gate_forward",
@@ -262,6 +263,35 @@ def dequantize(qw, mat_index=0):
     c = qw.c()
     check(lib().dmoe_dequantize(_ptr(out), C.byref(c), mat_index, _stream()))
     return out
+
+
+class ResidentWeight:
+    """A weight stack made resident once in the kernels' layout (dmoe_resident_weight)."""
+
+    def __init__(self, qw):
+        self.h = _Handle()
+        self.rows, self.cols, self.n_mats = qw.rows, qw.cols, qw.n_mats
+        c = qw.c()
+        source = 1 if qw.w.is_cuda else 0   # DMOE_WEIGHTS_COPY_FROM_DEVICE / _FROM_HOST
+        check(lib().dmoe_resident_weight_create(C.byref(self.h), C.byref(c), source, _stream()))
+
+    def gather_qmm(self, x, rhs_indices, ws, lhs_indices=None, sorted_indices=False):
+        R = rhs_indices.numel()
+        out = torch.empty((R, self.rows), dtype=torch.bfloat16, device=x.device)
+        check(lib().dmoe_gather_qmm_resident(_ptr(out), _ptr(x), self.h, _ptr(lhs_indices), _ptr(rhs_indices), R,
+                                             int(sorted_indices), ws.h, _stream()))
+        return out
+
+    def close(self):
+        if self.h.ctx:
+            check(lib().dmoe_resident_weight_destroy(self.h))
+            self.h = _Handle()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 def gather_qmm(x, qw, rhs_indices, ws, lhs_indices=None, sorted_indices=False):

@@ -586,11 +586,8 @@ int dmoe_debug_last_activations(uint16_t *d_out, dmoe_layer layer, int T, dmoe_w
     return DMOE_OK;
 }
 
-int dmoe_gather_qmm(uint16_t *d_out, const uint16_t *d_x, const dmoe_qweight *qw, const uint32_t *d_lhs_indices,
-                    const uint32_t *d_rhs_indices, int R, int sorted, dmoe_workspace ws, dmoe_stream s) {
-    (void)sorted; // the counting sort below is a no-op on already grouped rows
-    QView v;
-    DMOE_TRY(make_qview(&v, qw, "gather_qmm"));
+static int gather_qmm_view(uint16_t *d_out, const uint16_t *d_x, const QView &v, const uint32_t *d_lhs_indices,
+                           const uint32_t *d_rhs_indices, int R, dmoe_workspace ws, dmoe_stream s) {
     DMOE_REQUIRE(R >= 0, "gather_qmm: R=%d", R);
     if (R == 0) return DMOE_OK;
     DMOE_REQUIRE(d_out && d_x && d_rhs_indices, "gather_qmm: null pointer");
@@ -631,6 +628,47 @@ int dmoe_gather_qmm(uint16_t *d_out, const uint16_t *d_x, const dmoe_qweight *qw
     g.max_tiles = max_tiles;
     g.tile_m = tile_m;
     return run_gemm(g, small, st, small ? 0 : prefill_small_rows(v, v));
+}
+
+int dmoe_gather_qmm(uint16_t *d_out, const uint16_t *d_x, const dmoe_qweight *qw, const uint32_t *d_lhs_indices,
+                    const uint32_t *d_rhs_indices, int R, int sorted, dmoe_workspace ws, dmoe_stream s) {
+    (void)sorted; // the counting sort is a no-op on already grouped rows
+    QView v;
+    DMOE_TRY(make_qview(&v, qw, "gather_qmm"));
+    return gather_qmm_view(d_out, d_x, v, d_lhs_indices, d_rhs_indices, R, ws, s);
+}
+
+int dmoe_resident_weight_create(dmoe_resident_weight *out, const dmoe_qweight *qw, int weight_source, dmoe_stream s) {
+    DMOE_REQUIRE(out && qw, "resident_weight_create: null argument");
+    out->ctx = nullptr;
+    DMOE_REQUIRE(weight_source >= 0 && weight_source <= 2, "resident_weight_create: bad weight_source %d", weight_source);
+    QOwned *q = new (std::nothrow) QOwned();
+    DMOE_REQUIRE(q != nullptr, "resident_weight_create: out of host memory");
+    int rc = adopt(q, qw, weight_source, "resident_weight", to_hip(s));
+    if (rc == DMOE_OK && hipStreamSynchronize(to_hip(s)) != hipSuccess) rc = hip_fail(hipGetLastError(), "hipStreamSynchronize");
+    if (rc != DMOE_OK) {
+        free_owned(*q);
+        delete q;
+        return rc;
+    }
+    out->ctx = q;
+    return DMOE_OK;
+}
+
+int dmoe_resident_weight_destroy(dmoe_resident_weight w) {
+    QOwned *q = (QOwned *)w.ctx;
+    if (!q) return DMOE_OK;
+    free_owned(*q);
+    delete q;
+    return DMOE_OK;
+}
+
+int dmoe_gather_qmm_resident(uint16_t *d_out, const uint16_t *d_x, dmoe_resident_weight w, const uint32_t *d_lhs_indices,
+                             const uint32_t *d_rhs_indices, int R, int sorted, dmoe_workspace ws, dmoe_stream s) {
+    (void)sorted;
+    const QOwned *q = (const QOwned *)w.ctx;
+    DMOE_REQUIRE(q != nullptr, "gather_qmm_resident: null weight handle");
+    return gather_qmm_view(d_out, d_x, q->view, d_lhs_indices, d_rhs_indices, R, ws, s);
 }
 
 } // extern "C"

@@ -567,6 +567,36 @@ inline Array gatherQmm(const Context &ctx, const Array &x, const QuantizedWeight
                           (const uint32_t *)rhs_indices.data(), R, sorted ? 1 : 0, ctx.workspace(), ctx.stream()));
     return out;
 }
+// A QuantizedWeight made resident once in the layout the kernels stream (the long-lived weight Arrays of the
+// reference's layer structs); gatherQmm on it gives the same bits as on the MLX layout, about five times faster at
+// decode sizes.
+class ResidentWeight {
+  public:
+    ResidentWeight(const Context &ctx, const QuantizedWeight &w, int weight_source) : rows_(w.rows), cols_(w.cols) {
+        dmoe_qweight q = w.c();
+        check(dmoe_resident_weight_create(&handle_, &q, weight_source, ctx.stream()));
+    }
+    ~ResidentWeight() { dmoe_resident_weight_destroy(handle_); }
+    ResidentWeight(const ResidentWeight &) = delete;
+    ResidentWeight &operator=(const ResidentWeight &) = delete;
+    Array gatherQmm(const Context &ctx, const Array &x, const Array *lhs_indices, const Array &rhs_indices, bool sorted) const {
+        if (x.dtype() != DType::bfloat16 || x.shape().size() != 2 || x.shape()[1] != cols_)
+            throw Error(DMOE_ERR_INVALID, "gatherQmm: x must be bfloat16 [rows, cols of the weights]");
+        if (rhs_indices.dtype() != DType::uint32 || (lhs_indices && (lhs_indices->dtype() != DType::uint32 ||
+                                                                     lhs_indices->size() != rhs_indices.size())))
+            throw Error(DMOE_ERR_INVALID, "gatherQmm: indices must be uint32 and of equal length");
+        const int R = (int)rhs_indices.size();
+        Array out(ctx, DType::bfloat16, {R, rows_});
+        check(dmoe_gather_qmm_resident((uint16_t *)out.data(), (const uint16_t *)x.data(), handle_,
+                                       lhs_indices ? (const uint32_t *)lhs_indices->data() : nullptr,
+                                       (const uint32_t *)rhs_indices.data(), R, sorted ? 1 : 0, ctx.workspace(), ctx.stream()));
+        return out;
+    }
+
+  private:
+    dmoe_resident_weight handle_{};
+    int rows_ = 0, cols_ = 0;
+};
 // mlx_dequantize of one matrix of the stack -> bf16 [rows, cols]
 inline Array dequantize(const Context &ctx, const QuantizedWeight &w, int mat_index) {
     Array out(ctx, DType::bfloat16, {w.rows, w.cols});

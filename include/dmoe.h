@@ -55,6 +55,7 @@ typedef struct dmoe_stream_ { void *ctx; } dmoe_stream;           /* ctx = hipSt
 typedef struct dmoe_workspace_ { void *ctx; } dmoe_workspace;     /* grow-only device scratch */
 typedef struct dmoe_layer_ { void *ctx; } dmoe_layer;             /* resident expert weights of one MoE layer */
 typedef struct dmoe_gate_ { void *ctx; } dmoe_gate;               /* resident router of one MoE layer */
+typedef struct dmoe_resident_weight_ { void *ctx; } dmoe_resident_weight; /* one weight stack in the kernels' layout */
 
 /* "affine" -> DMOE_QUANT_AFFINE, "mxfp4" -> DMOE_QUANT_MXFP4, "fp8" -> DMOE_QUANT_FP8_ROW,
  * "none" | "bf16" -> DMOE_QUANT_NONE; -1 if unknown */
@@ -209,6 +210,19 @@ int dmoe_dequantize(uint16_t *d_out, const dmoe_qweight *qw, int mat_index, dmoe
 int dmoe_gather_qmm(uint16_t *d_out, const uint16_t *d_x, const dmoe_qweight *qw,
                     const uint32_t *d_lhs_indices, const uint32_t *d_rhs_indices, int R, int sorted,
                     dmoe_workspace ws, dmoe_stream s);
+
+/* The same call on a stack that was made resident once: mlx-zig's QuantizedWeight is a long-lived object (the w /
+ * scales / biases Arrays of DSV4SwitchGLU live as long as the model, deepseek_v4.zig:687-717), and its counterpart
+ * here is a copy in HBM re-ordered into the layout the kernels stream (rows in blocks of 32, one contiguous KiB per
+ * wavefront and reduction step). dmoe_gather_qmm on the MLX layout gives the same bits but reads 32 cache lines per
+ * load; at decode sizes the resident stack streams about five times faster. `weight_source` as in dmoe_layer_desc
+ * (the stack is always copied: it is re-ordered). Shapes that cannot be re-ordered (rows not a multiple of 32) stay
+ * in the MLX layout inside the handle. */
+int dmoe_resident_weight_create(dmoe_resident_weight *out, const dmoe_qweight *qw, int weight_source, dmoe_stream s);
+int dmoe_resident_weight_destroy(dmoe_resident_weight w);
+int dmoe_gather_qmm_resident(uint16_t *d_out, const uint16_t *d_x, dmoe_resident_weight w,
+                             const uint32_t *d_lhs_indices, const uint32_t *d_rhs_indices, int R, int sorted,
+                             dmoe_workspace ws, dmoe_stream s);
 
 /* ---- resident MoE layer -------------------------------------------------------------------- */
 

@@ -322,6 +322,11 @@ static void test_gather_mm(Context &ctx) {
             EXPECT(from_bf16(gathered[(size_t)r * rows + n]) == (float)((rhs[r] + 1) * (lhs[r] * 16 + n)));
         }
     const QuantizedWeight q = QuantizedWeight::unquantized(wa.data(), E, rows, cols);
+    {   // the same product on a resident copy of the stack (taken from device memory)
+        quantize_mod::ResidentWeight res(ctx, q, DMOE_WEIGHTS_COPY_FROM_DEVICE);
+        auto again = res.gatherQmm(ctx, xa, &la, ra, false).dataSlice<uint16_t>();
+        for (size_t i = 0; i < again.size(); ++i) EXPECT(again[i] == gathered[i]);
+    }
     auto back = quantize_mod::dequantize(ctx, q, 1).dataSlice<uint16_t>();
     for (int i = 0; i < rows * cols; ++i) EXPECT(back[i] == w[(size_t)rows * cols + i]);
 }

@@ -87,6 +87,35 @@ def test_gather_qmm_matches_oracle(dmoe, orc, ws, fmt, R, n_mats, rows, cols):
 
 
 @pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("R,n_mats,rows,cols", [(40, 16, 256, 2048), (900, 6, 256, 1024), (12, 3, 96, 512), (50, 4, 40, 256)])
+def test_gather_qmm_on_a_resident_stack(dmoe, orc, ws, fmt, R, n_mats, rows, cols):
+    """dmoe_gather_qmm_resident: the stack copied once into the kernels' layout. At decode sizes the same bits as the
+    call on the MLX layout (the same kernel with other addressing); at prefill sizes the packed 4-bit formats take
+    another kernel, so the two agree to rounding. Always within the output bar of the oracle. The last shape cannot
+    be re-ordered (rows not a multiple of 32) and stays in the MLX layout inside the handle."""
+    qw = _stack(fmt, n_mats, rows, cols, 7)
+    g = torch.Generator(device="cuda").manual_seed(R)
+    x = torch.randn((R + 3, cols), generator=g, device="cuda").to(torch.bfloat16)
+    rhs = torch.randint(0, n_mats, (R,), generator=g, device="cuda", dtype=torch.int32)
+    lhs = torch.randint(0, R + 3, (R,), generator=g, device="cuda", dtype=torch.int32)
+    res = dmoe.ResidentWeight(qw)
+    for use_lhs in (False, True):
+        got = res.gather_qmm(x, rhs, ws, lhs if use_lhs else None)
+        plain = dmoe.gather_qmm(x, qw, rhs, ws, lhs if use_lhs else None)
+        if R <= 8 * n_mats:
+            assert torch.equal(got, plain), (fmt, use_lhs)
+        else:
+            # one bf16 step of the largest output at most (2^-7 of its value)
+            assert max_abs_rel(got.float().cpu().numpy(), plain.float().cpu().numpy()) < 8e-3, (fmt, use_lhs)
+        want = orc.gather_qmm(bf16_bits(x), qmat(qw), to_np_u32(rhs), to_np_u32(lhs) if use_lhs else None)
+        assert max_abs_rel(got.float().cpu().numpy(), want) < OUT_TOL
+    res.close()
+    host = dmoe.ResidentWeight(qw.to("cpu"))          # the same stack handed over from host memory
+    assert torch.equal(host.gather_qmm(x, rhs, ws), got if False else dmoe.ResidentWeight(qw).gather_qmm(x, rhs, ws))
+    host.close()
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
 @pytest.mark.parametrize("R", [9, 16, 17, 29, 32])
 def test_gather_qmm_one_expert_takes_every_row(dmoe, orc, ws, fmt, R):
     """Small-M path with a single tile of 9..32 rows (activations restaged span by span) beside empty experts."""
