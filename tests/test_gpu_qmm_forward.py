@@ -116,6 +116,31 @@ def test_gather_qmm_on_a_resident_stack(dmoe, orc, ws, fmt, R, n_mats, rows, col
 
 
 @pytest.mark.parametrize("fmt", FORMATS)
+def test_gather_qmm_seeded_random_shapes(dmoe, orc, ws, fmt):
+    """Twelve seeded shapes per format across both paths and both layouts: odd expert counts, weight rows that are
+    not a multiple of the 32-row blocks, reductions from one to 24 granules, row counts on either side of the
+    decode / prefill threshold, with and without a row gather."""
+    rng = np.random.default_rng(sum(map(ord, fmt)))
+    for case in range(12):
+        n_mats = int(rng.integers(1, 13))
+        rows = 4 * int(rng.integers(2, 81)) if case % 3 else 32 * int(rng.integers(1, 9))
+        cols = 128 * int(rng.integers(1, 13)) if fmt == "affine4g128" else 64 * int(rng.integers(1, 25))
+        R = int(rng.integers(1, 40)) if case % 2 else int(rng.integers(8 * n_mats + 1, 8 * n_mats + 600))
+        qw = _stack(fmt, n_mats, rows, cols, 100 + case)
+        g = torch.Generator(device="cuda").manual_seed(case)
+        x = torch.randn((R + 2, cols), generator=g, device="cuda").to(torch.bfloat16)
+        rhs = torch.randint(0, n_mats, (R,), generator=g, device="cuda", dtype=torch.int32)
+        lhs = torch.randint(0, R + 2, (R,), generator=g, device="cuda", dtype=torch.int32) if case % 4 == 0 else None
+        want = orc.gather_qmm(bf16_bits(x), qmat(qw), to_np_u32(rhs), None if lhs is None else to_np_u32(lhs))
+        got = dmoe.gather_qmm(x, qw, rhs, ws, lhs).float().cpu().numpy()
+        assert max_abs_rel(got, want) < OUT_TOL, (fmt, "MLX layout", n_mats, rows, cols, R, max_abs_rel(got, want))
+        res = dmoe.ResidentWeight(qw)
+        got_r = res.gather_qmm(x, rhs, ws, lhs).float().cpu().numpy()
+        res.close()
+        assert max_abs_rel(got_r, want) < OUT_TOL, (fmt, "resident", n_mats, rows, cols, R, max_abs_rel(got_r, want))
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
 @pytest.mark.parametrize("R", [9, 16, 17, 29, 32])
 def test_gather_qmm_one_expert_takes_every_row(dmoe, orc, ws, fmt, R):
     """Small-M path with a single tile of 9..32 rows (activations restaged span by span) beside empty experts."""
