@@ -342,6 +342,32 @@ def test_unquantized_tiny_model_shape(dmoe, orc, ws):
     layer.close()
 
 
+@pytest.mark.parametrize("fmt", ["affine4", "mxfp4", "affine8", "bf16"])
+def test_layer_seeded_random_shapes(dmoe, orc, ws, fmt):
+    """Eight seeded layers per routed format: hidden / FFN sizes in steps of 64, 2..40 experts, top-1..8, 1..600
+    tokens (both GEMM paths), no shared expert or one in the routed format, FP8 or 4-bit affine, either position of
+    the routing weight, with and without the SwiGLU limits and a selection bias."""
+    rng = np.random.default_rng(sum(map(ord, fmt)) + 1)
+    for case in range(8):
+        D, F = 64 * int(rng.integers(2, 17)), 64 * int(rng.integers(2, 13))
+        E = int(rng.integers(2, 41))
+        K = int(rng.integers(1, min(E, 8) + 1))
+        T = int(rng.integers(1, 33)) if case % 2 else int(rng.integers(33, 601))
+        g = torch.Generator(device="cuda").manual_seed(1000 + case)
+        x = torch.randn((T, D), generator=g, device="cuda").to(torch.bfloat16)
+        scores = torch.sigmoid(torch.randn((T, E), generator=g, device="cuda"))
+        bias = torch.randn((E,), generator=g, device="cuda") * 0.1 if case % 3 == 0 else None
+        sfmt = [None, fmt, "fp8row", "affine4"][case % 4]
+        shared = None if sfmt is None else (_stack(sfmt, 1, F, D, 70 + case), _stack(sfmt, 1, F, D, 80 + case),
+                                            _stack(sfmt, 1, D, F, 90 + case))
+        wl = workloads.Workload(f"random {fmt} #{case}", T, D, F, E, E, K, x, scores, bias, None, None, True, 1.5,
+                                _stack(fmt, E, F, D, 40 + case), _stack(fmt, E, F, D, 50 + case),
+                                _stack(fmt, E, D, F, 60 + case), shared,
+                                swiglu_limit=7.0 if case % 2 else 0.0, shared_swiglu_limit=3.0 if case % 4 == 1 else 0.0,
+                                score_before_down=bool(case & 4))
+        _check_layer(dmoe, orc, ws, wl)
+
+
 def test_forward_edge_cases(dmoe, orc, ws):
     wl = workloads.make(1, scale=0.125)
     layer = dmoe.Layer(wl.D, wl.F, wl.K, wl.gate, wl.up, wl.down, swiglu_limit=wl.swiglu_limit, shared=wl.shared)
