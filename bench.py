@@ -6,16 +6,26 @@ gate routing (top-k on biased scores, renormalised weights) -> token->expert pac
 GEMM + limited SwiGLU -> grouped down GEMM -> weighted combine + shared expert, all through the C ABI
 (dmoe_moe_layer_forward). Prints ONE JSON line.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1] [--windows 9] [--settle-ms 1000]
 
---config selects the benchmark configuration (0..4, as listed in BASELINE.json) (default 1: the 64-sequence decode step the headline metric is
-quoted on; 3 = the 8k-token ragged prefill). `roofline` describes the dominant kernel of the step, timed
-with HIP events recorded inside the library on the launch stream; `cpu_baseline` is the CPU restatement of
-the dmlx/MLX op sequence (the oracle) timed on this box's host cores on a bounded sample.
+--config selects the benchmark configuration (0..4, as listed in BASELINE.json); default 1: the 64-sequence decode
+step the headline metric is quoted on. The metric's other half - the fraction of the bf16 MFMA peak at the 8k-token
+ragged prefill, configuration 3 - is measured in the same run with the same procedure and reported under the key
+`prefill_c3` (switch off with --no-prefill).
+
+Timing procedure, per configuration: a pre-run of at least --settle-ms of steps brings clocks and memory to their
+loaded state (reported as `settle`, separate from `warmup`); then W untimed warm-up steps; then --windows windows of
+EXACTLY K steps each, every window bracketed by device synchronisations. `ms_per_step` is the MEDIAN window, all
+windows are listed in `window_ms_per_step`. Each window is followed by K more steps with the library's per-stage HIP
+events (recorded on the launch stream) switched on; `roofline` describes the dominant kernel of the step with the
+median of those per-window stage times. `cpu_baseline` is the CPU restatement of the dmlx/MLX op sequence (the oracle)
+timed on this box's host cores on a bounded sample. `roofline.traffic` and `mfma_busy` are read from the rocprofv3
+counter summaries under profiles/ (a counter cannot be read from inside the timed run).
 """
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -24,13 +34,19 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 COPY_PROBE_BYTES = 256 << 20  # --copy-probe: bytes read (and written) by each calibration copy
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
-# (scaled by the same counters' reading for the --copy-probe copies; profiles/hbm_traffic_gemm_kernels.txt).
-# A counter cannot be read from inside the timed run, so these are the recorded values for the default workloads.
-MEASURED_TRAFFIC = {(1, "gate_up+down"): 1509859000,
-                    (3, "gate_up"): 4045122000, (3, "down"): 2207021000}
+COUNTERS_FILE = os.path.join(ROOT, "profiles", "counters.json")   # written from the rocprofv3 --pmc summaries
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
+WIDE_TILE_ROWS = 128         # rows per tile of the library's matrix-core kernels (kMfmaWideTileM in csrc/common.h)
+
+
+def recorded_counters():
+    """Counter readings per (configuration, kernel) recorded under profiles/ ({} when the file is missing)."""
+    try:
+        with open(COUNTERS_FILE) as f:
+            return json.load(f)
+    except OSError:
+        return {}
 
 
 def cpu_baseline(wl, max_tokens, min_seconds=10.0, max_runs=5):
@@ -91,28 +107,12 @@ def measured_peaks(torch):
     return out
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", type=int, default=1, choices=[0, 1, 2, 3, 4])
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--copy-probe", action="store_true",
-                    help="also run three plain 256 MiB device copies first: the known-size kernel that scales the "
-                         "FETCH_SIZE / WRITE_SIZE counters when this command runs under rocprofv3 --pmc")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py measures the one-GPU path only: this build has no multi-GPU path (run with --gpus 1)",
-              file=sys.stderr)
-        sys.exit(2)
-
-    import torch
+def run_config(torch, config, steps, warmup, windows, settle_ms, copy_probe=False):
+    """Builds configuration `config`, times it as the module docstring says and returns (workload, timing, analysis
+    inputs). The layer and its workspace are released before returning."""
     from dmlx_amd import capi, workloads
 
-    torch.cuda.set_device(0)
-    capi.init(0)
-    wl = workloads.make(args.config, device="cuda")
+    wl = workloads.make(config, device="cuda")
     layer = capi.Layer(wl.D, wl.F, wl.K, wl.gate, wl.up, wl.down, swiglu_limit=wl.swiglu_limit,
                        score_before_down=wl.score_before_down, shared=wl.shared,
                        shared_swiglu_limit=wl.shared_swiglu_limit, remap=wl.remap, borrow=True)
@@ -120,9 +120,9 @@ def main():
     out = torch.empty((wl.T, wl.D), dtype=torch.bfloat16, device="cuda")
 
     def step():
-        return layer.layer_forward(wl.x, wl.scores, wl.bias, wl.resident_mask, wl.renorm, wl.route_scale, ws)
+        return layer.layer_forward(wl.x, wl.scores, wl.bias, wl.resident_mask, wl.renorm, wl.route_scale, ws, out=out)
 
-    if args.copy_probe:
+    if copy_probe:
         src = torch.ones(COPY_PROBE_BYTES // 4, dtype=torch.float32, device="cuda")
         dst = torch.empty_like(src)
         for _ in range(3):
@@ -130,33 +130,57 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    for _ in range(args.warmup):
-        out = step()
+    # clock-settling pre-run: steps in batches until the wall clock says enough
+    step()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        out = step()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
-    assert torch.isfinite(out.float()).all()
+    settle_steps, t0 = 0, time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < settle_ms:
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        settle_steps += steps
+    settle = {"steps": settle_steps, "ms": (time.perf_counter() - t0) * 1e3}
 
-    # the same K steps again with per-stage HIP events (recorded by the library on the launch stream)
-    ws.set_stage_timing(True)
-    for _ in range(args.steps):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    stages = {k: (ms / n if n else 0.0) for k, (ms, n) in ws.stage_times().items()}
-    ws.set_stage_timing(False)
+    window_ms, window_stages = [], []
+    for _ in range(windows):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        window_ms.append((time.perf_counter() - t0) * 1e3 / steps)
+        # the same K steps again with per-stage HIP events (recorded by the library on the launch stream)
+        ws.set_stage_timing(True)
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        window_stages.append({k: (ms / n if n else 0.0) for k, (ms, n) in ws.stage_times().items()})
+        ws.set_stage_timing(False)
+    ws.check()   # no bounded wait gave up, no expert id out of range, in any step above
+    assert torch.isfinite(out.float()).all()
+    stages = {k: statistics.median(w[k] for w in window_stages) for k in window_stages[0]}
 
     # distinct live experts of this batch (each expert's weights are read once per step)
     idx, _ = capi.gate_route(wl.scores, wl.bias, wl.resident_mask, wl.K, wl.renorm, wl.route_scale)
     if wl.remap is not None:
         idx = capi.remap_indices(torch.tensor(wl.remap, dtype=torch.int32, device="cuda"), idx)
     packed = capi.pack(idx, wl.E, ws)
-    U = int(packed["n_live"].item())
+    n_live = int(packed["n_live"].item())
     counts = packed["counts"].cpu()
-    rows = wl.T * wl.K
+    layer.close()
+    ws.close()
+    timing = {"ms_per_step": statistics.median(window_ms), "window_ms_per_step": window_ms, "settle": settle,
+              "stages": stages}
+    return wl, timing, n_live, counts
 
+
+def describe(torch, wl, config, timing, U, counts, steps, warmup, counters):
+    """The JSON fields of one configuration: throughput, roofline of the dominant kernel, whole-step fractions."""
+    stages, ms_per_step = timing["stages"], timing["ms_per_step"]
+    rows = wl.T * wl.K
     gate_up_w = (wl.gate.nbytes() + wl.up.nbytes()) // wl.E
     down_w = wl.down.nbytes() // wl.E
     kern = "gate_up" if stages["gate_up"] >= stages["down"] else "down"
@@ -170,11 +194,12 @@ def main():
     k_experts, k_rows = U + (1 if folded else 0), rows + (wl.T if folded else 0)
     # Prefill on packed 4-bit weights: each grouped GEMM is two launches on one tile list. The matrix-core kernel (the
     # dominant one, timed as the gate_up / down stage) takes the tiles above 8 rows; an expert's rows are cut into
-    # tiles of 128, so only a remainder of at most 8 rows goes to the weight-streaming kernel (stages *_small).
+    # tiles of `tile` rows, so only a remainder of at most 8 rows goes to the weight-streaming kernel (stages *_small).
     split = (not decode) and stages.get("gate_up_small", 0.0) > 0.0
     if split:
+        tile = WIDE_TILE_ROWS
         c = counts.to(torch.int64)
-        rem = c % 128
+        rem = c % tile
         wide = c - torch.where(rem <= 8, rem, torch.zeros_like(rem))
         k_experts, k_rows = int((wide > 0).sum()), int(wide.sum())
     gu_bytes = k_experts * gate_up_w + min(wl.T, k_rows) * wl.D * 2 + k_rows * wl.F * 2
@@ -191,16 +216,27 @@ def main():
     else:
         k_bytes, k_flops = dn_bytes, dn_flops
     k_ms = stages["gate_up"] if paired else stages[kern]
-    if decode:
-        achieved = k_bytes / (k_ms * 1e-3) / 1e9
-        roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": achieved / HBM_PEAK_GBS, "traffic": None}
+    hbm = k_bytes / (k_ms * 1e-3) / 1e9
+    mfma = k_flops / (k_ms * 1e-3) / 1e12
+    by_bound = {"hbm": {"bound": "hbm", "achieved": hbm, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": hbm / HBM_PEAK_GBS},
+                "mfma": {"bound": "mfma", "achieved": mfma, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": mfma / MFMA_BF16_PEAK_TFLOPS}}
+    # decode is bound by HBM and the 4-bit prefill by the matrix core; the mixed batch (configuration 4, 8-bit weights,
+    # 2080 tokens) sits between the two: both are reported, the one with the larger fraction as the bound
+    if config == 4:
+        first = "hbm" if by_bound["hbm"]["frac"] >= by_bound["mfma"]["frac"] else "mfma"
     else:
-        achieved = k_flops / (k_ms * 1e-3) / 1e12
-        roof = {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None}
-    roof["traffic"] = MEASURED_TRAFFIC.get((args.config, kern))
-    roof["measured_peaks"] = measured_peaks(torch)
+        first = "hbm" if decode else "mfma"
+    roof = dict(by_bound[first])
+    if config == 4:
+        roof["other_bound"] = by_bound["mfma" if first == "hbm" else "hbm"]
+    rec = counters.get(f"c{config}", {}).get(kern, {})
+    roof["traffic"] = rec.get("traffic_bytes")
+    if "mfma_busy" in rec:
+        roof["mfma_busy"] = rec["mfma_busy"]              # SQ_VALU_MFMA_BUSY_CYCLES / (SIMDs x kernel cycles)
+        roof["valu_per_mfma"] = rec.get("valu_per_mfma")  # other vector instructions per MFMA
+    if rec:
+        roof["counters_from"] = rec.get("source")
     launches = (["qgemm_skinny_kernel (gate/up and down tiles in one launch)"] if paired else ["qgemm_skinny_kernel"] if decode else
                 ["qgemm_wide_kernel"] if split else ["qgemm_mfma_kernel"])
     if split:
@@ -212,12 +248,10 @@ def main():
 
     step_bytes = U * wl.expert_bytes() + wl.shared_bytes() + 2 * wl.T * wl.D * 2 + wl.T * wl.E_total * 4 + rows * 8
     step_flops = wl.routed_flops() + wl.shared_flops()
-    result = {
-        "metric": "MoE-FFN tokens/s; HBM GB/s at decode, MFMA % at prefill (4-bit top-6/256)",
-        "value": wl.T / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": wl.name, "baseline_config": args.config, "tokens": wl.T, "hidden": wl.D,
+    return {
+        "value": wl.T / (ms_per_step * 1e-3), "unit": "tokens/s", "steps": steps, "warmup": warmup,
+        "ms_per_step": ms_per_step, "window_ms_per_step": timing["window_ms_per_step"], "settle": timing["settle"],
+        "config": {"workload": wl.name, "baseline_config": config, "tokens": wl.T, "hidden": wl.D,
                    "ffn": wl.F, "experts": wl.E_total, "resident_experts": wl.E, "top_k": wl.K,
                    "shared_expert": wl.shared is not None,
                    "weights": {0: "affine", 1: "mxfp4", 2: "fp8row", 3: "unquantized"}[wl.gate.mode] + f"-{wl.gate.bits}bit",
@@ -233,10 +267,61 @@ def main():
                  "mfma_frac": step_flops / (ms_per_step * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                  "stage_ms": stages},
     }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--windows", type=int, default=9, help="timed windows of --steps steps; the median is reported")
+    ap.add_argument("--settle-ms", type=float, default=1000.0, help="clock-settling pre-run before the warm-up")
+    ap.add_argument("--config", type=int, default=1, choices=[0, 1, 2, 3, 4])
+    ap.add_argument("--no-prefill", action="store_true", help="with --config 1: do not also time configuration 3")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-peaks", action="store_true", help="skip the library copy / GEMM reference measurements")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run three plain 256 MiB device copies first: the known-size kernel that scales the "
+                         "FETCH_SIZE / WRITE_SIZE counters when this command runs under rocprofv3 --pmc")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures the one-GPU path only: this build has no multi-GPU path (run with --gpus 1)",
+              file=sys.stderr)
+        sys.exit(2)
+    assert args.steps >= 1 and args.windows >= 1 and args.warmup >= 0
+
+    import torch
+    from dmlx_amd import capi
+
+    torch.cuda.set_device(0)
+    capi.init(0)
+    counters = recorded_counters()
+
+    wl, timing, U, counts = run_config(torch, args.config, args.steps, args.warmup, args.windows, args.settle_ms,
+                                       args.copy_probe)
+    body = describe(torch, wl, args.config, timing, U, counts, args.steps, args.warmup, counters)
+    result = {"metric": "MoE-FFN tokens/s; HBM GB/s at decode, MFMA % at prefill (4-bit top-6/256)",
+              "value": body.pop("value"), "unit": body.pop("unit"), "n_gpus": 1, "steps": args.steps,
+              "warmup": args.warmup, "ms_per_step": body.pop("ms_per_step"), "higher_is_better": True,
+              "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic"}
+    body.pop("steps"), body.pop("warmup")
+    result.update(body)
+    result["timing"] = (f"median of {args.windows} windows of {args.steps} steps after a {args.settle_ms:.0f} ms "
+                        f"pre-run and {args.warmup} warm-up steps")
+    if not args.no_peaks:
+        result["roofline"]["measured_peaks"] = measured_peaks(torch)
+    decode = wl.T * wl.K <= 8 * wl.E
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(wl, max_tokens=64 if decode else 256)
     else:
         result["cpu_baseline"] = None
+    del wl
+    torch.cuda.empty_cache()
+
+    if args.config == 1 and not args.no_prefill:
+        # the metric's prefill half: configuration 3 with the same procedure, its own roofline block
+        wl3, timing3, U3, counts3 = run_config(torch, 3, args.steps, args.warmup, args.windows, args.settle_ms)
+        result["prefill_c3"] = describe(torch, wl3, 3, timing3, U3, counts3, args.steps, args.warmup, counters)
     print(json.dumps(result))
 
 

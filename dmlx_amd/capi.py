@@ -63,7 +63,7 @@ EXPORTS = [
     "dmoe_stream_create", "dmoe_stream_destroy", "dmoe_stream_synchronize",
     "dmoe_malloc", "dmoe_free", "dmoe_copy_to_device", "dmoe_copy_to_host",
     "dmoe_workspace_create", "dmoe_workspace_destroy", "dmoe_workspace_reserved",
-    "dmoe_workspace_check", "dmoe_workspace_set_wait_limit",
+    "dmoe_workspace_check", "dmoe_workspace_set_wait_limit", "dmoe_workspace_set_paired_launch",
     "dmoe_workspace_set_stage_timing", "dmoe_workspace_read_stage_times",
     "dmoe_topk_route", "dmoe_gate_route", "dmoe_remap_indices", "dmoe_expand_tokens",
     "dmoe_reduce_experts", "dmoe_smelt_build_mask", "dmoe_build_remap", "dmoe_preload_remap",
@@ -126,6 +126,9 @@ class Workspace:
 
     def set_wait_limit(self, polls):
         check(lib().dmoe_workspace_set_wait_limit(self.h, C.c_uint(polls)))
+
+    def set_paired_launch(self, enabled):
+        check(lib().dmoe_workspace_set_paired_launch(self.h, int(enabled)))
 
     STAGES = ("route", "pack", "gate_up", "down", "shared", "combine", "gate_up_small", "down_small")
 
@@ -435,9 +438,11 @@ class Layer:
                                                       ws.h, _stream()))
         return out
 
-    def layer_forward(self, x, scores, bias, resident_mask, renorm, route_scale, ws, want_routing=False):
+    def layer_forward(self, x, scores, bias, resident_mask, renorm, route_scale, ws, want_routing=False, out=None):
+        """dmoe_moe_layer_forward; pass `out` to reuse an output tensor"""
         T, E_total = scores.shape
-        out = torch.empty((T, self.hidden), dtype=torch.bfloat16, device=x.device)
+        if out is None:
+            out = torch.empty((T, self.hidden), dtype=torch.bfloat16, device=x.device)
         idx = w = None
         if want_routing:
             idx = torch.empty((T, self.top_k), dtype=torch.int32, device=x.device)

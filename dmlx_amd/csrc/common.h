@@ -39,10 +39,14 @@ int hip_fail(hipError_t e, const char *what);
 inline hipStream_t to_hip(dmoe_stream s) { return (hipStream_t)s.ctx; }
 
 // ---- workspace: one grow-only device allocation, carved with a bump allocator ---------------------
+// Per stage a ring of event pairs: the steps of a measurement run are enqueued back to back, and the host waits for
+// events only when a ring is full or the totals are read.
+constexpr int kStageRing = 64;
 struct StageTimer {
     bool enabled = false;
-    hipEvent_t start[DMOE_STAGE_COUNT] = {}, stop[DMOE_STAGE_COUNT] = {};
-    bool pending[DMOE_STAGE_COUNT] = {};
+    hipEvent_t start[DMOE_STAGE_COUNT][kStageRing] = {}, stop[DMOE_STAGE_COUNT][kStageRing] = {};
+    int pending[DMOE_STAGE_COUNT] = {}; // event pairs recorded and not yet read, slots 0 .. pending - 1
+    bool open[DMOE_STAGE_COUNT] = {};   // start recorded, stop not yet
     float total_ms[DMOE_STAGE_COUNT] = {};
     int samples[DMOE_STAGE_COUNT] = {};
 };
@@ -57,10 +61,15 @@ struct Workspace {
     hipEvent_t fork = nullptr, join = nullptr;
     hipEvent_t packed = nullptr, small_done = nullptr; // prefill: the small tiles' GEMMs run on the side stream
     bool last_with_shared = true; // layout of the last forward on this workspace (for dmoe_debug_last_activations)
-    // Device words that outlive workspace growth: [0] counts waits inside a paired GEMM launch that gave up (see
-    // GemmArgs::wait_expired), read and cleared by dmoe_workspace_check. [1] is unused.
+    // Device words that outlive workspace growth, read and cleared by dmoe_workspace_check: [0] counts waits inside a
+    // paired GEMM launch that gave up (see GemmArgs::wait_expired), [1] counts expert ids outside [0, E) met by the
+    // pack kernels (see PackOut::bad_ids).
     uint32_t *flags = nullptr;
     uint32_t spin_limit = 1u << 16; // polls of ~0.25 us a waiting workgroup makes before it gives up (~16 ms)
+    // gate/up and down of a decode step share one launch (down workgroups wait per tile for gate/up). Switched off by
+    // dmoe_workspace_set_paired_launch, and by dmoe_workspace_check once a wait gave up: the two GEMMs then run as two
+    // launches in a row, which wait for nothing.
+    bool paired = true;
 };
 int side_stream_ready(Workspace *w);  // creates the side stream and its events on first use
 
@@ -110,6 +119,9 @@ struct PackOut {
     // optional per-tile completion counters (n_done of them), zeroed by the pack kernels: see GemmArgs::tile_done
     uint32_t *tile_done = nullptr;
     uint32_t n_done = 0;
+    // optional device counter: +1 for every expert id >= E met (such a row is packed under expert E - 1 so that every
+    // access stays in bounds; the host learns about it from dmoe_workspace_check)
+    uint32_t *bad_ids = nullptr;
 };
 
 inline int pack_max_tiles(size_t n, int E, int tile_m) {

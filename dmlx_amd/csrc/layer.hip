@@ -264,6 +264,7 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     // per-tile completion counters of the paired gate/up + down launch, zeroed with the tile list
     po.tile_done = at<uint32_t>(w, f.tile_done);
     po.n_done = (uint32_t)f.max_tiles;
+    po.bad_ids = w->flags + 1;
     DMOE_TRY(launch_pack(po, d_slots, n, L->K, L->E, f.tile_m, at<void>(w, f.scratch), st));
     DMOE_TRY(stage_end(w, DMOE_STAGE_PACK, st));
 
@@ -302,14 +303,14 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     gu.tile_done = po.tile_done;
     dn.spin_limit = w->spin_limit;
     dn.wait_expired = w->flags;
-    if (f.small && qgemm_skinny_pair_supports(gu, dn)) {
+    if (f.small && w->paired && qgemm_skinny_pair_supports(gu, dn)) {
         DMOE_TRY(stage_begin(w, DMOE_STAGE_GATE_UP, st));
         DMOE_TRY(launch_qgemm_skinny_pair(gu, dn, st));
         DMOE_TRY(stage_end(w, DMOE_STAGE_GATE_UP, st));
         return DMOE_OK;
     }
     const int small_rows = f.small ? 0 : prefill_small_rows(L->gate.view, L->down.view);
-    if (small_rows > 0 && !w->timer.enabled) {
+    if (small_rows > 0 && !w->timer.enabled && w->paired) {
         // Prefill: the small tiles' two GEMMs (one paired launch) depend on the tile list only. They go to the side
         // stream and fill the tails of the two matrix-core launches, which take the large tiles on `st`. (With stage
         // timing on, the launches stay in a row on `st` so that every stage's time covers all of its tiles.)
@@ -328,7 +329,7 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
             return DMOE_OK;
         }
     }
-    if (small_rows > 0) { // stage timing on: the four launches in a row, each its own stage
+    if (small_rows > 0) { // stage timing on, or no paired launch: the four launches in a row, each its own stage
         GemmArgs gu_small = gu, dn_small = dn, gu_big = gu, dn_big = dn;
         gu_small.max_rows = dn_small.max_rows = small_rows;
         gu_big.min_rows = dn_big.min_rows = small_rows + 1;
@@ -607,6 +608,7 @@ static int gather_qmm_view(uint16_t *d_out, const uint16_t *d_x, const QView &v,
     po.order = at<uint32_t>(w, o_order);
     po.tiles = at<Tile>(w, o_tiles);
     po.n_tiles = at<uint32_t>(w, o_nt);
+    po.bad_ids = w->flags + 1;
     DMOE_TRY(launch_pack(po, d_rhs_indices, (size_t)R, 1, v.n_mats, tile_m, at<void>(w, o_scr), st));
     const uint32_t *a_rows = po.order;
     if (d_lhs_indices) {

@@ -183,6 +183,17 @@ static int index_file(const char *path, StFile *f, std::map<std::string, StTenso
     return DMOE_OK;
 }
 
+// a * b * c * d as a byte count; false if any factor is not positive or the product does not fit
+static bool checked_bytes(long long a, long long b, long long c, long long d, size_t *out) {
+    unsigned long long r = 1;
+    for (long long f : {a, b, c, d}) {
+        if (f <= 0 || __builtin_mul_overflow(r, (unsigned long long)f, &r)) return false;
+    }
+    if (r > (unsigned long long)SIZE_MAX / 2) return false;
+    *out = (size_t)r;
+    return true;
+}
+
 // one projection (weight + scales [+ biases]) of `prefix`, validated against the quantization parameters
 static int find_proj(const std::map<std::string, StTensor> &index, const std::string &prefix, int mode, int bits,
                      int group, bool stacked, dmoe_qweight *q) {
@@ -195,7 +206,9 @@ static int find_proj(const std::map<std::string, StTensor> &index, const std::st
         DMOE_REQUIRE(tw.dtype == "BF16", "safetensors: %s.weight has dtype %s, expected BF16 (unquantized experts)",
                      prefix.c_str(), tw.dtype.c_str());
         const long long n = stacked ? tw.shape[0] : 1, rows = tw.shape[nd - 2], cols = tw.shape[nd - 1];
-        DMOE_REQUIRE(n >= 1 && rows >= 1 && cols >= 1 && tw.bytes == (size_t)(n * rows * cols * 2),
+        size_t want_bytes = 0;
+        DMOE_REQUIRE(n <= 1024 && rows <= INT32_MAX && cols <= INT32_MAX && checked_bytes(n, rows, cols, 2, &want_bytes) &&
+                         tw.bytes == want_bytes,
                      "safetensors: %s.weight: bad shape or byte count", prefix.c_str());
         q->w = tw.data;
         q->scales = nullptr;
@@ -210,21 +223,28 @@ static int find_proj(const std::map<std::string, StTensor> &index, const std::st
     }
     DMOE_REQUIRE(s != index.end(), "safetensors: tensor %s.scales not found (pass mode \"none\" for unquantized experts)",
                  prefix.c_str());
+    // the quantization parameters come from the caller: check them before they divide anything
+    DMOE_REQUIRE(bits == 4 || bits == 8, "safetensors: %s: bits must be 4 or 8, got %d", prefix.c_str(), bits);
+    DMOE_REQUIRE(group == 32 || group == 64 || group == 128, "safetensors: %s: group size must be 32, 64 or 128, got %d",
+                 prefix.c_str(), group);
     const StTensor &tw = w->second, &ts = s->second;
     DMOE_REQUIRE(tw.shape.size() == nd && ts.shape.size() == nd, "safetensors: %s: expected %zu-dimensional weight and scales",
                  prefix.c_str(), nd);
     DMOE_REQUIRE(tw.dtype == "U32", "safetensors: %s.weight has dtype %s, expected U32 (packed codes)", prefix.c_str(),
                  tw.dtype.c_str());
     const long long n = stacked ? tw.shape[0] : 1, rows = tw.shape[nd - 2], words = tw.shape[nd - 1];
+    DMOE_REQUIRE(n >= 1 && n <= 1024 && rows >= 1 && rows <= INT32_MAX && words >= 1 && words <= INT32_MAX / 8,
+                 "safetensors: %s: bad shape", prefix.c_str());
     const long long cols = words * 32 / bits;
-    DMOE_REQUIRE(n >= 1 && rows >= 1 && cols >= group && cols % group == 0, "safetensors: %s: bad shape", prefix.c_str());
-    DMOE_REQUIRE(tw.bytes == (size_t)(n * rows * words * 4), "safetensors: %s.weight: byte count does not match its shape",
-                 prefix.c_str());
+    DMOE_REQUIRE(cols >= group && cols % group == 0, "safetensors: %s: bad shape", prefix.c_str());
+    size_t w_bytes = 0, s_bytes = 0;
+    DMOE_REQUIRE(checked_bytes(n, rows, words, 4, &w_bytes) && tw.bytes == w_bytes,
+                 "safetensors: %s.weight: byte count does not match its shape", prefix.c_str());
     const char *want_s = mode == DMOE_QUANT_MXFP4 ? "U8" : "BF16";
     const size_t s_elem = mode == DMOE_QUANT_MXFP4 ? 1 : 2;
     DMOE_REQUIRE(ts.dtype == want_s, "safetensors: %s.scales has dtype %s, expected %s", prefix.c_str(), ts.dtype.c_str(), want_s);
     DMOE_REQUIRE((stacked ? ts.shape[0] : 1) == n && ts.shape[nd - 2] == rows && ts.shape[nd - 1] == cols / group &&
-                     ts.bytes == (size_t)(n * rows * (cols / group)) * s_elem,
+                     checked_bytes(n, rows, cols / group, (long long)s_elem, &s_bytes) && ts.bytes == s_bytes,
                  "safetensors: %s.scales does not match weight shape / group size %d", prefix.c_str(), group);
     q->w = tw.data;
     q->scales = ts.data;
@@ -321,6 +341,9 @@ extern "C" int dmoe_layer_create_from_safetensors(dmoe_layer *out, const char *c
     // (deepseek_v4_loader.zig:2151-2168)
     Subset sub[3];
     std::vector<int32_t> remap;
+    DMOE_REQUIRE(d.up.n_mats == d.gate.n_mats && d.down.n_mats == d.gate.n_mats,
+                 "layer_create_from_safetensors: gate / up / down hold %d / %d / %d experts", d.gate.n_mats, d.up.n_mats,
+                 d.down.n_mats);
     if (o->resident_mask) {
         const int n_total = d.gate.n_mats;
         DMOE_REQUIRE(o->n_experts_total == n_total, "layer_create_from_safetensors: mask length %d, file holds %d experts",

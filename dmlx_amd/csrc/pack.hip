@@ -140,7 +140,10 @@ __device__ __forceinline__ void pack_fused_body(const PackOut &o, uint32_t e, bo
     const int tid = (int)threadIdx.x, lane = lane_id(), wave = tid >> 6;
     for (int i = tid; i < kPackWaves * E; i += kPackThreads) pack_sm[i] = 0;
     __syncthreads();
-    if (active && e >= (uint32_t)E) e = (uint32_t)E - 1; // ids are validated by the caller's contract; stay in bounds
+    if (active && e >= (uint32_t)E) { // a corrupt id: stay in bounds, and tell the host
+        if (o.bad_ids) atomicAdd(o.bad_ids, 1u);
+        e = (uint32_t)E - 1;
+    }
     if (active) atomicAdd(&pack_sm[wave * E + e], 1u);
     __syncthreads();
     uint32_t count = 0;
@@ -174,7 +177,8 @@ __global__ __launch_bounds__(kPackThreads) void pack_fused_kernel(PackOut o, con
 // ---- three launches, any n --------------------------------------------------------------------------------
 __global__ __launch_bounds__(kScatterWaves * 64) void pack_hist_kernel(uint32_t *__restrict__ cnt,
                                                                        const uint32_t *__restrict__ idx,
-                                                                       size_t n, int E, int n_sub) {
+                                                                       size_t n, int E, int n_sub,
+                                                                       uint32_t *__restrict__ bad_ids) {
     extern __shared__ uint32_t pack_sm[]; // hist[kScatterWaves][E]
     const int tid = (int)threadIdx.x, lane = lane_id(), wave = tid >> 6;
     for (int i = tid; i < kScatterWaves * E; i += kScatterWaves * 64) pack_sm[i] = 0;
@@ -185,7 +189,10 @@ __global__ __launch_bounds__(kScatterWaves * 64) void pack_hist_kernel(uint32_t 
             size_t i = (size_t)sub * kSubRows + (size_t)g * 64 + lane;
             if (i < n) {
                 uint32_t e = idx[i];
-                if (e >= (uint32_t)E) e = (uint32_t)E - 1;
+                if (e >= (uint32_t)E) { // counted here once; the scatter kernel clamps the same way
+                    if (bad_ids) atomicAdd(bad_ids, 1u);
+                    e = (uint32_t)E - 1;
+                }
                 atomicAdd(&pack_sm[wave * E + e], 1u);
             }
         }
@@ -276,7 +283,7 @@ int launch_pack(const PackOut &o, const uint32_t *d_idx, size_t n, int K, int E,
     int n_sub = (int)((n + kSubRows - 1) / kSubRows);
     dim3 grid((unsigned)ceil_div(n_sub, kScatterWaves)), block(kScatterWaves * 64);
     size_t lds = sizeof(uint32_t) * (size_t)kScatterWaves * E;
-    hipLaunchKernelGGL(pack_hist_kernel, grid, block, lds, st, cnt, d_idx, n, E, n_sub);
+    hipLaunchKernelGGL(pack_hist_kernel, grid, block, lds, st, cnt, d_idx, n, E, n_sub, o.bad_ids);
     DMOE_LAUNCH_CHECK();
     hipLaunchKernelGGL(pack_scan_kernel, dim3(1), dim3(kPackThreads), 0, st, o, cnt, n, E, n_sub, tile_m);
     DMOE_LAUNCH_CHECK();
@@ -306,5 +313,6 @@ extern "C" int dmoe_pack(uint32_t *d_out_order, uint32_t *d_out_inv_order, uint3
     o.offsets = d_out_offsets;
     o.live = d_out_live_experts;
     o.n_live = d_out_n_live;
+    o.bad_ids = w->flags + 1;
     return launch_pack(o, d_indices, n, K, E, 0, w->base, to_hip(s));
 }

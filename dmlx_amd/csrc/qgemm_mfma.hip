@@ -212,9 +212,6 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
     // steps add 0 * w and the loop body is one straight line with no guarded copy. While a trip computes from one
     // LDS buffer, the next block is staged into the other; one barrier per trip publishes it.
     static_assert(kMfmaRing == 4, "the staging schedule below is written for four steps per trip");
-#ifdef DMOE_MFMA_CLOCK // debug aid: cycles per reduction step of a few workgroups
-    const long long exp_t0 = clock64();
-#endif
 #pragma unroll 1
     for (int trip = 0; trip < n_trips; ++trip) {
         const int s0 = trip * kMfmaRing;
@@ -239,11 +236,6 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
         }
     }
 
-#ifdef DMOE_MFMA_CLOCK // debug aid: cycles per reduction step of a few workgroups
-    if (blockIdx.x == 3 && (blockIdx.y % 97) == 5 && tid == 0)
-        printf("MT %d gate_up %d slot %d steps %d clk/step %lld\n", MT, (int)GATE_UP, (int)blockIdx.y, n_steps,
-               (clock64() - exp_t0) / n_steps);
-#endif
     // ---- epilogue: lane = token row (ln), registers r -> output column 8*(r/4) + 4*h + r%4 -------------
     if (!wave_on) return;
 #pragma unroll

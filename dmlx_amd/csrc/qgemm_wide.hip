@@ -157,9 +157,6 @@ __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) read_x(0, 0, mt);
 
-#ifdef DMOE_MFMA_CLOCK // debug aid: cycles per reduction step of a few workgroups
-    const long long exp_t0 = clock64();
-#endif
     // The loop always runs whole trips of kWideRing steps: surplus steps multiply zeroed activations with weights
     // clamped onto the last valid step. Step j of a trip computes from buffer j, requests block s + AHEAD into buffer
     // (j + AHEAD) % 4 during its first three MFMA groups, and at the start of the fourth waits for block s + 1 and
@@ -231,11 +228,6 @@ __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint
             if (!stage && s + AHEAD < n_trips * kWideRing) zero_block((j + AHEAD) % kWideRing); // a surplus step: zeros
         }
     }
-#ifdef DMOE_MFMA_CLOCK
-    if (blockIdx.x == 3 && (blockIdx.y % 97) == 5 && tid == 0)
-        printf("MT %d gate_up %d slot %d steps %d clk/step %lld\n", MT, (int)GATE_UP, (int)blockIdx.y, n_steps,
-               (clock64() - exp_t0) / n_steps);
-#endif
 
     // ---- epilogue: lane = token row (ln), registers r -> output column 8*(r/4) + 4*h + r%4 -------------
     if (!wave_on) return;

@@ -51,13 +51,14 @@ int side_stream_ready(Workspace *w) {
 int stage_flush(Workspace *w) {
     StageTimer &t = w->timer;
     for (int i = 0; i < DMOE_STAGE_COUNT; ++i) {
-        if (!t.pending[i]) continue;
-        DMOE_HIP(hipEventSynchronize(t.stop[i]));
-        float ms = 0.0f;
-        DMOE_HIP(hipEventElapsedTime(&ms, t.start[i], t.stop[i]));
-        t.total_ms[i] += ms;
-        t.samples[i] += 1;
-        t.pending[i] = false;
+        for (int k = 0; k < t.pending[i]; ++k) {
+            DMOE_HIP(hipEventSynchronize(t.stop[i][k]));
+            float ms = 0.0f;
+            DMOE_HIP(hipEventElapsedTime(&ms, t.start[i][k], t.stop[i][k]));
+            t.total_ms[i] += ms;
+            t.samples[i] += 1;
+        }
+        t.pending[i] = 0;
     }
     return DMOE_OK;
 }
@@ -65,16 +66,18 @@ int stage_flush(Workspace *w) {
 int stage_begin(Workspace *w, int stage, hipStream_t st) {
     StageTimer &t = w->timer;
     if (!t.enabled) return DMOE_OK;
-    if (t.pending[stage]) DMOE_TRY(stage_flush(w)); // the event pair is about to be reused
-    DMOE_HIP(hipEventRecord(t.start[stage], st));
+    if (t.pending[stage] == kStageRing) DMOE_TRY(stage_flush(w)); // the ring is full: read it out (waits for the device)
+    DMOE_HIP(hipEventRecord(t.start[stage][t.pending[stage]], st));
+    t.open[stage] = true;
     return DMOE_OK;
 }
 
 int stage_end(Workspace *w, int stage, hipStream_t st) {
     StageTimer &t = w->timer;
-    if (!t.enabled) return DMOE_OK;
-    DMOE_HIP(hipEventRecord(t.stop[stage], st));
-    t.pending[stage] = true;
+    if (!t.enabled || !t.open[stage]) return DMOE_OK;
+    DMOE_HIP(hipEventRecord(t.stop[stage][t.pending[stage]], st));
+    t.pending[stage] += 1;
+    t.open[stage] = false;
     return DMOE_OK;
 }
 
@@ -200,18 +203,20 @@ int dmoe_workspace_set_stage_timing(dmoe_workspace ws, int enabled) {
     Workspace *w = (Workspace *)ws.ctx;
     DMOE_REQUIRE(w != nullptr, "workspace handle is null");
     StageTimer &t = w->timer;
-    if (enabled && !t.start[0]) {
-        for (int i = 0; i < DMOE_STAGE_COUNT; ++i) {
-            DMOE_HIP(hipEventCreate(&t.start[i]));
-            DMOE_HIP(hipEventCreate(&t.stop[i]));
-        }
+    if (enabled && !t.start[0][0]) {
+        for (int i = 0; i < DMOE_STAGE_COUNT; ++i)
+            for (int k = 0; k < kStageRing; ++k) {
+                DMOE_HIP(hipEventCreate(&t.start[i][k]));
+                DMOE_HIP(hipEventCreate(&t.stop[i][k]));
+            }
     }
     if (!enabled && t.enabled) DMOE_TRY(stage_flush(w));
     if (enabled && !t.enabled)
         for (int i = 0; i < DMOE_STAGE_COUNT; ++i) {
             t.total_ms[i] = 0.0f;
             t.samples[i] = 0;
-            t.pending[i] = false;
+            t.pending[i] = 0;
+            t.open[i] = false;
         }
     t.enabled = enabled != 0;
     return DMOE_OK;
@@ -231,10 +236,11 @@ int dmoe_workspace_read_stage_times(float *h_out_total_ms, int *h_out_samples, d
 int dmoe_workspace_destroy(dmoe_workspace ws) {
     Workspace *w = (Workspace *)ws.ctx;
     if (!w) return DMOE_OK;
-    for (int i = 0; i < DMOE_STAGE_COUNT; ++i) {
-        if (w->timer.start[i]) (void)hipEventDestroy(w->timer.start[i]);
-        if (w->timer.stop[i]) (void)hipEventDestroy(w->timer.stop[i]);
-    }
+    for (int i = 0; i < DMOE_STAGE_COUNT; ++i)
+        for (int k = 0; k < kStageRing; ++k) {
+            if (w->timer.start[i][k]) (void)hipEventDestroy(w->timer.start[i][k]);
+            if (w->timer.stop[i][k]) (void)hipEventDestroy(w->timer.stop[i][k]);
+        }
     if (w->side) (void)hipStreamSynchronize(w->side);
     if (w->fork) (void)hipEventDestroy(w->fork);
     if (w->join) (void)hipEventDestroy(w->join);
@@ -256,14 +262,30 @@ int dmoe_workspace_check(dmoe_workspace ws, dmoe_stream s) {
     DMOE_REQUIRE(w != nullptr, "workspace handle is null");
     DMOE_HIP(hipStreamSynchronize(to_hip(s)));
     if (w->side) DMOE_HIP(hipStreamSynchronize(w->side));
-    uint32_t expired = 0;
-    DMOE_HIP(hipMemcpy(&expired, w->flags, sizeof expired, hipMemcpyDeviceToHost));
-    if (expired) {
-        DMOE_HIP(hipMemset(w->flags, 0, sizeof expired));
-        set_error("%u workgroup(s) gave up waiting for their tile's gate/up results: outputs since the last check are invalid",
-                  (unsigned)expired);
+    uint32_t flags[2] = {0, 0}; // [0] waits that gave up, [1] expert ids out of range
+    DMOE_HIP(hipMemcpy(flags, w->flags, sizeof flags, hipMemcpyDeviceToHost));
+    if (flags[0] || flags[1]) DMOE_HIP(hipMemset(w->flags, 0, sizeof flags));
+    if (flags[0]) {
+        // the paired launch relies on the order in which the hardware starts workgroups; after one failure this
+        // workspace stays on the two-launch path, which waits for nothing
+        w->paired = false;
+        set_error("%u workgroup(s) gave up waiting for their tile's gate/up results: outputs since the last check are "
+                  "invalid; this workspace now runs gate/up and down as two launches",
+                  (unsigned)flags[0]);
         return DMOE_ERR_TIMEOUT;
     }
+    if (flags[1]) {
+        set_error("%u expert id(s) outside the layer's expert range reached the packing step (computed as the last "
+                  "expert): outputs since the last check are invalid", (unsigned)flags[1]);
+        return DMOE_ERR_INVALID;
+    }
+    return DMOE_OK;
+}
+
+int dmoe_workspace_set_paired_launch(dmoe_workspace ws, int enabled) {
+    Workspace *w = (Workspace *)ws.ctx;
+    DMOE_REQUIRE(w != nullptr, "workspace handle is null");
+    w->paired = enabled != 0;
     return DMOE_OK;
 }
 

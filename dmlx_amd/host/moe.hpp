@@ -62,6 +62,9 @@ class Context {
     // gave up throws here, as a failed lazy graph throws at eval() in the reference)
     void synchronize() const { check(dmoe_workspace_check(ws_, stream_)); }
     void setWaitLimit(unsigned polls) const { check(dmoe_workspace_set_wait_limit(ws_, polls)); }
+    // decode steps: gate/up and down in one launch (default) or as two launches that wait for nothing; a step that
+    // reported a time-out at synchronize() has already switched the workspace to two launches
+    void setPairedLaunch(bool enabled) const { check(dmoe_workspace_set_paired_launch(ws_, enabled ? 1 : 0)); }
 
   private:
     dmoe_stream stream_{};

@@ -51,6 +51,11 @@ pub const Context = struct {
     pub fn setWaitLimit(self: Context, polls: c_uint) Error!void {
         try check(c.dmoe_workspace_set_wait_limit(self.ws, polls));
     }
+    /// decode steps: gate/up and down in one launch (default) or as two launches that wait for nothing; after `eval`
+    /// reported a time-out the workspace is already on two launches
+    pub fn setPairedLaunch(self: Context, enabled: bool) Error!void {
+        try check(c.dmoe_workspace_set_paired_launch(self.ws, @intFromBool(enabled)));
+    }
 };
 
 /// Dense row-major device array; `deinit` frees it (handles are owned, as `Array.fromHandle` results are).

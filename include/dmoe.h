@@ -38,7 +38,7 @@ typedef enum {
     DMOE_ERR_HIP = 2,         /* a HIP runtime call failed                   */
     DMOE_ERR_UNSUPPORTED = 3, /* valid request this build does not implement */
     DMOE_ERR_NO_DEVICE = 4,   /* no gfx950 device visible                    */
-    DMOE_ERR_TIMEOUT = 5      /* a bounded wait inside a kernel gave up      */
+    DMOE_ERR_TIMEOUT = 5      /* a bounded wait inside a kernel gave up (see dmoe_workspace_check) */
 } dmoe_status;
 
 /* quantization mode; the reference passes it as the C strings "affine"/"mxfp4"
@@ -84,20 +84,33 @@ int dmoe_workspace_create(dmoe_workspace *out, size_t initial_bytes);
 int dmoe_workspace_destroy(dmoe_workspace ws);
 /* bytes currently reserved; growth happens inside calls (it synchronizes the device) */
 int dmoe_workspace_reserved(size_t *out_bytes, dmoe_workspace ws);
-/* Waits for stream s, then reports whether any kernel launched with this workspace since the last check gave up a
- * bounded wait: at decode sizes the down projection's workgroups wait, inside the launch they share with the gate/up
- * projection, for their tile's gate/up workgroups, and give up after the workspace's poll limit (~16 ms) so that the
- * launch ends whatever happens. Returns DMOE_ERR_TIMEOUT (and clears the count) if that happened: the outputs of the
- * calls since the last check must then be discarded. Plays the role of c.check(rc) after Array.eval() in the
- * reference (moe_router.zig:68,74), where a failed lazy graph surfaces at the sync point. */
+/* Waits for stream s, then reports what the kernels launched with this workspace since the last check could not
+ * report through a return code. Plays the role of c.check(rc) after Array.eval() in the reference
+ * (moe_router.zig:68,74), where a failed lazy graph surfaces at the sync point: the outputs of dmoe_moe_forward,
+ * dmoe_moe_layer_forward, dmoe_switch_glu_forward_no_scores, dmoe_gather_qmm* and dmoe_pack are valid once a check
+ * that follows them returns DMOE_OK. Both conditions are cleared by the call that reports them.
+ *   DMOE_ERR_TIMEOUT  a bounded wait gave up. At decode sizes the gate/up and the down projection share one launch:
+ *                     a down workgroup waits for its own tile's gate/up workgroups and gives up after the workspace's
+ *                     poll limit (~16 ms), so that the launch ends whatever happens. That a waiting workgroup's
+ *                     producers are running or done rests on the hardware starting workgroups in index order, which
+ *                     holds on gfx950 but is not promised by the programming model. After this error the workspace
+ *                     runs the two projections as two launches in a row (dmoe_workspace_set_paired_launch(ws, 0)),
+ *                     which wait for nothing; the outputs since the last check must be discarded and recomputed.
+ *   DMOE_ERR_INVALID  an expert id outside the layer's [0, n_experts) reached the packing step. Such a row is computed
+ *                     as the last expert so that every access stays in bounds; the outputs must be discarded. */
 int dmoe_workspace_check(dmoe_workspace ws, dmoe_stream s);
 /* polls (~0.25 us each) a waiting workgroup makes before it gives up; default 65536. For tests of the give-up path. */
 int dmoe_workspace_set_wait_limit(dmoe_workspace ws, unsigned polls);
+/* 1 (default): decode-sized calls run gate/up and down in one launch, as described at dmoe_workspace_check;
+ * 0: always two launches in a row (same results, a few per cent slower, no waits inside kernels). No counterpart in
+ * the reference. */
+int dmoe_workspace_set_paired_launch(dmoe_workspace ws, int enabled);
 
 /* Per-stage device timing of the layer forward calls made with this workspace (HIP events recorded on the
- * call's stream around each stage). Off by default; while on, every forward call waits for the previous
- * call's events, so use it for measurement runs only. No counterpart in the reference, which logs host wall
- * time per token step (expert_stream.zig:587-610). */
+ * call's stream around each stage). Off by default. While on, prefill-sized calls keep their launches in a row on
+ * one stream (so that a stage's time covers all of its tiles), and a forward call waits for the device once 64 calls'
+ * events are unread: use it for measurement runs. No counterpart in the reference, which logs host wall time per
+ * token step (expert_stream.zig:587-610). */
 enum {
     DMOE_STAGE_ROUTE = 0,        /* dmoe_gate_route inside dmoe_moe_layer_forward */
     DMOE_STAGE_PACK = 1,         /* remap + counting sort                         */
@@ -242,7 +255,10 @@ typedef struct {
     dmoe_qweight gate, up, down;/* gate/up: rows=F, cols=D; down: rows=D, cols=F; n_mats = resident slots */
     float swiglu_limit;         /* limitedSwiGLU clamp, 0 = none (:947-966)   */
     int score_before_down;      /* 1 = DSV4SwitchGLU.forward (:796-806); 0 = provider paths
-                                   (expert_stream.zig:575-580, expert_preload.zig:283-289) */
+                                   (expert_stream.zig:575-580, expert_preload.zig:283-289). With 1 the product
+                                   activation * score is rounded to bf16 before the down projection (the
+                                   reference keeps it in f32 after promoting bf16 x f32, :801): one more bf16
+                                   rounding of that operand, inside the 1e-2 output tolerance */
     int has_shared;             /* shared expert (DSV4Expert, :489-517), n_mats = 1, rows/cols as above with its own F */
     dmoe_qweight shared_gate, shared_up, shared_down;
     float shared_swiglu_limit;  /* the reference builds the shared expert with 0 (deepseek_v4_loader.zig:1893) */

@@ -48,3 +48,38 @@ def oracle_forward(wl, idx_slots, weights, want_h=False):
     return oracle.moe_forward(bf16_bits(wl.x), idx_slots, weights, qmat(wl.gate), qmat(wl.up), qmat(wl.down),
                               swiglu_limit=wl.swiglu_limit, score_before_down=wl.score_before_down,
                               shared=shared, shared_swiglu_limit=wl.shared_swiglu_limit, want_h=want_h)
+
+
+def max_abs_rel_rows(got, ref):
+    """Largest per-row error: max over rows of (max |got - ref| over the row) / (max |ref| over the row)."""
+    got = np.asarray(got, np.float64)
+    ref = np.asarray(ref, np.float64)
+    denom = np.abs(ref).max(axis=-1)
+    denom[denom == 0] = 1.0
+    return float((np.abs(got - ref).max(axis=-1) / denom).max())
+
+
+def dense_reference_f64(x_bits, idx, w, gate, up, down, limit=0.0, shared=None, shared_limit=0.0):
+    """The layer in float64 with no intermediate rounding: sum_k w[t,k] * down_e(silu(min(g, L)) * clip(u, -L, L)) +
+    shared(x), from the dequantized weights (oracle.QMat stacks; idx = slot ids). Rows are grouped by expert so that
+    each expert is dequantized once; this is the exact value both the kernels and the oracle approximate."""
+    x = oracle.bf16_to_f32(x_bits).astype(np.float64)
+    T, K = idx.shape
+
+    def ffn(xr, g_, u_, d_, L):          # xr [n, D]
+        g, u = xr @ g_.T, xr @ u_.T
+        if L > 0:
+            g, u = np.minimum(g, L), np.clip(u, -L, L)
+        return (g / (1.0 + np.exp(-g)) * u) @ d_.T
+
+    deq = lambda qm, m: oracle.dequantize_f32(qm, m).astype(np.float64)
+    out = np.zeros((T, down.rows))
+    flat = idx.reshape(-1).astype(np.int64)
+    for e in np.unique(flat):
+        pos = np.nonzero(flat == e)[0]
+        tok = pos // K
+        y = ffn(x[tok], deq(gate, int(e)), deq(up, int(e)), deq(down, int(e)), limit)
+        np.add.at(out, tok, y * w.reshape(-1)[pos].astype(np.float64)[:, None])
+    if shared is not None:
+        out += ffn(x, deq(shared[0], 0), deq(shared[1], 0), deq(shared[2], 0), shared_limit)
+    return out

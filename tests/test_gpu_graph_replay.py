@@ -67,8 +67,9 @@ def test_decode_step_is_reproducible_call_after_call(dmoe, ws, config):
 def test_decode_step_reports_a_wait_that_gave_up(dmoe, ws):
     """Failure handling of the decode launch: its down-projection workgroups wait a bounded number of polls for
     their tile's gate/up workgroups. With the bound forced to zero from the host they give up at once (every kernel
-    still runs to its end), and the workspace check at the next sync point must say so, once; with the default
-    bound back in place the same call is clean and gives the reference bits again."""
+    still runs to its end), and the workspace check at the next sync point must say so, once. From then on the
+    workspace runs the two projections as two launches, which wait for nothing: the next steps are correct and
+    clean even with the zero bound still in place. Switching the paired launch back on restores it."""
     from dmlx_amd.capi import DmoeError
     wl = workloads.make(1, scale=0.25)
     layer = dmoe.Layer(wl.D, wl.F, wl.K, wl.gate, wl.up, wl.down, swiglu_limit=wl.swiglu_limit,
@@ -84,9 +85,35 @@ def test_decode_step_reports_a_wait_that_gave_up(dmoe, ws):
         with pytest.raises(DmoeError, match="gave up"):
             ws.check()
         ws.check()                               # reported once, then cleared
+        for _ in range(3):                       # fallen back to two launches: no wait, so no time-out, right bits
+            out = step()
+            ws.check()
+            assert torch.equal(out, want)
     finally:
         ws.set_wait_limit(1 << 16)
+    ws.set_paired_launch(True)
+    out = step()
+    ws.check()
+    assert torch.equal(out, want)
+    ws.set_paired_launch(False)                  # the API switch gives the same bits
     out = step()
     ws.check()
     assert torch.equal(out, want)
     layer.close()
+
+
+def test_pack_reports_expert_ids_out_of_range(dmoe, ws):
+    """An expert id >= E is packed under the last expert (every access stays in bounds) and the workspace check
+    reports it once, for the one-launch and the three-launch packing kernels."""
+    from dmlx_amd.capi import DmoeError
+    E, K = 16, 2
+    for T in (64, 2000):
+        idx = torch.randint(0, E, (T, K), dtype=torch.int32, device="cuda")
+        dmoe.pack(idx, E, ws)
+        ws.check()
+        idx[T // 2, 1] = E + 3
+        p = dmoe.pack(idx, E, ws)
+        with pytest.raises(DmoeError, match="outside the layer's expert range"):
+            ws.check()
+        ws.check()
+        assert int(p["counts"].sum()) == T * K and int(p["offsets"][E]) == T * K

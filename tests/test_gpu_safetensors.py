@@ -1,6 +1,8 @@
 """Resident upload of a layer's experts from MLX-format safetensors files (dmoe_layer_create_from_safetensors):
-the layer built from the file must behave bit for bit like the layer built from the same tensors in memory,
-including the Smelt subset with its remap; malformed files are rejected with a message."""
+the layer built from the file must give the oracle's outputs when the oracle is fed the bytes an independent numpy
+reader takes from the same file (the reference's own check is "partial read == load + take, bitwise",
+src/tests/numerical_equivalence_test.zig:97-213), including the Smelt subset with its remap; it must also behave bit
+for bit like the layer built from the same tensors in memory; malformed files are rejected with a message."""
 import json
 import os
 import struct
@@ -10,7 +12,10 @@ import pytest
 import torch
 
 from dmlx_amd import workloads
-from tests.helpers import to_np_u32
+from oracle import oracle
+from tests.helpers import bf16_bits, max_abs_rel, to_np_u32
+
+OUT_TOL = 1e-2   # bf16 outputs against the oracle, as everywhere else
 
 pytestmark = pytest.mark.gpu
 
@@ -36,6 +41,91 @@ def write_safetensors(path, tensors, metadata=None):
         f.write(hj)
         for b in blobs:
             f.write(b)
+
+
+_NP = {"U32": np.uint32, "U8": np.uint8, "BF16": np.uint16, "F32": np.float32}
+
+
+def read_safetensors_numpy(path):
+    """An independent reader for the test: 8-byte little-endian header length, JSON header, then the data section the
+    offsets are relative to. bf16 comes back as uint16 bit patterns."""
+    with open(path, "rb") as f:
+        blob = f.read()
+    (n,) = struct.unpack("<Q", blob[:8])
+    header = json.loads(blob[8:8 + n].decode())
+    data = blob[8 + n:]
+    out = {}
+    for name, meta in header.items():
+        if name == "__metadata__":
+            continue
+        a, b = meta["data_offsets"]
+        out[name] = np.frombuffer(data[a:b], dtype=_NP[meta["dtype"]]).reshape(meta["shape"]).copy()
+    return out
+
+
+def _oracle_stack(tensors, layer_idx, group, proj, mode, bits, group_size):
+    """oracle.QMat of `model.layers.{i}.ffn.{group}.{proj}` from the arrays read back from the file"""
+    base = f"model.layers.{layer_idx}.ffn.{group}.{proj}."
+    w = tensors[base + "weight"]
+    if w.ndim == 2:
+        w = w[None]
+    per_word = 32 // bits
+    rows, cols = w.shape[1], w.shape[2] * per_word
+    scales = tensors[base + "scales"]
+    biases = tensors.get(base + "biases")
+    return oracle.QMat(np.ascontiguousarray(w), np.ascontiguousarray(scales),
+                       None if biases is None else np.ascontiguousarray(biases), rows, cols, mode, bits, group_size)
+
+
+@pytest.mark.parametrize("config,mode,group", [(1, "affine", 64), (2, "mxfp4", 32)])
+def test_layer_from_safetensors_against_the_oracle(dmoe, orc, ws, tmp_path, config, mode, group):
+    """File -> HBM -> kernels against file -> numpy -> oracle: routed experts and the shared expert, two shards."""
+    wl = workloads.make(config, scale=0.125)
+    tensors = _layer_tensors(wl, 5, with_shared=True)
+    keys = sorted(tensors)
+    p1, p2 = str(tmp_path / "a.safetensors"), str(tmp_path / "b.safetensors")
+    write_safetensors(p1, {k: tensors[k] for k in keys[::2]}, metadata={"format": "mlx"})
+    write_safetensors(p2, {k: tensors[k] for k in keys[1::2]})
+    disk = dmoe.Layer.from_safetensors([p1, p2], 5, wl.K, mode, group, 4, swiglu_limit=wl.swiglu_limit)
+    back = {**read_safetensors_numpy(p1), **read_safetensors_numpy(p2)}
+    omode = oracle.AFFINE if mode == "affine" else oracle.MXFP4
+    stack = lambda grp, proj: _oracle_stack(back, 5, grp, proj, omode, 4, group)
+    routed = [stack("switch_mlp", p) for p in ("gate_proj", "up_proj", "down_proj")]
+    shared = tuple(stack("shared_experts", p) for p in ("gate_proj", "up_proj", "down_proj"))
+    assert routed[0].n == wl.E and (routed[0].rows, routed[0].cols) == (wl.F, wl.D)
+    idx, w = dmoe.gate_route(wl.scores, wl.bias, wl.resident_mask, wl.K, wl.renorm, wl.route_scale)
+    if wl.remap is not None:   # the file holds the resident experts only: ids go through the workload's remap
+        idx = dmoe.remap_indices(torch.tensor(wl.remap, dtype=torch.int32, device="cuda"), idx)
+    got = disk.forward(wl.x, idx, w, ws).float().cpu().numpy()
+    ws.check()
+    want = orc.moe_forward(bf16_bits(wl.x), to_np_u32(idx), w.cpu().numpy(), *routed, swiglu_limit=wl.swiglu_limit,
+                           shared=shared)
+    err = max_abs_rel(got, want)
+    assert err < OUT_TOL, err
+    disk.close()
+
+
+def test_smelt_subset_from_safetensors_against_the_oracle(dmoe, orc, ws, tmp_path):
+    """Partial read == load + take: the layer uploads only the masked experts and remaps router ids to slots; the
+    oracle takes ALL experts from the same file and the router ids as they are."""
+    wl = workloads.make(1, scale=0.125)
+    path = str(tmp_path / "l0.safetensors")
+    write_safetensors(path, _layer_tensors(wl, 0, with_shared=False))
+    mask = np.zeros(wl.E, np.uint8)
+    mask[1::3] = 1
+    disk = dmoe.Layer.from_safetensors([path], 0, wl.K, "affine", 64, 4, swiglu_limit=wl.swiglu_limit,
+                                       load_shared=False, resident_mask=mask.tolist())
+    assert disk.n_slots == int(mask.sum())
+    back = read_safetensors_numpy(path)
+    routed = [_oracle_stack(back, 0, "switch_mlp", p, oracle.AFFINE, 4, 64) for p in ("gate_proj", "up_proj", "down_proj")]
+    idx, w = dmoe.gate_route(wl.scores, wl.bias, torch.from_numpy(mask).cuda(), wl.K, wl.renorm, wl.route_scale)
+    assert mask[to_np_u32(idx)].all()
+    got = disk.forward(wl.x, idx, w, ws).float().cpu().numpy()   # router ids in, the layer's own remap applied
+    ws.check()
+    want = orc.moe_forward(bf16_bits(wl.x), to_np_u32(idx), w.cpu().numpy(), *routed, swiglu_limit=wl.swiglu_limit)
+    err = max_abs_rel(got, want)
+    assert err < OUT_TOL, err
+    disk.close()
 
 
 def _layer_tensors(wl, layer_idx, with_shared):
@@ -157,6 +247,19 @@ def test_malformed_safetensors_are_rejected(dmoe, tmp_path):
         load([good], group=32)                                 # scales shape contradicts the group size
     with pytest.raises(dmoe.DmoeError, match="dtype"):
         load([good], mode="mxfp4", group=32)                   # bf16 scales are not E8M0 bytes
+    with pytest.raises(dmoe.DmoeError, match="group size must be"):
+        load([good], group=0)                                  # would divide by zero
+    with pytest.raises(dmoe.DmoeError, match="bits must be"):
+        dmoe.Layer.from_safetensors([good], 0, wl.K, "affine", 64, 0, load_shared=False)
+    uneven = dict(tensors)                                     # up_proj with one expert less than gate_proj
+    for kind in ("weight", "scales", "biases"):
+        k = f"model.layers.0.ffn.switch_mlp.up_proj.{kind}"
+        uneven[k] = tensors[k][:-1]
+    bad_n = str(tmp_path / "uneven.safetensors")
+    write_safetensors(bad_n, uneven)
+    mask = [1] * wl.E
+    with pytest.raises(dmoe.DmoeError, match="experts"):
+        dmoe.Layer.from_safetensors([bad_n], 0, wl.K, "affine", 64, 4, load_shared=False, resident_mask=mask)
     bad = str(tmp_path / "bad.safetensors")
     with open(good, "rb") as f:
         blob = f.read()

@@ -373,6 +373,24 @@ def test_moe_forward_against_dense_float64(orc, fmt, before):
     np.testing.assert_allclose(perm, routed1, rtol=1e-5, atol=1e-6)
 
 
+def test_grouped_float64_reference_equals_the_row_by_row_one(orc):
+    """tests/helpers.dense_reference_f64 (rows grouped by expert, used by the GPU accuracy-margin tests at full size)
+    against the row-by-row float64 evaluation above, with separate limits for routed and shared experts."""
+    from tests.helpers import dense_reference_f64
+    gate, up, down = (qmat(q) for q in _small_layer("affine4"))
+    sh = tuple(qmat(q) for q in _small_layer("affine4", E=1, seed=12))
+    rng = np.random.default_rng(9)
+    T, K = 7, 3
+    x_bits = orc.f32_to_bf16(rng.standard_normal((T, 256)).astype(np.float32) * 2)
+    idx = np.stack([rng.choice(4, K, replace=False) for _ in range(T)]).astype(np.uint32)
+    w = rng.random((T, K)).astype(np.float32)
+    want = _dense_reference(orc, x_bits, idx, w, gate, up, down, 0.7, sh)
+    got = dense_reference_f64(x_bits, idx, w, gate, up, down, 0.7, sh, 0.0)
+    np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-14)
+    clamped = dense_reference_f64(x_bits, idx, w, gate, up, down, 0.7, sh, 0.01)
+    assert np.abs(clamped - want).max() > 1e-6      # the shared expert's own limit is applied
+
+
 # ---------------------------------------------------------------- batch builder --------------------------------
 
 def test_batch_builder_reference_cases(orc, golden):
