@@ -70,7 +70,8 @@ EXPORTS = [
     "dmoe_pack", "dmoe_dequantize", "dmoe_gather_qmm",
     "dmoe_resident_weight_create", "dmoe_resident_weight_destroy", "dmoe_gather_qmm_resident",
     "dmoe_layer_create", "dmoe_layer_destroy", "dmoe_moe_forward",
-    "dmoe_switch_glu_forward_no_scores", "dmoe_moe_layer_forward", "dmoe_debug_last_activations",
+    "dmoe_switch_glu_forward_no_scores", "dmoe_moe_layer_forward", "dmoe_moe_layer_forward_static",
+    "dmoe_debug_last_activations",
     "dmoe_gate_create", "dmoe_gate_destroy", "dmoe_gate_forward",
     "dmoe_layer_create_from_safetensors", "dmoe_layer_dims", "dmoe_batch_build", "dmoe_block_post",
 ]
@@ -439,7 +440,8 @@ class Layer:
         return out
 
     def layer_forward(self, x, scores, bias, resident_mask, renorm, route_scale, ws, want_routing=False, out=None):
-        """dmoe_moe_layer_forward; pass `out` to reuse an output tensor"""
+        """dmoe_moe_layer_forward; ws=None calls dmoe_moe_layer_forward_static (the library's static device scratch,
+        no allocation: pass `out` to keep torch from allocating too)."""
         T, E_total = scores.shape
         if out is None:
             out = torch.empty((T, self.hidden), dtype=torch.bfloat16, device=x.device)
@@ -447,9 +449,14 @@ class Layer:
         if want_routing:
             idx = torch.empty((T, self.top_k), dtype=torch.int32, device=x.device)
             w = torch.empty((T, self.top_k), dtype=torch.float32, device=x.device)
-        check(lib().dmoe_moe_layer_forward(_ptr(out), _ptr(idx), _ptr(w), self.h, _ptr(x), _ptr(scores),
-                                           _ptr(bias), _ptr(resident_mask), T, E_total, int(renorm),
-                                           C.c_float(route_scale), ws.h, _stream()))
+        if ws is None:
+            check(lib().dmoe_moe_layer_forward_static(_ptr(out), _ptr(idx), _ptr(w), self.h, _ptr(x), _ptr(scores),
+                                                      _ptr(bias), _ptr(resident_mask), T, E_total, int(renorm),
+                                                      C.c_float(route_scale), _stream()))
+        else:
+            check(lib().dmoe_moe_layer_forward(_ptr(out), _ptr(idx), _ptr(w), self.h, _ptr(x), _ptr(scores),
+                                               _ptr(bias), _ptr(resident_mask), T, E_total, int(renorm),
+                                               C.c_float(route_scale), ws.h, _stream()))
         return (out, idx, w) if want_routing else out
 
     def last_activations(self, T, ws):

@@ -70,6 +70,9 @@ struct Workspace {
     // dmoe_workspace_set_paired_launch, and by dmoe_workspace_check once a wait gave up: the two GEMMs then run as two
     // launches in a row, which wait for nothing.
     bool paired = true;
+    // a workspace over memory it does not own (the static device scratch of the allocation-free entry point):
+    // reserve() never grows it, and nothing that would create a stream or an event runs on it
+    bool fixed = false;
 };
 int side_stream_ready(Workspace *w);  // creates the side stream and its events on first use
 
@@ -80,6 +83,8 @@ int stage_flush(Workspace *w);
 
 // makes sure at least `bytes` are reserved (may synchronize the device and reallocate)
 int workspace_reserve(dmoe_workspace ws, size_t bytes, Workspace **out);
+// the current device's workspace over the static device scratch (layer.hip); resolves its address on first use
+int static_workspace(Workspace **out);
 
 struct Bump {
     size_t off = 0;

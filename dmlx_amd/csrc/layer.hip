@@ -4,6 +4,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <mutex>
 #include <new>
 
 #include "common.h"
@@ -310,7 +311,7 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
         return DMOE_OK;
     }
     const int small_rows = f.small ? 0 : prefill_small_rows(L->gate.view, L->down.view);
-    if (small_rows > 0 && !w->timer.enabled && w->paired) {
+    if (small_rows > 0 && !w->timer.enabled && w->paired && !w->fixed) {
         // Prefill: the small tiles' two GEMMs (one paired launch) depend on the tile list only. They go to the side
         // stream and fill the tails of the two matrix-core launches, which take the large tiles on `st`. (With stage
         // timing on, the launches stay in a row on `st` so that every stage's time covers all of its tiles.)
@@ -329,7 +330,7 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
             return DMOE_OK;
         }
     }
-    if (small_rows > 0) { // stage timing on, or no paired launch: the four launches in a row, each its own stage
+    if (small_rows > 0) { // stage timing on, or no paired launch / no side stream: the four launches in a row, each its own stage
         GemmArgs gu_small = gu, dn_small = dn, gu_big = gu, dn_big = dn;
         gu_small.max_rows = dn_small.max_rows = small_rows;
         gu_big.min_rows = dn_big.min_rows = small_rows + 1;
@@ -383,6 +384,41 @@ static int shared_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     dn.max_tiles = ceil_div(T, tile_m);
     dn.tile_m = tile_m;
     DMOE_TRY(run_gemm(dn, small, st));
+    return DMOE_OK;
+}
+
+// ---- static device scratch of the allocation-free entry point ---------------------------------------------
+// One array per GPU, part of the library's code object (held by every GPU the library runs on until the process
+// ends). In host code `scratch` is only a handle for hipGetSymbolAddress: the device address is looked up once per
+// device and everything below uses that pointer.
+constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
+constexpr size_t kStaticFlagBytes = 256;   // the workspace's flag words sit in front of the bump area
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kStaticMaxDevices = 64;
+static Workspace g_static_ws[kStaticMaxDevices];
+static bool g_static_ready[kStaticMaxDevices];
+static std::mutex g_static_mutex;
+
+int static_workspace(Workspace **out) {
+    int dev = 0;
+    DMOE_HIP(hipGetDevice(&dev));
+    DMOE_REQUIRE(dev >= 0 && dev < kStaticMaxDevices, "static scratch: device index %d is out of range", dev);
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    Workspace &w = g_static_ws[dev];
+    if (!g_static_ready[dev]) {
+        void *ptr = nullptr;
+        DMOE_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch))); // this device's copy (the current device)
+        DMOE_REQUIRE(ptr != nullptr && ((uintptr_t)ptr % 256) == 0, "static scratch: bad device address %p", ptr);
+        w.flags = (uint32_t *)ptr; // never read back on this path (no bounded waits; bad ids stay clamped)
+        w.base = (unsigned char *)ptr + kStaticFlagBytes;
+        w.bytes = kStaticScratchBytes - kStaticFlagBytes;
+        w.device = dev;
+        w.fixed = true;   // never grows, never creates a stream or an event
+        w.paired = false; // gate/up and down as two launches: nothing waits inside a kernel, nothing to check later
+        g_static_ready[dev] = true;
+    }
+    *out = &w;
     return DMOE_OK;
 }
 
@@ -506,7 +542,8 @@ static int forward_common(uint16_t *d_out, uint16_t *y_out, Layer *L, const uint
     // The routed launches are enqueued first: they are the critical path, and the host has all of their run
     // time to enqueue the side stream's work.
     const bool shared = with_shared && L->has_shared && !y_out;
-    const bool side_shared = shared && !f.fold; // else the shared expert is part of the routed launches
+    // else the shared expert is part of the routed launches, or (static scratch: no streams, no events) follows them
+    const bool side_shared = shared && !f.fold && !w->fixed;
     if (side_shared) {
         DMOE_TRY(side_stream_ready(w));
         DMOE_HIP(hipEventRecord(w->fork, st));
@@ -519,6 +556,7 @@ static int forward_common(uint16_t *d_out, uint16_t *y_out, Layer *L, const uint
         DMOE_TRY(stage_end(w, DMOE_STAGE_SHARED, w->side));
         DMOE_HIP(hipEventRecord(w->join, w->side));
     }
+    if (shared && !f.fold && w->fixed) DMOE_TRY(shared_forward(L, w, f, d_x, T, st));
     if (y_out) return DMOE_OK;
     if (side_shared) DMOE_HIP(hipStreamWaitEvent(st, w->join, 0));
     DMOE_TRY(stage_begin(w, DMOE_STAGE_COMBINE, st));
@@ -571,6 +609,28 @@ int dmoe_moe_layer_forward(uint16_t *d_out, uint32_t *d_out_indices, float *d_ou
     DMOE_TRY(dmoe_gate_route(idx, wts, d_scores, d_bias, d_resident_mask, T, E_total, L->K, renorm, route_scale, s));
     DMOE_TRY(stage_end(w, DMOE_STAGE_ROUTE, to_hip(s)));
     return forward_common(d_out, nullptr, L, d_x, idx, wts, T, true, true, ws, s);
+}
+
+int dmoe_moe_layer_forward_static(uint16_t *d_out, uint32_t *d_out_indices, float *d_out_weights, dmoe_layer layer,
+                                  const uint16_t *d_x, const float *d_scores, const float *d_bias,
+                                  const uint8_t *d_resident_mask, int T, int E_total, int renorm, float route_scale,
+                                  dmoe_stream s) {
+    DMOE_REQUIRE(layer.ctx, "moe_layer_forward_static: layer handle is null");
+    const Layer *L = (const Layer *)layer.ctx;
+    DMOE_REQUIRE(T >= 0, "moe_layer_forward_static: T=%d", T);
+    Workspace *w = nullptr;
+    DMOE_TRY(static_workspace(&w));
+    DMOE_REQUIRE(L->device == w->device, "moe_layer_forward_static: the layer lives on device %d, the current device is %d",
+                 L->device, w->device);
+    // same layout as dmoe_moe_layer_forward: the forward's buffers, then the routing outputs
+    const size_t need = forward_layout(L, T).total + 2 * (((size_t)T * L->K * 4 + 255) & ~(size_t)255);
+    DMOE_REQUIRE(need <= w->bytes,
+                 "moe_layer_forward_static: T=%d tokens need %zu bytes of scratch memory, the static device scratch holds "
+                 "%zu (use dmoe_moe_layer_forward with a workspace for larger batches)", T, need, w->bytes);
+    dmoe_workspace ws;
+    ws.ctx = w;
+    return dmoe_moe_layer_forward(d_out, d_out_indices, d_out_weights, layer, d_x, d_scores, d_bias, d_resident_mask, T,
+                                  E_total, renorm, route_scale, ws, s);
 }
 
 int dmoe_debug_last_activations(uint16_t *d_out, dmoe_layer layer, int T, dmoe_workspace ws, dmoe_stream s) {

@@ -25,6 +25,8 @@ int workspace_reserve(dmoe_workspace ws, size_t bytes, Workspace **out) {
     Workspace *w = (Workspace *)ws.ctx;
     DMOE_REQUIRE(w != nullptr, "workspace handle is null");
     if (bytes > w->bytes) {
+        DMOE_REQUIRE(!w->fixed, "this call needs %zu bytes of scratch memory, the static device scratch holds %zu",
+                     bytes, w->bytes);
         // growth is rare (first call at a new size); in-flight work may still use the old block
         DMOE_HIP(hipDeviceSynchronize());
         if (w->base) DMOE_HIP(hipFree(w->base));
@@ -40,6 +42,7 @@ int workspace_reserve(dmoe_workspace ws, size_t bytes, Workspace **out) {
 
 int side_stream_ready(Workspace *w) {
     if (w->side) return DMOE_OK;
+    DMOE_REQUIRE(!w->fixed, "internal: a side stream was asked for on the static device scratch");
     DMOE_HIP(hipStreamCreateWithFlags(&w->side, hipStreamNonBlocking));
     DMOE_HIP(hipEventCreateWithFlags(&w->fork, hipEventDisableTiming));
     DMOE_HIP(hipEventCreateWithFlags(&w->join, hipEventDisableTiming));
@@ -119,6 +122,9 @@ int dmoe_init(int device) {
         set_error("device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
         return DMOE_ERR_NO_DEVICE;
     }
+    // resolve this device's copy of the static scratch now, so that the allocation-free entry point finds it ready
+    Workspace *unused = nullptr;
+    DMOE_TRY(static_workspace(&unused));
     return DMOE_OK;
 }
 

@@ -323,6 +323,23 @@ int dmoe_moe_layer_forward(uint16_t *d_out, uint32_t *d_out_indices, float *d_ou
                            const uint8_t *d_resident_mask, int T, int E_total, int renorm, float route_scale,
                            dmoe_workspace ws, dmoe_stream s);
 
+/* dmoe_moe_layer_forward for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc. It has no counterpart in the reference. Same arguments without the
+ * workspace: all intermediate buffers live in a 16 MiB device array that is part of the library (one per GPU, held
+ * until the process ends), so the call makes no hipMalloc / hipFree and creates no stream or event. Differences from
+ * dmoe_moe_layer_forward:
+ *   - a batch whose buffers do not fit is rejected with DMOE_ERR_INVALID and a message naming the size (at D = 4096,
+ *     F = 2048, K = 6 with a folded shared expert: up to 195 tokens);
+ *   - gate/up and down always run as two launches and a shared expert of another format runs after them on the same
+ *     stream, so nothing waits inside a kernel and there is nothing to check afterwards; results are bit-identical;
+ *   - every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race.
+ * The array's address is resolved by dmoe_init on the device it selects, else by the first call on a device (do not
+ * make that first call under stream capture). */
+int dmoe_moe_layer_forward_static(uint16_t *d_out, uint32_t *d_out_indices, float *d_out_weights, dmoe_layer layer,
+                                  const uint16_t *d_x, const float *d_scores, const float *d_bias,
+                                  const uint8_t *d_resident_mask, int T, int E_total, int renorm, float route_scale,
+                                  dmoe_stream s);
+
 /* ---- router (gate) from the hidden states on ------------------------------------------------ */
 
 /* DSV4Config.ScoringFunc (deepseek_v4.zig:82-86) */
