@@ -250,8 +250,10 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 // limited SwiGLU on the bf16-rounded projections (deepseek_v4.zig:947-966); limit <= 0: plain SwiGLU
 __device__ __forceinline__ float limited_swiglu(float g, float u, float limit) {
-    g = round_bf16(g);
-    u = round_bf16(u);
+    // both roundings in one v_cvt_pk_bf16_f32, the halves widened again with a shift and a mask
+    const uint32_t gu = pack_bf16x2(g, u);
+    g = __uint_as_float(gu << 16);
+    u = __uint_as_float(gu & 0xffff0000u);
     if (limit > 0.0f) {
         g = fminf(g, limit);
         u = fminf(fmaxf(u, -limit), limit);

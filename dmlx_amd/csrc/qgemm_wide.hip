@@ -11,9 +11,12 @@
 //
 //  * Activations go from global memory into LDS without passing through registers (global_load_lds_dwordx4).
 //    One such instruction moves 1 KiB: 8 rows x 128 bytes (one reduction step of 64 bf16). Inside that KiB the
-//    16-byte pieces of row r are stored at position piece ^ r, so that the MFMA operand reads (32 rows at the
-//    same reduction offset) hit 32 different banks; the swizzle costs nothing because each lane picks its
-//    global source address freely.
+//    16-byte pieces of row r are stored at position piece ^ ((r >> 1) & 7). The LDS serves a 16-byte read
+//    instruction 16 lanes (256 bytes, all 64 banks) per cycle, and a lane's place among the banks is
+//    (row & 1) * 8 + position: rows 2q and 2q + 1 differ in the first term, the eight row pairs of a 16-lane group in
+//    the second, so the MFMA operand reads (32 rows at the same reduction offset) run at the full 256 bytes per
+//    cycle (position piece ^ (r & 7) made rows r and r + 8 collide: 155 bytes per cycle measured). The swizzle
+//    costs nothing because each lane picks its global source address freely.
 //  * Four LDS buffers of one reduction step each (4 x 16 KiB): while step s computes, the loads of step s+2
 //    are in flight. The compiler does not know about these loads (they are issued from inline assembly), so
 //    their completion is tracked by hand: VMEM operations return in order, hence "at most MT operations
@@ -88,7 +91,8 @@ __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint
 
     // ---- activation staging -------------------------------------------------------------------------------
     // operation i of this wavefront moves rows (wave + 4 i) * 8 .. + 7; lane = (row r8 of the eight, position c),
-    // and fetches piece c ^ r8 of its row. Rows past the segment end alias the tile's first row (never stored).
+    // and fetches piece c ^ ((row >> 1) & 7) of its row. Rows past the segment end alias the tile's first row (never
+    // stored).
     const int r8 = lane >> 3, c = lane & 7;
     const uint8_t *a_src[MT];
 #pragma unroll
@@ -96,7 +100,7 @@ __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint
         const int r = (wave + 4 * i) * 8 + r8;
         const uint32_t pr = t.row0 + (uint32_t)(r < (int)t.nrows ? r : 0);
         const size_t src = g.a_rows ? g.a_rows[pr] : pr;
-        a_src[i] = (const uint8_t *)(g.a + src * (size_t)cols) + ((c ^ r8) * 16);
+        a_src[i] = (const uint8_t *)(g.a + src * (size_t)cols) + ((c ^ (((r >> 1) & 7))) * 16);
     }
     const uint32_t lds_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
     auto stage_op = [&](int blk, int buf, int i) {
@@ -129,10 +133,10 @@ __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint
     // only safe because those tiles also wait for their own LDS reads before each barrier (see below).
     constexpr int AHEAD = MT <= 2 ? 3 : 2;
     bf16x8_t xf[XB][MT];
-    // fragment (mt, j) of a step: row mt * 32 + ln, piece h * 4 + j, stored at piece ^ (row & 7)
+    // fragment (mt, j) of a step: row mt * 32 + ln, piece h * 4 + j, stored at piece ^ ((row >> 1) & 7)
     const uint8_t *x_rd[NJ];
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) x_rd[j] = lds + (ln >> 3) * 1024 + (ln & 7) * 128 + (((h * 4 + j) ^ (ln & 7)) * 16);
+    for (int j = 0; j < NJ; ++j) x_rd[j] = lds + (ln >> 3) * 1024 + (ln & 7) * 128 + (((h * 4 + j) ^ ((ln >> 1) & 7)) * 16);
     auto read_x = [&](int buf, int j, int mt) {
         uint4 q = *(const uint4 *)(x_rd[j] + buf * kWideBufBytes + mt * 4096);
         xf[j % XB][mt] = __builtin_bit_cast(bf16x8_t, q);
@@ -230,39 +234,61 @@ __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint
     }
 
     // ---- epilogue: lane = token row (ln), registers r -> output column 8*(r/4) + 4*h + r%4 -------------
+    // In that layout a store instruction would touch 32 rows with 16 bytes each. The tile goes through LDS instead
+    // (the activation ring is free once every wavefront has left the loop; each wavefront uses its own 16 KiB): written
+    // as held, read back row-major, so that a store instruction writes whole 64- or 128-byte runs of 16 or 8 rows.
+    __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
+    __syncthreads();
     if (!wave_on) return;
+    constexpr int ROWB = GATE_UP ? 64 : 128;  // bytes of one output row held by this wavefront (32 / 64 columns)
+    constexpr int PITCH = ROWB + 16;
+    constexpr int LPR = ROWB / 16;            // lanes per row when reading back
+    constexpr int RPI = 64 / LPR;             // rows per store instruction
+    uint8_t *mine = lds + wave * (kWideLdsBytes / kWideWaves);
+    const bool wide_store = (((uintptr_t)g.out | ((uintptr_t)g.ldo * 2)) % 16) == 0;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int rl = mt * 32 + ln;
-        if (rl >= (int)t.nrows) continue;
-        const uint32_t p = t.row0 + (uint32_t)rl;
-        const size_t dst = g.out_rows ? g.out_rows[p] : p;
+        const uint32_t p = t.row0 + (uint32_t)(rl < (int)t.nrows ? rl : 0);
+        const uint32_t dst = g.out_rows ? g.out_rows[p] : p;
         float rscale = 1.0f;
         if (g.row_scale) rscale = g.row_scale[g.row_scale_idx ? g.row_scale_idx[p] : p];
-        uint16_t *orow = g.out + dst * (size_t)g.ldo;
+        uint8_t *wrow = mine + ln * PITCH;
         if (GATE_UP) {
 #pragma unroll
             for (int rg = 0; rg < 4; ++rg) {
-                const int n0 = col_base + 8 * rg + 4 * h;
-                if (n0 >= n_out) continue;
                 float v[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                     v[i] = limited_swiglu(acc[mt][0][4 * rg + i], acc[mt][1][4 * rg + i], g.swiglu_limit) * rscale;
-                *(uint2 *)(orow + n0) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+                *(uint2 *)(wrow + (8 * rg + 4 * h) * 2) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
             }
         } else {
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
                 for (int rg = 0; rg < 4; ++rg) {
-                    const int n0 = col_base + 32 * nt + 8 * rg + 4 * h;
-                    if (n0 >= n_out) continue;
                     float v[4];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) v[i] = acc[mt][nt][4 * rg + i] * rscale;
-                    *(uint2 *)(orow + n0) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+                    *(uint2 *)(wrow + (32 * nt + 8 * rg + 4 * h) * 2) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
                 }
+            }
+        }
+        // the same wavefront reads what it wrote: LDS operations of a wavefront complete in order
+#pragma unroll
+        for (int q = 0; q < 32 / RPI; ++q) {
+            const int row = q * RPI + lane / LPR, piece = lane % LPR;
+            const uint32_t drow = (uint32_t)__shfl((int)dst, row, 64); // lane `row` holds that row's destination
+            const uint4 v = *(const uint4 *)(mine + row * PITCH + piece * 16);
+            const int n0 = col_base + piece * 8;
+            if (mt * 32 + row >= (int)t.nrows || n0 >= n_out) continue;
+            uint16_t *o = g.out + (size_t)drow * (size_t)g.ldo + n0;
+            if (wide_store && n0 + 8 <= n_out) {
+                *(uint4 *)o = v;
+            } else {
+                *(uint2 *)o = make_uint2(v.x, v.y);
+                if (n0 + 4 < n_out) *(uint2 *)(o + 4) = make_uint2(v.z, v.w);
             }
         }
     }
@@ -274,7 +300,9 @@ __global__ __launch_bounds__(kWideWaves * 64, 2) void qgemm_wide_kernel(GemmArgs
     Tile t;
     // Workgroups go to the eight XCDs round-robin in launch order. All column strips of a tile are given to ONE XCD
     // (tile = 8 * (k / strips) + xcd for the k-th workgroup of that XCD), so the tile's activations are fetched into one
-    // L2 instead of eight; gridDim.y is a multiple of 8, which makes this a permutation of the grid.
+    // L2 instead of eight; gridDim.y is a multiple of 8, which makes this a permutation of the grid. (Also giving an XCD
+    // runs of 2..16 consecutive tiles of the list, their workgroups of one strip started back to back so that the tiles
+    // of an expert could share its weights through that L2, measured 0.5 % to 15 % slower the longer the run.)
     const uint32_t nx = gridDim.x, b = blockIdx.y * nx + blockIdx.x, k = b >> 3;
     const uint32_t slot = (k / nx) * 8u + (b & 7u);
     const int strip = (int)(k % nx);
@@ -323,7 +351,7 @@ int launch_qgemm_wide(const GemmArgs &g, hipStream_t st) {
                  g.b0.rows, g.b0.cols);
     DMOE_REQUIRE(g.tile_m > 0 && g.tile_m <= kMfmaWideTileM && g.tile_m % 32 == 0, "wide MFMA GEMM: bad tile size %d",
                  g.tile_m);
-    DMOE_REQUIRE(g.max_tiles >= 0 && g.max_tiles <= 65535, "wide MFMA GEMM: %d tiles exceed the grid limit", g.max_tiles);
+    DMOE_REQUIRE(g.max_tiles >= 0 && g.max_tiles <= 65528, "wide MFMA GEMM: %d tiles exceed the grid limit", g.max_tiles);
     DMOE_REQUIRE(g.a && g.out && g.ldo > 0 && g.ldo % 4 == 0 && ((uintptr_t)g.out % 8) == 0 &&
                      ((uintptr_t)g.a % 16) == 0,
                  "wide MFMA GEMM: bad output / activation pointer or pitch");
