@@ -63,7 +63,7 @@ EXPORTS = [
     "dmoe_stream_create", "dmoe_stream_destroy", "dmoe_stream_synchronize",
     "dmoe_malloc", "dmoe_free", "dmoe_copy_to_device", "dmoe_copy_to_host",
     "dmoe_workspace_create", "dmoe_workspace_destroy", "dmoe_workspace_reserved",
-    "dmoe_workspace_check", "dmoe_workspace_set_wait_limit", "dmoe_workspace_set_paired_launch",
+    "dmoe_workspace_check", "dmoe_workspace_set_wait_limit", "dmoe_workspace_set_paired_launch", "dmoe_workspace_set_weight_cache",
     "dmoe_workspace_set_stage_timing", "dmoe_workspace_read_stage_times",
     "dmoe_topk_route", "dmoe_gate_route", "dmoe_remap_indices", "dmoe_expand_tokens",
     "dmoe_reduce_experts", "dmoe_smelt_build_mask", "dmoe_build_remap", "dmoe_preload_remap",
@@ -127,6 +127,10 @@ class Workspace:
 
     def set_wait_limit(self, polls):
         check(lib().dmoe_workspace_set_wait_limit(self.h, C.c_uint(polls)))
+
+    def set_weight_cache(self, enabled):
+        """gather_qmm keeps re-ordered resident copies of the stacks it sees (dmoe_workspace_set_weight_cache)"""
+        check(lib().dmoe_workspace_set_weight_cache(self.h, int(enabled)))
 
     def set_paired_launch(self, enabled):
         check(lib().dmoe_workspace_set_paired_launch(self.h, int(enabled)))

@@ -66,6 +66,11 @@ struct Workspace {
     // pack kernels (see PackOut::bad_ids).
     uint32_t *flags = nullptr;
     uint32_t spin_limit = 1u << 16; // polls of ~0.25 us a waiting workgroup makes before it gives up (~16 ms)
+    // Opt-in (dmoe_workspace_set_weight_cache): re-ordered resident copies of the borrowed MLX-layout stacks that
+    // dmoe_gather_qmm has been called with on this workspace, keyed by the stack's pointers and shape. Owned by
+    // layer.hip (weight_cache_find_or_add / weight_cache_clear).
+    bool cache_weights = false;
+    void *weight_cache = nullptr;
     // gate/up and down of a decode step share one launch (down workgroups wait per tile for gate/up). Switched off by
     // dmoe_workspace_set_paired_launch, and by dmoe_workspace_check once a wait gave up: the two GEMMs then run as two
     // launches in a row, which wait for nothing.
@@ -83,6 +88,8 @@ int stage_flush(Workspace *w);
 
 // makes sure at least `bytes` are reserved (may synchronize the device and reallocate)
 int workspace_reserve(dmoe_workspace ws, size_t bytes, Workspace **out);
+// drops every cached resident copy of the workspace (layer.hip)
+void weight_cache_clear(Workspace *w);
 // the current device's workspace over the static device scratch (layer.hip); resolves its address on first use
 int static_workspace(Workspace **out);
 

@@ -6,6 +6,7 @@
 #include <algorithm>
 #include <mutex>
 #include <new>
+#include <vector>
 
 #include "common.h"
 
@@ -387,6 +388,52 @@ static int shared_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     return DMOE_OK;
 }
 
+// ---- per-workspace cache of resident copies for dmoe_gather_qmm --------------------------------------------
+struct CachedStack {
+    dmoe_qweight key; // the caller's stack as passed (pointers, shape, format)
+    QOwned owned;     // its re-ordered copy
+};
+struct WeightCache {
+    std::vector<CachedStack *> items;
+};
+static bool same_stack(const dmoe_qweight &a, const dmoe_qweight &b) {
+    return a.w == b.w && a.scales == b.scales && a.biases == b.biases && a.n_mats == b.n_mats && a.rows == b.rows &&
+           a.cols == b.cols && a.mode == b.mode && a.bits == b.bits && a.group_size == b.group_size;
+}
+void weight_cache_clear(Workspace *w) {
+    WeightCache *c = (WeightCache *)w->weight_cache;
+    if (!c) return;
+    for (CachedStack *it : c->items) {
+        free_owned(it->owned);
+        delete it;
+    }
+    delete c;
+    w->weight_cache = nullptr;
+}
+// the cached resident view of `qw`, made on first sight (one re-ordering pass, waits for it)
+static int weight_cache_find_or_add(Workspace *w, const dmoe_qweight *qw, const QView **out, hipStream_t st) {
+    if (!w->weight_cache) w->weight_cache = new (std::nothrow) WeightCache();
+    WeightCache *c = (WeightCache *)w->weight_cache;
+    DMOE_REQUIRE(c != nullptr, "gather_qmm: out of host memory");
+    for (CachedStack *it : c->items)
+        if (same_stack(it->key, *qw)) {
+            *out = &it->owned.view;
+            return DMOE_OK;
+        }
+    CachedStack *it = new (std::nothrow) CachedStack();
+    DMOE_REQUIRE(it != nullptr, "gather_qmm: out of host memory");
+    it->key = *qw;
+    int rc = adopt(&it->owned, qw, DMOE_WEIGHTS_BORROW_DEVICE, "gather_qmm (cached stack)", st);
+    if (rc != DMOE_OK) {
+        free_owned(it->owned);
+        delete it;
+        return rc;
+    }
+    c->items.push_back(it);
+    *out = &it->owned.view;
+    return DMOE_OK;
+}
+
 // ---- static device scratch of the allocation-free entry point ---------------------------------------------
 // One array per GPU, part of the library's code object (held by every GPU the library runs on until the process
 // ends). In host code `scratch` is only a handle for hipGetSymbolAddress: the device address is looked up once per
@@ -697,6 +744,13 @@ int dmoe_gather_qmm(uint16_t *d_out, const uint16_t *d_x, const dmoe_qweight *qw
     (void)sorted; // the counting sort is a no-op on already grouped rows
     QView v;
     DMOE_TRY(make_qview(&v, qw, "gather_qmm"));
+    Workspace *w = (Workspace *)ws.ctx;
+    if (w && w->cache_weights && can_pack(v)) {
+        // the workspace keeps a re-ordered copy of this stack: the same kernels on the layout they stream
+        const QView *cached = nullptr;
+        DMOE_TRY(weight_cache_find_or_add(w, qw, &cached, to_hip(s)));
+        return gather_qmm_view(d_out, d_x, *cached, d_lhs_indices, d_rhs_indices, R, ws, s);
+    }
     return gather_qmm_view(d_out, d_x, v, d_lhs_indices, d_rhs_indices, R, ws, s);
 }
 

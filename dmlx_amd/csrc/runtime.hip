@@ -248,6 +248,7 @@ int dmoe_workspace_destroy(dmoe_workspace ws) {
             if (w->timer.stop[i][k]) (void)hipEventDestroy(w->timer.stop[i][k]);
         }
     if (w->side) (void)hipStreamSynchronize(w->side);
+    weight_cache_clear(w);
     if (w->fork) (void)hipEventDestroy(w->fork);
     if (w->join) (void)hipEventDestroy(w->join);
     if (w->packed) (void)hipEventDestroy(w->packed);
@@ -285,6 +286,19 @@ int dmoe_workspace_check(dmoe_workspace ws, dmoe_stream s) {
                   "expert): outputs since the last check are invalid", (unsigned)flags[1]);
         return DMOE_ERR_INVALID;
     }
+    return DMOE_OK;
+}
+
+int dmoe_workspace_set_weight_cache(dmoe_workspace ws, int enabled) {
+    Workspace *w = (Workspace *)ws.ctx;
+    DMOE_REQUIRE(w != nullptr, "workspace handle is null");
+    DMOE_REQUIRE(!w->fixed, "the static device scratch keeps no weight cache");
+    if (!enabled) {
+        // copies may still be read by kernels in flight
+        DMOE_HIP(hipDeviceSynchronize());
+        weight_cache_clear(w);
+    }
+    w->cache_weights = enabled != 0;
     return DMOE_OK;
 }
 

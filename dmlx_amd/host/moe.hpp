@@ -64,6 +64,8 @@ class Context {
     void setWaitLimit(unsigned polls) const { check(dmoe_workspace_set_wait_limit(ws_, polls)); }
     // decode steps: gate/up and down in one launch (default) or as two launches that wait for nothing; a step that
     // reported a time-out at synchronize() has already switched the workspace to two launches
+    // gatherQmm on borrowed MLX-layout arrays: keep re-ordered resident copies of the stacks seen (see dmoe.h)
+    void setWeightCache(bool enabled) const { check(dmoe_workspace_set_weight_cache(ws_, enabled ? 1 : 0)); }
     void setPairedLaunch(bool enabled) const { check(dmoe_workspace_set_paired_launch(ws_, enabled ? 1 : 0)); }
 
   private:

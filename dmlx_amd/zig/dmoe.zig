@@ -51,6 +51,10 @@ pub const Context = struct {
     pub fn setWaitLimit(self: Context, polls: c_uint) Error!void {
         try check(c.dmoe_workspace_set_wait_limit(self.ws, polls));
     }
+    /// gatherQmm on borrowed MLX-layout arrays: keep re-ordered resident copies of the stacks seen (see dmoe.h)
+    pub fn setWeightCache(self: Context, enabled: bool) Error!void {
+        try check(c.dmoe_workspace_set_weight_cache(self.ws, @intFromBool(enabled)));
+    }
     /// decode steps: gate/up and down in one launch (default) or as two launches that wait for nothing; after `eval`
     /// reported a time-out the workspace is already on two launches
     pub fn setPairedLaunch(self: Context, enabled: bool) Error!void {

@@ -224,6 +224,15 @@ int dmoe_gather_qmm(uint16_t *d_out, const uint16_t *d_x, const dmoe_qweight *qw
                     const uint32_t *d_lhs_indices, const uint32_t *d_rhs_indices, int R, int sorted,
                     dmoe_workspace ws, dmoe_stream s);
 
+/* Opt-in for callers that keep the gatherQmm call surface unchanged (borrowed MLX-layout arrays on every call): with
+ * the cache on, dmoe_gather_qmm makes the re-ordered resident copy of a stack the first time it sees it on this
+ * workspace (one pass over the stack, the call waits for it) and streams that copy from then on, as
+ * dmoe_gather_qmm_resident does. A stack is recognised by its three pointers, shape and format: the caller promises
+ * that the arrays behind cached pointers neither change nor are freed while the cache is on. Costs the stack's size
+ * in HBM again. enabled = 0 (the default) drops every copy; so does dmoe_workspace_destroy. Same results either way.
+ * No counterpart in the reference (its QuantizedWeight arrays live as long as the model). */
+int dmoe_workspace_set_weight_cache(dmoe_workspace ws, int enabled);
+
 /* The same call on a stack that was made resident once: mlx-zig's QuantizedWeight is a long-lived object (the w /
  * scales / biases Arrays of DSV4SwitchGLU live as long as the model, deepseek_v4.zig:687-717), and its counterpart
  * here is a copy in HBM re-ordered into the layout the kernels stream (rows in blocks of 32, one contiguous KiB per

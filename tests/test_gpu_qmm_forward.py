@@ -115,6 +115,36 @@ def test_gather_qmm_on_a_resident_stack(dmoe, orc, ws, fmt, R, n_mats, rows, col
     host.close()
 
 
+def test_gather_qmm_weight_cache_gives_the_resident_results(dmoe, orc, ws):
+    """dmoe_workspace_set_weight_cache: the unchanged gatherQmm call (borrowed MLX-layout arrays) is served from a
+    re-ordered copy the workspace makes on first sight. Same bits as the explicit resident handle, the oracle's values
+    within the output tolerance, one copy per stack however often it is called, and dropped when switched off."""
+    g = torch.Generator(device="cuda").manual_seed(77)
+    stacks = [_stack("affine4", 6, 256, 512, 301), _stack("mxfp4", 5, 128, 256, 302), _stack("affine8", 4, 128, 256, 303)]
+    R = 24
+    ws.set_weight_cache(True)
+    try:
+        for rep in range(3):
+            for qw in stacks:
+                x = torch.randn((R, qw.cols), generator=g, device="cuda").to(torch.bfloat16)
+                rhs = torch.randint(0, qw.n_mats, (R,), generator=g, device="cuda", dtype=torch.int32)
+                got = dmoe.gather_qmm(x, qw, rhs, ws)
+                res = dmoe.ResidentWeight(qw)
+                assert torch.equal(got, res.gather_qmm(x, rhs, ws))
+                res.close()
+                want = orc.gather_qmm(bf16_bits(x), qmat(qw), to_np_u32(rhs), None)
+                assert max_abs_rel(got.float().cpu().numpy(), want) < OUT_TOL
+        ws.check()
+    finally:
+        ws.set_weight_cache(False)
+    qw = stacks[0]
+    x = torch.randn((R, qw.cols), generator=g, device="cuda").to(torch.bfloat16)
+    rhs = torch.randint(0, qw.n_mats, (R,), generator=g, device="cuda", dtype=torch.int32)
+    plain = dmoe.gather_qmm(x, qw, rhs, ws)       # cache off again: the MLX-layout path, same values
+    want = orc.gather_qmm(bf16_bits(x), qmat(qw), to_np_u32(rhs), None)
+    assert max_abs_rel(plain.float().cpu().numpy(), want) < OUT_TOL
+
+
 @pytest.mark.parametrize("fmt", FORMATS)
 def test_gather_qmm_seeded_random_shapes(dmoe, orc, ws, fmt):
     """Twelve seeded shapes per format across both paths and both layouts: odd expert counts, weight rows that are
