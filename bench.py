@@ -107,6 +107,44 @@ def measured_peaks(torch):
     return out
 
 
+FP32_VALU_PEAK_TFLOPS = 157.3    # MI355X fp32 vector, published
+
+
+def time_gate(torch, steps, windows):
+    """DSV4Gate.forward (router matmul + sqrt-softplus scoring + biased top-6, deepseek_v4.zig:546-681) from the
+    hidden states on, at the decode and the prefill batch size of the benchmark configurations. It runs in front
+    of the timed step (which starts from the scores) and is bound by the fp32 vector ALU: the matmul's additions are
+    kept in a fixed order so that the selected experts are reproducible bit for bit."""
+    from dmlx_amd import capi
+
+    g = torch.Generator(device="cuda").manual_seed(1)
+    E, D, K = 256, 4096, 6
+    wg = (torch.randn((E, D), generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+    bias = torch.randn((E,), generator=g, device="cuda") * 0.1
+    gate = capi.Gate(wg, K, capi.SCORE_SQRTSOFTPLUS, 1.5, bias=bias)
+    ws = capi.Workspace()
+    out = []
+    for T in (64, 8192):
+        x = torch.randn((T, D), generator=g, device="cuda").to(torch.bfloat16)
+        for _ in range(steps):
+            gate.forward(x, ws)
+        torch.cuda.synchronize()
+        ms = []
+        for _ in range(windows):
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                gate.forward(x, ws)
+            torch.cuda.synchronize()
+            ms.append((time.perf_counter() - t0) * 1e3 / steps)
+        m = statistics.median(ms)
+        tf = 2.0 * T * D * E / (m * 1e-3) / 1e12
+        out.append({"tokens": T, "experts": E, "hidden": D, "ms": m, "fp32_TFLOPs": tf,
+                    "frac_of_fp32_valu_peak": tf / FP32_VALU_PEAK_TFLOPS})
+    gate.close()
+    ws.close()
+    return out
+
+
 def run_config(torch, config, steps, warmup, windows, settle_ms, copy_probe=False):
     """Builds configuration `config`, times it as the module docstring says and returns (workload, timing, analysis
     inputs). The layer and its workspace are released before returning."""
@@ -278,6 +316,7 @@ def main():
     ap.add_argument("--settle-ms", type=float, default=1000.0, help="clock-settling pre-run before the warm-up")
     ap.add_argument("--config", type=int, default=1, choices=[0, 1, 2, 3, 4])
     ap.add_argument("--no-prefill", action="store_true", help="with --config 1: do not also time configuration 3")
+    ap.add_argument("--no-gate", action="store_true", help="do not also time the router (DSV4Gate.forward) in front of the step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-peaks", action="store_true", help="skip the library copy / GEMM reference measurements")
     ap.add_argument("--copy-probe", action="store_true",
@@ -322,6 +361,8 @@ def main():
         # the metric's prefill half: configuration 3 with the same procedure, its own roofline block
         wl3, timing3, U3, counts3 = run_config(torch, 3, args.steps, args.warmup, args.windows, args.settle_ms)
         result["prefill_c3"] = describe(torch, wl3, 3, timing3, U3, counts3, args.steps, args.warmup, counters)
+    if not args.no_gate:
+        result["gate"] = time_gate(torch, args.steps, args.windows)
     print(json.dumps(result))
 
 

@@ -50,6 +50,9 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
     using G = MfmaGeom<Fmt>;
     constexpr int KV = G::KV, KSTEP = G::KSTEP, NJ = G::NJ, KB = G::KB, LDA = G::LDA, NI = G::NI;
     constexpr int NT = 2; // 32-column MFMA tiles per wavefront
+    // Weight steps held in registers. Tiles of at most 64 rows leave half of the accumulator registers free and are
+    // bound by the weight stream (a few dozen rows per expert against 8-bit weights): they keep four steps in flight.
+    constexpr int WR = (MT <= 2 && PACKED && kMfmaRing % 4 == 0) ? 4 : kMfmaWRing;
     const int tid = (int)threadIdx.x, lane = tid & 63, ln = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int cols = g.b0.cols, n_out = g.b0.rows;
@@ -70,8 +73,8 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
         if (n >= n_out) n = n_out - 1; // keep addresses valid; such rows are never stored
         cs[nt].init(b, e, (on ? base : 0) >> 5, ln, h, n);
     }
-    uint4 ring_raw[kMfmaWRing][NT];
-    uint32_t ring_sb[kMfmaWRing][NT][2];
+    uint4 ring_raw[WR][NT];
+    uint32_t ring_sb[WR][NT][2];
     auto load_b = [&](int step, int slot_) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
@@ -82,7 +85,7 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
     };
     // weight loads depend on the tile only: start them first (steps past the end are clamped, their data unused)
 #pragma unroll
-    for (int j = 0; j < kMfmaWRing; ++j) load_b(j < n_steps ? j : n_steps - 1, j);
+    for (int j = 0; j < WR; ++j) load_b(j < n_steps ? j : n_steps - 1, j);
 
     // ---- activation staging ------------------------------------------------------------------------------
     // thread -> (row a_row + 32 * p, 16-byte piece a_piece of each 128-byte granule): eight lanes cover one full
@@ -219,10 +222,10 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
 #pragma unroll
         for (int j = 0; j < kMfmaRing; ++j) {
             const int s = s0 + j;
-            const int s_ahead = s + kMfmaWRing < n_steps ? s + kMfmaWRing : n_steps - 1;
-            load_b(s_ahead, j % kMfmaWRing); // this slot was decoded one step ago
+            const int s_ahead = s + WR < n_steps ? s + WR : n_steps - 1;
+            load_b(s_ahead, j % WR); // this slot was decoded one step ago
             // steps 0, 1: fetch the two halves of the next block; steps 2, 3: store them into the other buffer
-            step_body((j + 1) % kMfmaWRing, j & 1, rd_off, j, [&](int u) {
+            step_body((j + 1) % WR, j & 1, rd_off, j, [&](int u) {
                 constexpr int NU = NJ * MT * NT, every = NU / kOpsPerHalf;
                 static_assert(NU % kOpsPerHalf == 0, "staging operations must spread evenly over the units");
                 if (u % every != 0) return;
