@@ -602,6 +602,7 @@ static inline float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
 /* limitedSwiGLU, deepseek_v4.zig:947-966 (routed) / :500-513 (shared), on bf16
  * operands: every MLX op rounds its result to bf16. The gate is clamped from above
  * only; up is clamped on both sides; limit <= 0 disables the clamp. */
+/* deepseek_v4.zig:947-966; bf16 flow for every limit, see (u9) in the header: parity unpinned vs MLX */
 static inline float limited_swiglu_bf16(float g, float u, float limit) {
     if (limit > 0.0f) {
         g = g < limit ? g : limit;   /* minimum(gate, L)       */

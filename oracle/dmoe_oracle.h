@@ -28,7 +28,14 @@
  *        compared bit for bit; against libm they agree to a few ulp (tests).
  *   (u8) the f32 matmul inside mhcPost sums its hc_mult terms in MLX's order, unknown;
  *        orc_block_post takes them in ascending order with fused multiply-adds.
- * Functions whose results depend on one of (u1), (u3)..(u6) are marked
+ *   (u9) limitedSwiGLU with limit > 0 clamps against f32 scalar ARRAYS (ops.scalarF32,
+ *        deepseek_v4.zig:948-955): if MLX promotes bf16 (+) f32-array to f32 as (u5) assumes for
+ *        the score multiply, the activation and everything after it would be f32 for limit > 0 and
+ *        bf16 only for limit = 0. The oracle keeps ONE flow for both: sigmoid, silu and the product
+ *        are each rounded to bf16, as the limit = 0 branch does on bf16 arrays. It therefore rounds
+ *        at least as often as either reading of the reference; how far the kernels are from the
+ *        exact value is bounded separately against float64 (tests/test_gpu_accuracy_margin.py).
+ * Functions whose results depend on one of (u1), (u3)..(u6), (u9) are marked
  * "parity unpinned vs MLX" at their definition.
  *
  * All matrices are dense row-major. bf16 values travel as uint16_t.

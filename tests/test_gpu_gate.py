@@ -29,6 +29,8 @@ def _case(seed, T, D, E, with_bias, with_mask, spread):
     (1, 128, 8, 2, False, False),
     (700, 1024, 64, 4, True, False),     # several segments per wavefront, sums through scratch
     (4200, 256, 128, 6, True, False),    # many tokens: a wavefront walks all segments itself
+    (1100, 4096, 256, 6, True, False),   # the prefill shape of configurations 3 / 4
+    (900, 520, 300, 5, False, True),     # more than 256 experts, short last segment
 ])
 def test_gate_forward_bit_exact(dmoe, orc, ws, func, T, D, E, K, with_bias, with_mask):
     x, wg, bias, mask = _case(7 + func, T, D, E, with_bias, with_mask, spread=2.0)
