@@ -20,7 +20,7 @@ from tests.helpers import (bf16_bits, dense_reference_f64, max_abs_rel, max_abs_
 
 pytestmark = pytest.mark.gpu
 
-OUT_TOL = 1e-2   # north_star: bf16 outputs within max-abs-rel 1e-2 of the reference
+OUT_TOL = 1e-2   # the stated tolerance: bf16 outputs within max-abs-rel 1e-2 of the reference
 ROW_TOL = 2e-2   # the same measure taken row by row
 
 
