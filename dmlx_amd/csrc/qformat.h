@@ -63,6 +63,7 @@ struct Meta {
 
 struct FmtAffine4 {
     static constexpr int kVals = 32;
+    static constexpr int kMetaEntryBytes = 2; // MLX layout: bf16 scale (and bias) per group
     static constexpr int kDecodeOps = 96; // vector instructions to decode one chunk (scheduling hint only)
     static constexpr bool kRowScale = false;
     __device__ static __forceinline__ void load_meta_raw(const QView &q, const uint8_t *row_s, const uint8_t *row_b,
@@ -159,6 +160,7 @@ struct FmtAffine4 {
 
 struct FmtAffine8 {
     static constexpr int kVals = 16;
+    static constexpr int kMetaEntryBytes = 2;
     static constexpr int kDecodeOps = 44;
     static constexpr bool kRowScale = false;
     __device__ static __forceinline__ void load_meta_raw(const QView &q, const uint8_t *row_s, const uint8_t *row_b,
@@ -208,6 +210,7 @@ struct FmtAffine8 {
 
 struct FmtMxfp4 {
     static constexpr int kVals = 32;
+    static constexpr int kMetaEntryBytes = 1; // MLX layout: one E8M0 byte per group of 32
     static constexpr int kDecodeOps = 20;
     static constexpr bool kRowScale = false;
     __device__ static __forceinline__ void load_meta_raw(const QView &, const uint8_t *row_s, const uint8_t *, int k0,
@@ -278,6 +281,7 @@ struct FmtMxfp4 {
 
 struct FmtFp8Row {
     static constexpr int kVals = 16;
+    static constexpr int kMetaEntryBytes = 0; // no per-group entries
     static constexpr int kDecodeOps = 10;
     static constexpr bool kRowScale = true; // scales: one f32 per row, applied after the reduction
     __device__ static __forceinline__ void load_meta_raw(const QView &, const uint8_t *, const uint8_t *, int,

@@ -31,6 +31,7 @@ namespace dmoe {
 
 constexpr int kSkinnyWaves = 4;          // 32-row blocks of weight rows per workgroup
 constexpr int kSkinnyStages = 8;
+constexpr int kSkinnyGroupedStages = 16; // ring depth when the loads are issued four steps at a time
 constexpr int kSkinnyRowBlock = 8;       // tile rows per row block: the LDS window holds 8 whole rows of activations
 
 __device__ __forceinline__ uint32_t vgpr_const32(uint32_t c) {
@@ -73,7 +74,10 @@ struct SkinnyStage {
 // reach g.tile_done_target before it reads its activations (the other role's output), its weight ring already in flight.
 constexpr int kSkinnySyncNone = 0, kSkinnySyncSignal = 1, kSkinnySyncWait = 2;
 
-template <typename Fmt, bool FACTORED, bool PACKED, int RJT>
+// MBLK (MLX layout only): the scale / bias entries of a row are not fetched one per step (32 cache lines touched per
+// load for 2 useful bytes each, again at every step: these loads, not the weights, bounded the MLX-layout path) but 16
+// bytes at a time - eight bf16 or sixteen E8M0 entries, the next block requested while the current one is in use.
+template <typename Fmt, bool FACTORED, bool PACKED, int RJT, bool MBLK>
 __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, uint8_t *skinny_lds, const bool gate_up,
                                             const int sync, const uint32_t slot) {
     using CS = ChunkStream<Fmt, PACKED>;
@@ -82,7 +86,14 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
     constexpr int NJ = KV / 8;       // MFMAs (K = 16) per step
     // depth of the weight ring: the large-tile copy keeps 16 accumulators per lane and takes a shallower ring to
     // stay inside the same register budget (span boundaries stay whole ring rounds either way)
-    constexpr int STAGES = RJT == 1 ? kSkinnyStages : kSkinnyStages / 2;
+    // MLX layout: a wavefront's load takes 32 bytes out of each of 32 rows, so the four steps that share a 128-byte
+    // line of a row are requested back to back (GROUPED), while the line is still in the vector cache
+    constexpr bool GROUPED = MBLK && RJT == 1;
+    constexpr int LG = 4; // steps per 128-byte line
+    constexpr int STAGES = GROUPED ? kSkinnyGroupedStages : RJT == 1 ? kSkinnyStages : kSkinnyStages / 2;
+    constexpr int PRE = GROUPED ? STAGES - LG : STAGES - 1; // stages requested before the first step is consumed
+    constexpr int ROUND = MBLK && STAGES < 8 ? 8 : STAGES;  // steps per unrolled round (MBLK: whole blocks of entries)
+    static_assert(ROUND % STAGES == 0 && (!MBLK || ROUND % 8 == 0), "rounds are whole turns of the ring");
     constexpr int NM = 1;                           // projections per wavefront
     constexpr int WAVES = 2 * kSkinnyWaves;         // eight wavefronts share one staging of the tile's activations
     const int cg = gate_up ? kSkinnyWaves : WAVES;  // 32-row blocks of weight rows per workgroup
@@ -110,7 +121,47 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
 #pragma unroll
         for (int mi = 0; mi < NM; ++mi) {
             s.raw[mi] = cs[mi].load_chunk_stream(step);
-            cs[mi].load_meta(qv, step, s.sb[mi]);
+            if (!MBLK) cs[mi].load_meta(qv, step, s.sb[mi]);
+        }
+    };
+    // ---- blocks of scale / bias entries (MBLK) -------------------------------------------------------------
+    constexpr int kEntryBytes = Fmt::kMetaEntryBytes;                 // 2: bf16 scale + bf16 bias, 1: E8M0 scale
+    constexpr int EPB = kEntryBytes ? 16 / kEntryBytes : 1;           // entries per 16-byte block
+    const int last_block = MBLK ? (n_steps >> 3) - 1 : 0; // a block spans eight steps
+    uint4 mblk_s[NM][2], mblk_b[NM][2]; // [.][0] in use, [.][1] requested for the steps after it
+    auto load_mblock = [&](int block) {
+        const int b = block < last_block ? block : last_block;
+#pragma unroll
+        for (int mi = 0; mi < NM; ++mi) {
+            mblk_s[mi][1] = *(const uint4 *)(cs[mi].srow + (size_t)b * 16);
+            mblk_b[mi][1] = cs[mi].brow ? *(const uint4 *)(cs[mi].brow + (size_t)b * 16) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    // Raw scale / bias entry of this lane for reduction step `gstep`, whose position in its block, `p8` = gstep % 8,
+    // the caller knows at compile time (the launcher takes this path only when a block spans exactly eight steps, and
+    // the unrolled rounds of the ring are whole multiples of eight). Steps must come in increasing order.
+    auto mblock_meta = [&](int gstep, int p8, uint32_t (*sb)[2]) {
+        if (p8 == 0) { // the step opens a block
+#pragma unroll
+            for (int mi = 0; mi < NM; ++mi) {
+                mblk_s[mi][0] = mblk_s[mi][1];
+                mblk_b[mi][0] = mblk_b[mi][1];
+            }
+            load_mblock((gstep >> 3) + 1);
+        }
+        // entries per step: one shared by both lane halves, or (groups of half a step) one for each half
+        constexpr int EPS = EPB / 8;
+        constexpr int per = 4 / (kEntryBytes ? kEntryBytes : 1); // entries per dword
+        const int e0 = p8 * EPS, dw = e0 / per, sub = e0 - dw * per; // compile-time once unrolled
+        const int shift = 8 * kEntryBytes * sub + (EPS == 2 ? 8 * kEntryBytes * h : 0);
+#pragma unroll
+        for (int mi = 0; mi < NM; ++mi) {
+            const uint4 bs = mblk_s[mi][0], bb = mblk_b[mi][0];
+            const uint32_t ws_ = dw == 0 ? bs.x : dw == 1 ? bs.y : dw == 2 ? bs.z : bs.w;
+            const uint32_t wb_ = dw == 0 ? bb.x : dw == 1 ? bb.y : dw == 2 ? bb.z : bb.w;
+            const uint32_t mask = kEntryBytes == 2 ? 0xffffu : 0xffu;
+            sb[mi][0] = (ws_ >> shift) & mask;
+            sb[mi][1] = (wb_ >> shift) & mask;
         }
     };
 
@@ -178,11 +229,12 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
     };
 
     SkinnyStage<NM> ring[STAGES];
+    if (MBLK) load_mblock(0); // taken over by step 0, which requests block 1
     if (sync == kSkinnySyncWait) {
         // the activations are still being written: start the weight ring, then wait for the tile's producers (one
         // wavefront polls, the barrier holds the others), then fetch the rows
 #pragma unroll
-        for (int j = 0; j < STAGES - 1; ++j)
+        for (int j = 0; j < PRE; ++j)
             if (j < n_steps) load_stage(j, ring[j]);
         if (wave == 0) {
             uint32_t polls = 0;
@@ -208,10 +260,10 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
 #pragma unroll
         for (int mi = 0; mi < NM; ++mi) cs[mi].pin(); // keeps the weight loads behind the requests above
 #pragma unroll
-        for (int j = 0; j < STAGES - 1; ++j)
+        for (int j = 0; j < PRE; ++j)
             if (j < n_steps) load_stage(j, ring[j]);
         // every ring stage holds at least NM loads younger than the activation requests
-        if (n_steps >= STAGES - 1) __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt((STAGES - 1) * NM));
+        if (n_steps >= PRE) __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt(PRE * NM));
         else __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt(0));
     }
     __syncthreads();
@@ -240,12 +292,19 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
 
         // One step: decode every projection's chunk first, then issue the matrix instructions of the projections
         // alternately (independent accumulation chains), then apply the scales. `xs` = step within the span.
-        auto consume = [&](int xs, const SkinnyStage<NM> &s) {
+        auto consume = [&](int gstep, int p8, int xs, const SkinnyStage<NM> &s) {
             const uint8_t *xstep = xlane + (size_t)xs * KSTEP * 2;
             const float *gs_step = gs_lds + xs * rp + 4 * h;
             Meta meta[NM];
+            if (MBLK) {
+                uint32_t sbm[NM][2];
+                mblock_meta(gstep, p8, sbm);
 #pragma unroll
-            for (int mi = 0; mi < NM; ++mi) meta[mi] = CS::meta(s.sb[mi]);
+                for (int mi = 0; mi < NM; ++mi) meta[mi] = CS::meta(sbm[mi]);
+            } else {
+#pragma unroll
+                for (int mi = 0; mi < NM; ++mi) meta[mi] = CS::meta(s.sb[mi]);
+            }
             f32x16_t p[NM];
             if (FACTORED) {
                 // word j of the chunk is exactly the B operand of the step's j-th matrix instruction: decode it
@@ -302,15 +361,15 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
             }
             // with 16 products per lane alive, letting the next step's matrix instructions start before this step's
             // scaling has finished would double them: keep the steps apart (other wavefronts fill the wait)
-            if (RJT > 1) __builtin_amdgcn_sched_barrier(0);
+            if (RJT > 1 || GROUPED) __builtin_amdgcn_sched_barrier(0);
         };
 
         // whole rounds of the ring run without guards (the look-ahead is clamped onto the last step: a few repeated
         // loads at the very end instead of a branch per step); a partial last round runs the guarded copy
-        const int full = n_steps / STAGES * STAGES;
+        const int full = n_steps / ROUND * ROUND;
         int x0 = 0, next_span = span_steps; // first step of the span in LDS, first step of the next one
 #pragma unroll 1
-        for (int s0 = 0; s0 < full; s0 += STAGES) {
+        for (int s0 = 0; s0 < full; s0 += ROUND) {
             if (RJT > 1 && s0 == next_span) {
                 // the next span of the activations replaces the one in LDS (the weight ring stays in flight; its
                 // loads are older than these requests, so the wait covers nothing that was not due anyway)
@@ -326,18 +385,33 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
                 next_span += span_steps;
             }
 #pragma unroll
-            for (int j = 0; j < STAGES; ++j) {
-                const int step = s0 + j, ahead = step + STAGES - 1;
-                load_stage(ahead < n_steps ? ahead : n_steps - 1, ring[(j + STAGES - 1) % STAGES]);
-                consume(step - x0, ring[j]);
+            for (int j = 0; j < ROUND; ++j) {
+                const int step = s0 + j, ahead = step + PRE;
+                if (GROUPED) {
+                    if (j % LG == 0) {
+#pragma unroll
+                        for (int i = 0; i < LG; ++i) load_stage(ahead + i < n_steps ? ahead + i : n_steps - 1, ring[(j + PRE + i) % STAGES]);
+                    }
+                } else {
+                    load_stage(ahead < n_steps ? ahead : n_steps - 1, ring[(j + PRE) % STAGES]);
+                }
+                consume(step, j & 7, step - x0, ring[j % STAGES]);
             }
         }
         if (RJT == 1 && full < n_steps) { // only tiles of one row block get here (larger ones need whole rounds per span)
 #pragma unroll
-            for (int j = 0; j < STAGES; ++j) {
+            for (int j = 0; j < ROUND; ++j) {
                 const int step = full + j;
-                if (step + STAGES - 1 < n_steps) load_stage(step + STAGES - 1, ring[(j + STAGES - 1) % STAGES]);
-                if (step < n_steps) consume(step, ring[j]);
+                if (GROUPED) {
+                    if (j % LG == 0) {
+#pragma unroll
+                        for (int i = 0; i < LG; ++i)
+                            if (step + PRE + i < n_steps) load_stage(step + PRE + i, ring[(j + PRE + i) % STAGES]);
+                    }
+                } else if (step + PRE < n_steps) {
+                    load_stage(step + PRE, ring[(j + PRE) % STAGES]);
+                }
+                if (step < n_steps) consume(step, j & 7, step, ring[j % STAGES]);
             }
         }
 
@@ -399,7 +473,7 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
 // y < a.max_tiles are the gate/up tiles, the next a.max_tiles the down tiles of the same list. The hardware starts
 // workgroups in index order, so every producer of a tile is running or done by the time a consumer of it starts to
 // wait; the down workgroups that become resident while the last gate/up workgroups drain stream their weights meanwhile.
-template <typename Fmt, bool FACTORED, bool PACKED>
+template <typename Fmt, bool FACTORED, bool PACKED, bool MBLK = false>
 __global__ __launch_bounds__(2 * kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArgs a, GemmArgs b, int paired) {
     extern __shared__ __attribute__((aligned(16))) uint8_t skinny_lds[];
     const bool second = paired && blockIdx.y >= (uint32_t)a.max_tiles; // workgroup-uniform
@@ -430,9 +504,9 @@ __global__ __launch_bounds__(2 * kSkinnyWaves * 64) void qgemm_skinny_kernel(Gem
         t.nrows = left < (uint32_t)g.tile_m ? left : (uint32_t)g.tile_m;
     }
     if (__builtin_amdgcn_readfirstlane((int)t.nrows) <= kSkinnyRowBlock)
-        skinny_tile<Fmt, FACTORED, PACKED, 1>(g, t, skinny_lds, g.gate_up, sync, slot);
+        skinny_tile<Fmt, FACTORED, PACKED, 1, MBLK>(g, t, skinny_lds, g.gate_up, sync, slot);
     else
-        skinny_tile<Fmt, FACTORED, PACKED, kSkinnyTileM / kSkinnyRowBlock>(g, t, skinny_lds, g.gate_up, sync, slot);
+        skinny_tile<Fmt, FACTORED, PACKED, kSkinnyTileM / kSkinnyRowBlock, MBLK>(g, t, skinny_lds, g.gate_up, sync, slot);
 }
 
 static int skinny_vals(const QView &b) {
@@ -457,13 +531,25 @@ bool qgemm_skinny_supports(const QView &b) {
     return b.mode != DMOE_QUANT_NONE && b.cols % (2 * skinny_vals(b)) == 0 && skinny_lds_bytes(b) <= 150 * 1024;
 }
 
+// rows of scales (and biases) that are 16-byte aligned and a whole number of 16-byte blocks long
+static bool mlx_meta_blocks(const QView &b) {
+    if (b.packed || b.group <= 0 || !b.scales) return false;
+    const size_t esz = b.mode == DMOE_QUANT_MXFP4 ? 1 : 2, row = (size_t)(b.cols / b.group) * esz;
+    if (b.mode != DMOE_QUANT_MXFP4 && b.mode != DMOE_QUANT_AFFINE) return false;
+    // a block of entries must span exactly eight reduction steps (affine 4-bit: groups of 64; MXFP4: 32; 8-bit: 32)
+    const int kstep = b.bits == 4 ? 64 : 32;
+    if ((int)(16 / esz) * b.group != 8 * kstep) return false;
+    return row >= 16 && row % 16 == 0 && b.s_row % 16 == 0 && b.s_mat % 16 == 0 && ((uintptr_t)b.scales % 16) == 0 &&
+           (!b.biases || ((uintptr_t)b.biases % 16) == 0);
+}
+
 struct SkinnyLaunch {
     const GemmArgs &g;
     hipStream_t st;
     const GemmArgs *second = nullptr; // paired launch: the down projection behind the gate/up GEMM `g`
-    template <typename Fmt, bool FACTORED, bool PACKED>
+    template <typename Fmt, bool FACTORED, bool PACKED, bool MBLK = false>
     int go() {
-        auto kern = qgemm_skinny_kernel<Fmt, FACTORED, PACKED>;
+        auto kern = qgemm_skinny_kernel<Fmt, FACTORED, PACKED, MBLK>;
         const size_t lds = skinny_lds_bytes(g.b0);
         static thread_local size_t allowed = 0; // per instantiation: raise the dynamic LDS limit once
         if (lds > allowed) {
@@ -493,6 +579,10 @@ struct SkinnyLaunch {
         constexpr bool can_factor = std::is_same<Fmt, FmtAffine4>::value;
         const bool factor = can_factor && g.b0.group >= 64;
         if (g.b0.packed) return factor ? go<Fmt, can_factor, true>() : go<Fmt, false, true>();
+        // MLX layout: scale / bias entries in 16-byte blocks when every row of them is a whole number of blocks
+        constexpr bool has_entries = Fmt::kMetaEntryBytes != 0;
+        if (has_entries && mlx_meta_blocks(g.b0) && (!second || mlx_meta_blocks(second->b0)) && (!g.gate_up || mlx_meta_blocks(g.b1)))
+            return factor ? go<Fmt, can_factor, false, has_entries>() : go<Fmt, false, false, has_entries>();
         return factor ? go<Fmt, can_factor, false>() : go<Fmt, false, false>();
     }
 };
