@@ -74,6 +74,13 @@ struct SkinnyStage {
 // reach g.tile_done_target before it reads its activations (the other role's output), its weight ring already in flight.
 constexpr int kSkinnySyncNone = 0, kSkinnySyncSignal = 1, kSkinnySyncWait = 2;
 
+// LDS: [activation window][sums of x per step][GROUPED only: 4 KiB per wavefront for turning weight lines]
+__host__ __device__ constexpr size_t skinny_turn_offset(int cols, int kstep) {
+    return (size_t)kSkinnyRowBlock * (size_t)cols * 2 + (size_t)kSkinnyTileM * 16 +
+           (size_t)(cols / kstep) * kSkinnyRowBlock * sizeof(float) + 128;
+}
+constexpr size_t kSkinnyTurnBytes = (size_t)2 * kSkinnyWaves * 4 * 1024;
+
 // MBLK (MLX layout only): the scale / bias entries of a row are not fetched one per step (32 cache lines touched per
 // load for 2 useful bytes each, again at every step: these loads, not the weights, bounded the MLX-layout path) but 16
 // bytes at a time - eight bf16 or sixteen E8M0 entries, the next block requested while the current one is in use.
@@ -86,12 +93,17 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
     constexpr int NJ = KV / 8;       // MFMAs (K = 16) per step
     // depth of the weight ring: the large-tile copy keeps 16 accumulators per lane and takes a shallower ring to
     // stay inside the same register budget (span boundaries stay whole ring rounds either way)
-    // MLX layout: a wavefront's load takes 32 bytes out of each of 32 rows, so the four steps that share a 128-byte
-    // line of a row are requested back to back (GROUPED), while the line is still in the vector cache
+    // MLX layout, tiles of one row block (GROUPED): in the operand layout a wavefront's load would take 32 bytes out of
+    // each of 32 rows (32 cache lines per instruction, a quarter of each used, the same lines again for the next three
+    // steps; measured 2.7 TB/s at best). Instead lane l of load i fetches 16 bytes of row 8 i + l / 8, eight lanes
+    // covering one 128-byte line = the row's codes of four steps; the four loads of such a group wait in the register
+    // ring like any other stage, and when their steps come up the wavefront turns them into the operand layout through
+    // 4 KiB of LDS of its own (written as loaded, read back per step; a wavefront's LDS operations complete in order, so
+    // no barrier is involved).
     constexpr bool GROUPED = MBLK && RJT == 1;
-    constexpr int LG = 4; // steps per 128-byte line
+    constexpr int LG = 4; // steps per 128-byte line = loads per group
     constexpr int STAGES = GROUPED ? kSkinnyGroupedStages : RJT == 1 ? kSkinnyStages : kSkinnyStages / 2;
-    constexpr int PRE = GROUPED ? STAGES - LG : STAGES - 1; // stages requested before the first step is consumed
+    constexpr int PRE = GROUPED ? STAGES : STAGES - 1; // stages requested before the first step is consumed
     constexpr int ROUND = MBLK && STAGES < 8 ? 8 : STAGES;  // steps per unrolled round (MBLK: whole blocks of entries)
     static_assert(ROUND % STAGES == 0 && (!MBLK || ROUND % 8 == 0), "rounds are whole turns of the ring");
     constexpr int NM = 1;                           // projections per wavefront
@@ -117,7 +129,29 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
     CS cs[NM];
 #pragma unroll
     for (int mi = 0; mi < NM; ++mi) cs[mi].init(qv, e, col0 >> 5, ln, h, n);
-    auto load_stage = [&](int step, SkinnyStage<NM> &s) {
+    // GROUPED: byte offset of this lane's piece in load i of a group, from the matrix's first row. Piece c of row r
+    // lands at position c ^ ((r >> 1) & 7) of the row's 128 bytes in LDS, so that the operand reads below (32 rows at
+    // the same piece) spread over all banks; the lane simply fetches the piece that belongs at its position.
+    uint32_t line_off[LG];
+    const uint8_t *const wmat = qv.w + e * qv.w_mat;
+    if (GROUPED) {
+#pragma unroll
+        for (int i = 0; i < LG; ++i) {
+            const int r = 8 * i + (lane >> 3);
+            int nr = col0 + r;
+            if (nr >= n_out) nr = n_out - 1;
+            line_off[i] = (uint32_t)nr * (uint32_t)qv.w_row + (uint32_t)(((lane & 7) ^ ((r >> 1) & 7)) * 16);
+        }
+    }
+    // stage `step`: the chunk of reduction step `step`; GROUPED: load `step % 4` of group `step / 4` (i = step % 4 is
+    // passed apart so that it stays a compile-time constant)
+    auto load_stage = [&](int step, SkinnyStage<NM> &s, int i = 0) {
+        if (GROUPED) {
+            typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+            const u32x4_t v = __builtin_nontemporal_load((const u32x4_t *)(wmat + line_off[i] + (size_t)(step >> 2) * 128));
+            s.raw[0] = make_uint4(v.x, v.y, v.z, v.w);
+            return;
+        }
 #pragma unroll
         for (int mi = 0; mi < NM; ++mi) {
             s.raw[mi] = cs[mi].load_chunk_stream(step);
@@ -235,7 +269,7 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
         // wavefront polls, the barrier holds the others), then fetch the rows
 #pragma unroll
         for (int j = 0; j < PRE; ++j)
-            if (j < n_steps) load_stage(j, ring[j]);
+            if (j < n_steps) load_stage(j, ring[j], j % LG);
         if (wave == 0) {
             uint32_t polls = 0;
             while (__hip_atomic_load(&g.tile_done[slot], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < g.tile_done_target &&
@@ -261,7 +295,7 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
         for (int mi = 0; mi < NM; ++mi) cs[mi].pin(); // keeps the weight loads behind the requests above
 #pragma unroll
         for (int j = 0; j < PRE; ++j)
-            if (j < n_steps) load_stage(j, ring[j]);
+            if (j < n_steps) load_stage(j, ring[j], j % LG);
         // every ring stage holds at least NM loads younger than the activation requests
         if (n_steps >= PRE) __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt(PRE * NM));
         else __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt(0));
@@ -364,6 +398,30 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
             if (RJT > 1 || GROUPED) __builtin_amdgcn_sched_barrier(0);
         };
 
+        // GROUPED: ring stages j .. j+3 (one group as loaded) -> the chunks of its four steps in the operand layout
+        uint8_t *const turn_lds = skinny_lds + skinny_turn_offset(cols, KSTEP) + wave * (LG * 1024);
+        const uint8_t *const turn_rd = turn_lds + ln * 128;
+        const int turn_sw = (ln >> 1) & 7;
+        uint4 turned_raw[LG];
+        SkinnyStage<NM> turned;
+        // A group is written one group ahead of its use, right behind the reads of the group before it (same
+        // buffer: the reads have been issued, and the LDS keeps a wavefront's operations in order), so the reads at
+        // the head of a group never wait for their own writes.
+        auto turn_write = [&](int j) {
+#pragma unroll
+            for (int i = 0; i < LG; ++i) *(uint4 *)(turn_lds + i * 1024 + lane * 16) = ring[j + i].raw[0];
+        };
+        auto turn_read = [&]() {
+#pragma unroll
+            for (int jj = 0; jj < LG; ++jj) turned_raw[jj] = *(const uint4 *)(turn_rd + (((2 * jj + h) ^ turn_sw) * 16));
+        };
+        if (GROUPED) {
+            turn_write(0);
+#pragma unroll
+            for (int i = 0; i < LG; ++i) // the stages of group 0 are free again: the group one round on
+                load_stage(STAGES + i < n_steps ? STAGES + i : n_steps - LG + i, ring[i], i);
+        }
+
         // whole rounds of the ring run without guards (the look-ahead is clamped onto the last step: a few repeated
         // loads at the very end instead of a branch per step); a partial last round runs the guarded copy
         const int full = n_steps / ROUND * ROUND;
@@ -389,12 +447,17 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
                 const int step = s0 + j, ahead = step + PRE;
                 if (GROUPED) {
                     if (j % LG == 0) {
+                        turn_read();
+                        turn_write((j + LG) % STAGES); // the next group; its stages then take the loads a round later
 #pragma unroll
-                        for (int i = 0; i < LG; ++i) load_stage(ahead + i < n_steps ? ahead + i : n_steps - 1, ring[(j + PRE + i) % STAGES]);
+                        for (int i = 0; i < LG; ++i) // past the end: the last group again (unused)
+                            load_stage(ahead + LG + i < n_steps ? ahead + LG + i : n_steps - LG + i, ring[(j + LG) % STAGES + i], i);
                     }
-                } else {
-                    load_stage(ahead < n_steps ? ahead : n_steps - 1, ring[(j + PRE) % STAGES]);
+                    turned.raw[0] = turned_raw[j % LG];
+                    consume(step, j & 7, step - x0, turned);
+                    continue;
                 }
+                load_stage(ahead < n_steps ? ahead : n_steps - 1, ring[(j + PRE) % STAGES]);
                 consume(step, j & 7, step - x0, ring[j % STAGES]);
             }
         }
@@ -402,15 +465,18 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
 #pragma unroll
             for (int j = 0; j < ROUND; ++j) {
                 const int step = full + j;
-                if (GROUPED) {
-                    if (j % LG == 0) {
-#pragma unroll
-                        for (int i = 0; i < LG; ++i)
-                            if (step + PRE + i < n_steps) load_stage(step + PRE + i, ring[(j + PRE + i) % STAGES]);
+                if (GROUPED) { // the reduction is a whole number of groups, and everything left is already in the ring
+                    if (step < n_steps) {
+                        if (j % LG == 0) {
+                            turn_read();
+                            if (step + LG < n_steps) turn_write((j + LG) % STAGES);
+                        }
+                        turned.raw[0] = turned_raw[j % LG];
+                        consume(step, j & 7, step, turned);
                     }
-                } else if (step + PRE < n_steps) {
-                    load_stage(step + PRE, ring[(j + PRE) % STAGES]);
+                    continue;
                 }
+                if (step + PRE < n_steps) load_stage(step + PRE, ring[(j + PRE) % STAGES]);
                 if (step < n_steps) consume(step, j & 7, step, ring[j % STAGES]);
             }
         }
@@ -513,9 +579,8 @@ static int skinny_vals(const QView &b) {
     return (b.mode == DMOE_QUANT_AFFINE && b.bits == 4) || b.mode == DMOE_QUANT_MXFP4 ? 32 : 16;
 }
 static size_t skinny_lds_bytes(const QView &b) {
-    size_t x = (size_t)kSkinnyRowBlock * (size_t)b.cols * 2 + (size_t)kSkinnyTileM * 16;
-    size_t sums = (size_t)(b.cols / (2 * skinny_vals(b))) * kSkinnyRowBlock * sizeof(float);
-    return x + sums + 128; // a two-row-block tile reads (and ignores) up to 24 floats past its last step's sums
+    // a two-row-block tile reads (and ignores) up to 24 floats past its last step's sums: the 128 bytes in the offset
+    return skinny_turn_offset(b.cols, 2 * skinny_vals(b));
 }
 
 // Rows per tile to build tile lists with for this weight shape: a tile of 2 (4) row blocks splits the reduction
@@ -539,6 +604,9 @@ static bool mlx_meta_blocks(const QView &b) {
     // a block of entries must span exactly eight reduction steps (affine 4-bit: groups of 64; MXFP4: 32; 8-bit: 32)
     const int kstep = b.bits == 4 ? 64 : 32;
     if ((int)(16 / esz) * b.group != 8 * kstep) return false;
+    if (skinny_lds_bytes(b) + kSkinnyTurnBytes > 150 * 1024 || b.w_row % 128 != 0 || ((uintptr_t)b.w % 16) != 0 || b.w_mat % 16 != 0 ||
+        (uint64_t)b.rows * (uint64_t)b.w_row >= (1ull << 32))
+        return false; // the line-wise weight loads of the small tiles: LDS to turn them in, whole lines per group
     return row >= 16 && row % 16 == 0 && b.s_row % 16 == 0 && b.s_mat % 16 == 0 && ((uintptr_t)b.scales % 16) == 0 &&
            (!b.biases || ((uintptr_t)b.biases % 16) == 0);
 }
@@ -550,7 +618,7 @@ struct SkinnyLaunch {
     template <typename Fmt, bool FACTORED, bool PACKED, bool MBLK = false>
     int go() {
         auto kern = qgemm_skinny_kernel<Fmt, FACTORED, PACKED, MBLK>;
-        const size_t lds = skinny_lds_bytes(g.b0);
+        const size_t lds = skinny_lds_bytes(g.b0) + (MBLK ? kSkinnyTurnBytes : 0);
         static thread_local size_t allowed = 0; // per instantiation: raise the dynamic LDS limit once
         if (lds > allowed) {
             DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(150 * 1024)));
@@ -563,7 +631,7 @@ struct SkinnyLaunch {
             GemmArgs a = g, b = *second;
             a.tile_done_target = b.tile_done_target = (uint32_t)blocks_x(g);
             b.tile_done = a.tile_done;
-            const size_t lds2 = std::max(lds, skinny_lds_bytes(second->b0));
+            const size_t lds2 = std::max(lds, skinny_lds_bytes(second->b0) + (MBLK ? kSkinnyTurnBytes : 0));
             dim3 grid((unsigned)std::max(blocks_x(a), blocks_x(b)), (unsigned)(2 * g.max_tiles));
             hipLaunchKernelGGL(kern, grid, block, lds2, st, a, b, 1);
         } else {

@@ -31,6 +31,9 @@ def _stack(fmt, n, rows, cols, seed):
     if fmt == "affine8":
         a, s, b = Q.quantize_affine(w, 64, 8)
         return QWeight(a, s, b, rows, cols, QUANT_AFFINE, 8, 64)
+    if fmt == "affine8g32":
+        a, s, b = Q.quantize_affine(w, 32, 8)
+        return QWeight(a, s, b, rows, cols, QUANT_AFFINE, 8, 32)
     if fmt == "mxfp4":
         a, s = Q.quantize_mxfp4(w)
         return QWeight(a, s, None, rows, cols, QUANT_MXFP4, 4, 32)
@@ -114,6 +117,30 @@ def test_gather_qmm_on_a_resident_stack(dmoe, orc, ws, fmt, R, n_mats, rows, col
     host = dmoe.ResidentWeight(qw.to("cpu"))          # the same stack handed over from host memory
     assert torch.equal(host.gather_qmm(x, rhs, ws), got if False else dmoe.ResidentWeight(qw).gather_qmm(x, rhs, ws))
     host.close()
+
+
+@pytest.mark.parametrize("fmt", ["affine4", "mxfp4", "affine8g32"])
+@pytest.mark.parametrize("rows,cols", [(96, 512), (200, 1536), (256, 4096), (64, 1024)])
+def test_gather_qmm_mlx_layout_line_loads(dmoe, orc, ws, fmt, rows, cols):
+    """Decode-sized calls on the MLX layout whose scale rows are whole 16-byte blocks: the weight-streaming kernel then
+    loads whole 128-byte lines and turns them in LDS, and takes scales / biases eight steps at a time. Reductions of one
+    half round (8 steps), of rounds plus a half, of several rounds; weight rows that end inside a wavefront's block.
+    Same bits as the re-ordered copy of the stack, and the oracle's values within the output bar."""
+    n_mats = 5
+    qw = _stack(fmt, n_mats, rows, cols, 11)
+    g = torch.Generator(device="cuda").manual_seed(rows + cols)
+    for R in (1, 7, 33):
+        x = torch.randn((R + 2, cols), generator=g, device="cuda").to(torch.bfloat16)
+        rhs = torch.randint(0, n_mats, (R,), generator=g, device="cuda", dtype=torch.int32)
+        lhs = torch.randint(0, R + 2, (R,), generator=g, device="cuda", dtype=torch.int32)
+        got = dmoe.gather_qmm(x, qw, rhs, ws, lhs)
+        want = orc.gather_qmm(bf16_bits(x), qmat(qw), to_np_u32(rhs), to_np_u32(lhs))
+        assert max_abs_rel(got.float().cpu().numpy(), want) < OUT_TOL, (fmt, R)
+        if rows % 32 == 0:
+            res = dmoe.ResidentWeight(qw)
+            assert torch.equal(got, res.gather_qmm(x, rhs, ws, lhs)), (fmt, R)
+            res.close()
+    ws.check()
 
 
 def test_gather_qmm_weight_cache_gives_the_resident_results(dmoe, orc, ws):
