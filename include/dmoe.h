@@ -236,8 +236,9 @@ int dmoe_workspace_set_weight_cache(dmoe_workspace ws, int enabled);
 /* The same call on a stack that was made resident once: mlx-zig's QuantizedWeight is a long-lived object (the w /
  * scales / biases Arrays of DSV4SwitchGLU live as long as the model, deepseek_v4.zig:687-717), and its counterpart
  * here is a copy in HBM re-ordered into the layout the kernels stream (rows in blocks of 32, one contiguous KiB per
- * wavefront and reduction step). dmoe_gather_qmm on the MLX layout gives the same bits but reads 32 cache lines per
- * load; at decode sizes the resident stack streams about five times faster. `weight_source` as in dmoe_layer_desc
+ * wavefront and reduction step). dmoe_gather_qmm on the MLX layout gives the same bits; at decode sizes the
+ * resident stack streams about 1.3 times faster (the MLX layout needs whole cache lines turned through LDS, and
+ * scales / biases fetched apart), and shapes whose scale rows are not whole 16-byte blocks several times faster. `weight_source` as in dmoe_layer_desc
  * (the stack is always copied: it is re-ordered). Shapes that cannot be re-ordered (rows not a multiple of 32) stay
  * in the MLX layout inside the handle. */
 int dmoe_resident_weight_create(dmoe_resident_weight *out, const dmoe_qweight *qw, int weight_source, dmoe_stream s);
