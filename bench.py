@@ -145,12 +145,13 @@ def time_gate(torch, steps, windows):
     return out
 
 
-def run_config(torch, config, steps, warmup, windows, settle_ms, copy_probe=False):
+def run_config(torch, config, steps, warmup, windows, settle_ms, copy_probe=False, score_before_down=False):
     """Builds configuration `config`, times it as the module docstring says and returns (workload, timing, analysis
     inputs). The layer and its workspace are released before returning."""
     from dmlx_amd import capi, workloads
 
     wl = workloads.make(config, device="cuda")
+    wl.score_before_down = bool(score_before_down)
     layer = capi.Layer(wl.D, wl.F, wl.K, wl.gate, wl.up, wl.down, swiglu_limit=wl.swiglu_limit,
                        score_before_down=wl.score_before_down, shared=wl.shared,
                        shared_swiglu_limit=wl.shared_swiglu_limit, remap=wl.remap, borrow=True)
@@ -292,6 +293,8 @@ def describe(torch, wl, config, timing, U, counts, steps, warmup, counters):
         "config": {"workload": wl.name, "baseline_config": config, "tokens": wl.T, "hidden": wl.D,
                    "ffn": wl.F, "experts": wl.E_total, "resident_experts": wl.E, "top_k": wl.K,
                    "shared_expert": wl.shared is not None,
+                   "routing_weight": "before the down projection (DSV4SwitchGLU.forward)" if wl.score_before_down
+                   else "after the down projection (expert provider paths)",
                    "weights": {0: "affine", 1: "mxfp4", 2: "fp8row", 3: "unquantized"}[wl.gate.mode] + f"-{wl.gate.bits}bit",
                    "max_rows_per_expert": int(counts.max()),
                    "experts_by_rows": {"0": int((counts == 0).sum()), "1-9": int(((counts >= 1) & (counts < 10)).sum()),
@@ -315,6 +318,9 @@ def main():
     ap.add_argument("--windows", type=int, default=9, help="timed windows of --steps steps; the median is reported")
     ap.add_argument("--settle-ms", type=float, default=1000.0, help="clock-settling pre-run before the warm-up")
     ap.add_argument("--config", type=int, default=1, choices=[0, 1, 2, 3, 4])
+    ap.add_argument("--score-before-down", type=int, default=0, choices=[0, 1],
+                    help="1: routing weight applied to the activation before the down projection (DSV4SwitchGLU.forward); "
+                         "0: to the expert outputs (expert provider paths)")
     ap.add_argument("--no-prefill", action="store_true", help="with --config 1: do not also time configuration 3")
     ap.add_argument("--no-gate", action="store_true", help="do not also time the router (DSV4Gate.forward) in front of the step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -337,7 +343,7 @@ def main():
     counters = recorded_counters()
 
     wl, timing, U, counts = run_config(torch, args.config, args.steps, args.warmup, args.windows, args.settle_ms,
-                                       args.copy_probe)
+                                       args.copy_probe, args.score_before_down)
     body = describe(torch, wl, args.config, timing, U, counts, args.steps, args.warmup, counters)
     result = {"metric": "MoE-FFN tokens/s; HBM GB/s at decode, MFMA % at prefill (4-bit top-6/256)",
               "value": body.pop("value"), "unit": body.pop("unit"), "n_gpus": 1, "steps": args.steps,
@@ -359,7 +365,8 @@ def main():
 
     if args.config == 1 and not args.no_prefill:
         # the metric's prefill half: configuration 3 with the same procedure, its own roofline block
-        wl3, timing3, U3, counts3 = run_config(torch, 3, args.steps, args.warmup, args.windows, args.settle_ms)
+        wl3, timing3, U3, counts3 = run_config(torch, 3, args.steps, args.warmup, args.windows, args.settle_ms,
+                                               score_before_down=args.score_before_down)
         result["prefill_c3"] = describe(torch, wl3, 3, timing3, U3, counts3, args.steps, args.warmup, counters)
     if not args.no_gate:
         result["gate"] = time_gate(torch, args.steps, args.windows)
