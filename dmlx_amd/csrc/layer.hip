@@ -230,6 +230,8 @@ static int prefill_small_rows(const QView &b0, const QView &b1) {
     // measured: pays with the kernel of the packed 4-bit formats (8k-token ragged prefill: gate/up 1.757 -> 1.715 ms, down
     // unchanged), not with the 8-bit kernel (2080-token mixed batch: +1 %)
     if (!qgemm_wide_supports(b0) || !qgemm_wide_supports(b1)) return 0;
+    const auto four_bit = [](const QView &b) { return b.mode == DMOE_QUANT_MXFP4 || (b.mode == DMOE_QUANT_AFFINE && b.bits == 4); };
+    if (!four_bit(b0) || !four_bit(b1)) return 0;
     // threshold measured on the same prefill: 8 rows 2.62 ms, 16 rows 2.63, 32 rows 2.64, 4 rows 2.67, no split 2.70
     return std::min(kPrefillSmallRows, std::min(qgemm_skinny_tile_m(b0), qgemm_skinny_tile_m(b1)));
 }

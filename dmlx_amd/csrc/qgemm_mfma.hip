@@ -1,4 +1,6 @@
-// Grouped quantized GEMM, MFMA path (prefill): bf16 matrix-core tiles with in-register dequantization.
+// Grouped quantized GEMM, MFMA path (prefill) for weights in the MLX layout: bf16 matrix-core tiles with in-register
+// dequantization. (Stacks in the packed resident layout take the kernel in qgemm_wide.hip, which launch_qgemm_mfma
+// forwards to.)
 //
 // One workgroup (4 wavefronts) computes a tile of up to 128 rows of ONE expert segment against a strip
 // of output columns. The four wavefronts split the strip, so every packed weight chunk is read and
@@ -50,9 +52,7 @@ __device__ __forceinline__ void mfma_tile(const GemmArgs &g, const Tile &t, uint
     using G = MfmaGeom<Fmt>;
     constexpr int KV = G::KV, KSTEP = G::KSTEP, NJ = G::NJ, KB = G::KB, LDA = G::LDA, NI = G::NI;
     constexpr int NT = 2; // 32-column MFMA tiles per wavefront
-    // Weight steps held in registers. Tiles of at most 64 rows leave half of the accumulator registers free and are
-    // bound by the weight stream (a few dozen rows per expert against 8-bit weights): they keep four steps in flight.
-    constexpr int WR = (MT <= 2 && PACKED && kMfmaRing % 4 == 0) ? 4 : kMfmaWRing;
+    constexpr int WR = kMfmaWRing; // weight steps held in registers
     const int tid = (int)threadIdx.x, lane = tid & 63, ln = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int cols = g.b0.cols, n_out = g.b0.rows;
@@ -344,7 +344,6 @@ struct MfmaLaunch {
     }
     template <typename Fmt>
     int operator()() {
-        if (g.b0.packed) return g.gate_up ? go<Fmt, true, true>() : go<Fmt, false, true>();
         return g.gate_up ? go<Fmt, true, false>() : go<Fmt, false, false>();
     }
 };
@@ -352,8 +351,8 @@ struct MfmaLaunch {
 int launch_qgemm_mfma(const GemmArgs &g, hipStream_t st) {
     if (qgemm_wide_supports(g.b0)) return launch_qgemm_wide(g, st);
     DMOE_REQUIRE(g.tile_m > 0 && g.tile_m <= kMfmaTileM && g.tile_m % 32 == 0, "MFMA GEMM: bad tile size %d", g.tile_m);
-    DMOE_REQUIRE(qgemm_mfma_supports(g.b0), "MFMA GEMM: unsupported weight shape (rows=%d cols=%d)", g.b0.rows,
-                 g.b0.cols);
+    DMOE_REQUIRE(qgemm_mfma_supports(g.b0) && !g.b0.packed, "MFMA GEMM: unsupported weight shape (rows=%d cols=%d)",
+                 g.b0.rows, g.b0.cols);
     DMOE_REQUIRE(g.max_tiles >= 0 && g.max_tiles <= 65535, "MFMA GEMM: %d tiles exceed the grid limit", g.max_tiles);
     DMOE_REQUIRE(g.a && g.out && g.ldo > 0 && g.ldo % 4 == 0 && ((uintptr_t)g.out % 8) == 0 &&
                      ((uintptr_t)g.a % 16) == 0,

@@ -1,13 +1,14 @@
-// Grouped quantized GEMM, wide MFMA path (prefill, 4-bit formats in the packed resident layout).
+// Grouped quantized GEMM, wide MFMA path (prefill, every quantized format in the packed resident layout).
 //
 // One workgroup (4 wavefronts) = one tile of up to 128 rows of ONE expert segment against a strip of output columns;
 // each wavefront dequantizes its own 64 weight rows straight into the A operand of v_mfma_f32_32x32x16_bf16 and
 // holds 128 x 64 f32 accumulators. The kernel is built so that TWO workgroups fit a compute unit (at most 256
 // registers per wavefront, 64 KiB of LDS): a lone wavefront on a SIMD issues a vector instruction only every ~5
-// cycles, two wavefronts every ~2.8, and the 4-bit decode (2.9 vector instructions per weight) is what this kernel
-// is bound by. A variant with 256-row tiles (every decoded fragment feeds eight MFMAs instead of four, but one
+// cycles, two wavefronts every ~2.8, and the 4-bit decode (2.1 vector instructions per weight) is the largest
+// item beside the MFMAs. A variant with 256-row tiles (every decoded fragment feeds eight MFMAs instead of four, but one
 // wavefront per SIMD: all 512 registers, 128 KiB of LDS) measured 5 % slower on the 8k-token ragged prefill.
-// Differences from the 8-bit / MLX-layout kernel in qgemm_mfma.hip:
+// The 8-bit formats run the same loop with two 16-byte chunk steps per 64-element step. Differences from the
+// MLX-layout kernel in qgemm_mfma.hip:
 //
 //  * Activations go from global memory into LDS without passing through registers (global_load_lds_dwordx4).
 //    One such instruction moves 1 KiB: 8 rows x 128 bytes (one reduction step of 64 bf16). Inside that KiB the
@@ -52,14 +53,22 @@ constexpr int kWaitLgkm0 = 0xc07f;
 template <typename Fmt, bool GATE_UP, int MT>
 __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint8_t *lds, const int strip) {
     using CS = ChunkStream<Fmt, true>;
-    static_assert(Fmt::kVals == 32, "one reduction step must be 64 elements = one 128-byte activation granule");
-    constexpr int KV = 32, KSTEP = 64, NJ = 4, NT = 2;
-    constexpr int NU = NJ * MT * NT;  // units (MFMAs) per step
-    constexpr int NP = NT * (KV / 2); // packed pairs to decode per step
+    // A step is 64 reduction elements = one 128-byte activation granule. A lane's 16-byte weight chunk holds 32 (4-bit
+    // formats) or 16 (8-bit formats) of them: the weights come in chunk steps of 2 * KV elements, CH of them per step,
+    // and ring, decode and the double-buffered decoded operands advance by chunk steps.
+    constexpr int KV = Fmt::kVals, KSTEP = 64, NJ = 4, NT = 2;
+    constexpr int CH = 32 / KV;           // chunk steps per step
+    static_assert(CH == 1 || CH == 2, "chunks of 32 or 16 values");
+    constexpr int NJC = NJ / CH;          // MFMA groups per chunk step
+    constexpr int NUC = NJC * MT * NT;    // units (MFMAs) per chunk step
+    constexpr int NPC = NT * (KV / 2);    // packed pairs to decode per chunk step
+    // chunk steps held in registers (twice as many for tiles of at most 64 rows moved the 8-bit mixed batch by nothing)
+    constexpr int WRC = kWideWRing * CH;
+    static_assert(kWideRing % kWideWRing == 0, "ring slots must line up across trips");
     const int tid = (int)threadIdx.x, lane = tid & 63, ln = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int cols = g.b0.cols, n_out = g.b0.rows;
-    const int n_steps = cols / KSTEP;
+    const int n_steps = cols / KSTEP, n_csteps = n_steps * CH;
     const int n_trips = (n_steps + kWideRing - 1) / kWideRing;
     const size_t e = t.expert;
 
@@ -76,18 +85,18 @@ __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint
         if (n >= n_out) n = n_out - 1;
         cs[nt].init(b, e, (on ? base : 0) >> 5, ln, h, n); // a switched-off tile aliases valid memory, never stored
     }
-    uint4 ring_raw[kWideWRing][NT];
-    uint32_t ring_sb[kWideWRing][NT][2];
-    auto load_b = [&](int step, int slot_) {
+    uint4 ring_raw[WRC][NT];
+    uint32_t ring_sb[WRC][NT][2];
+    auto load_b = [&](int cstep, int slot_) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             const QView &b = (GATE_UP && nt == 1) ? g.b1 : g.b0;
-            ring_raw[slot_][nt] = cs[nt].load_chunk(step);
-            cs[nt].load_meta(b, step, ring_sb[slot_][nt]);
+            ring_raw[slot_][nt] = cs[nt].load_chunk(cstep);
+            cs[nt].load_meta(b, cstep, ring_sb[slot_][nt]);
         }
     };
 #pragma unroll
-    for (int j = 0; j < kWideWRing; ++j) load_b(j < n_steps ? j : n_steps - 1, j);
+    for (int j = 0; j < WRC; ++j) load_b(j < n_csteps ? j : n_csteps - 1, j);
 
     // ---- activation staging -------------------------------------------------------------------------------
     // operation i of this wavefront moves rows (wave + 4 i) * 8 .. + 7; lane = (row r8 of the eight, position c),
@@ -133,10 +142,15 @@ __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint
     // only safe because those tiles also wait for their own LDS reads before each barrier (see below).
     constexpr int AHEAD = MT <= 2 ? 3 : 2;
     bf16x8_t xf[XB][MT];
-    // fragment (mt, j) of a step: row mt * 32 + ln, piece h * 4 + j, stored at piece ^ ((row >> 1) & 7)
+    // fragment (mt, j) of a step: row mt * 32 + ln, the piece that holds this lane's eight reduction elements of MFMA
+    // group j (chunk step c = j / NJC of the step, elements (2 c + h) * KV + 8 (j % NJC) onwards), stored at
+    // piece ^ ((row >> 1) & 7)
     const uint8_t *x_rd[NJ];
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) x_rd[j] = lds + (ln >> 3) * 1024 + (ln & 7) * 128 + (((h * 4 + j) ^ ((ln >> 1) & 7)) * 16);
+    for (int j = 0; j < NJ; ++j) {
+        const int piece = ((2 * (j / NJC) + h) * KV + 8 * (j % NJC)) >> 3;
+        x_rd[j] = lds + (ln >> 3) * 1024 + (ln & 7) * 128 + ((piece ^ ((ln >> 1) & 7)) * 16);
+    }
     auto read_x = [&](int buf, int j, int mt) {
         uint4 q = *(const uint4 *)(x_rd[j] + buf * kWideBufBytes + mt * 4096);
         xf[j % XB][mt] = __builtin_bit_cast(bf16x8_t, q);
@@ -171,61 +185,71 @@ __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint
 #pragma unroll
         for (int j = 0; j < kWideRing; ++j) {
             const int s = s0 + j;
-            const int s_ahead = s + kWideWRing < n_steps ? s + kWideWRing : n_steps - 1;
-            load_b(s_ahead, j % kWideWRing); // this slot was decoded one step ago
-            const int slot_next = (j + 1) % kWideWRing, which = j & 1, buf_next = (j + 1) % kWideRing;
+            const int buf_next = (j + 1) % kWideRing;
             const bool stage = s + AHEAD < n_steps; // uniform
-            Meta meta_next[NT];
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) meta_next[nt] = Fmt::pair_meta(CS::meta(ring_sb[slot_next][nt]));
-            uint32_t dstate[Fmt::kPairState] = {};
-            Fmt::pair_state(dstate);
+            for (int c = 0; c < CH; ++c) {
+                const int ci = j * CH + c; // chunk step within the trip
+                const int cs_ahead = s * CH + c + WRC < n_csteps ? s * CH + c + WRC : n_csteps - 1;
+                load_b(cs_ahead, ci % WRC); // this slot was decoded one chunk step ago
+                const int slot_next = (ci + 1) % WRC, which = ci & 1;
+                Meta meta_next[NT];
 #pragma unroll
-            for (int jj = 0; jj < NJ; ++jj) {
-                if (jj == NJ - 1) {
-                    // block s + 1 must have landed; the AHEAD - 1 younger requests of MT operations each may still
-                    // fly (fewer near the end of the reduction, when nothing is requested any more)
-                    if (AHEAD == 2) {
-                        if (stage) __builtin_amdgcn_s_waitcnt(wait_vmcnt(MT));
-                        else __builtin_amdgcn_s_waitcnt(wait_vmcnt(0));
-                    } else {
-                        // also drain this wavefront's LDS reads: the next step's requests overwrite the buffer
-                        // that the reads issued during the previous MFMA group came from
-                        if (stage) __builtin_amdgcn_s_waitcnt(wait_vmcnt_lgkm0(2 * MT));
-                        else if (s + AHEAD - 1 < n_steps) __builtin_amdgcn_s_waitcnt(wait_vmcnt_lgkm0(MT));
-                        else __builtin_amdgcn_s_waitcnt(wait_vmcnt_lgkm0(0));
-                    }
-                    asm volatile("" ::: "memory");
-                    __builtin_amdgcn_s_barrier();
-                    asm volatile("" ::: "memory");
-                    __builtin_amdgcn_sched_barrier(0);
-                }
+                for (int nt = 0; nt < NT; ++nt) meta_next[nt] = Fmt::pair_meta(CS::meta(ring_sb[slot_next][nt]));
+                uint32_t dstate[Fmt::kPairState] = {};
+                Fmt::pair_state(dstate);
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) {
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) {
-                        const int u = (jj * MT + mt) * NT + nt;
-                        uint4 q = make_uint4(wp[which][nt][4 * jj], wp[which][nt][4 * jj + 1], wp[which][nt][4 * jj + 2],
-                                             wp[which][nt][4 * jj + 3]);
-                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, q),
-                                                                              xf[jj % XB][mt], acc[mt][nt], 0, 0, 0);
-                        // fetch the fragment of the next group: after the last use of this one (one register set),
-                        // or at the first (two sets)
-                        if (nt == (XB == 1 ? NT - 1 : 0)) {
-                            if (jj + 1 < NJ) read_x(j, jj + 1, mt);
-                            else read_x(buf_next, 0, mt);
+                for (int jc = 0; jc < NJC; ++jc) {
+                    const int jj = c * NJC + jc; // MFMA group within the step
+                    if (jj == NJ - 1) {
+                        // block s + 1 must have landed; the AHEAD - 1 younger requests of MT operations each may still
+                        // fly (fewer near the end of the reduction, when nothing is requested any more), and so may
+                        // the weight chunks that the later chunk steps of this step have requested since (LATE, at
+                        // least one load per weight tile each)
+                        constexpr int LATE = (CH - 1) * NT;
+                        if (AHEAD == 2) {
+                            if (stage) __builtin_amdgcn_s_waitcnt(wait_vmcnt(MT + LATE));
+                            else __builtin_amdgcn_s_waitcnt(wait_vmcnt(LATE));
+                        } else {
+                            // also drain this wavefront's LDS reads: the next step's requests overwrite the buffer
+                            // that the reads issued during the previous MFMA group came from
+                            if (stage) __builtin_amdgcn_s_waitcnt(wait_vmcnt_lgkm0(2 * MT + LATE));
+                            else if (s + AHEAD - 1 < n_steps) __builtin_amdgcn_s_waitcnt(wait_vmcnt_lgkm0(MT + LATE));
+                            else __builtin_amdgcn_s_waitcnt(wait_vmcnt_lgkm0(LATE));
                         }
-                        if (u % 6 == 0 && u / 6 < MT) { // the staging requests all fall into the first three groups
-                            if (stage) stage_op(s + AHEAD, (j + AHEAD) % kWideRing, u / 6);
-                        }
-#pragma unroll
-                        for (int p = u * NP / NU; p < (u + 1) * NP / NU; ++p) {
-                            Fmt::decode_pair(ring_raw[slot_next][p / (KV / 2)], meta_next[p / (KV / 2)], p % (KV / 2),
-                                             wp[which ^ 1][p / (KV / 2)], dstate);
-                            // pin the slice here (the optimiser would sink a trip's last decode into the next trip)
-                            asm volatile("" : "+v"(wp[which ^ 1][p / (KV / 2)][p % (KV / 2)]));
-                        }
+                        asm volatile("" ::: "memory");
+                        __builtin_amdgcn_s_barrier();
+                        asm volatile("" ::: "memory");
                         __builtin_amdgcn_sched_barrier(0);
+                    }
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt) {
+                            const int uc = (jc * MT + mt) * NT + nt; // unit within the chunk step
+                            const int u = c * NUC + uc;              // unit within the step
+                            uint4 q = make_uint4(wp[which][nt][4 * jc], wp[which][nt][4 * jc + 1], wp[which][nt][4 * jc + 2],
+                                                 wp[which][nt][4 * jc + 3]);
+                            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, q),
+                                                                                  xf[jj % XB][mt], acc[mt][nt], 0, 0, 0);
+                            // fetch the fragment of the next group: after the last use of this one (one register set),
+                            // or at the first (two sets)
+                            if (nt == (XB == 1 ? NT - 1 : 0)) {
+                                if (jj + 1 < NJ) read_x(j, jj + 1, mt);
+                                else read_x(buf_next, 0, mt);
+                            }
+                            if (u % 6 == 0 && u / 6 < MT) { // the staging requests all fall into the first three groups
+                                if (stage) stage_op(s + AHEAD, (j + AHEAD) % kWideRing, u / 6);
+                            }
+#pragma unroll
+                            for (int p = uc * NPC / NUC; p < (uc + 1) * NPC / NUC; ++p) {
+                                Fmt::decode_pair(ring_raw[slot_next][p / (KV / 2)], meta_next[p / (KV / 2)], p % (KV / 2),
+                                                 wp[which ^ 1][p / (KV / 2)], dstate);
+                                // pin the slice here (the optimiser would sink a trip's last decode into the next trip)
+                                asm volatile("" : "+v"(wp[which ^ 1][p / (KV / 2)][p % (KV / 2)]));
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
                     }
                 }
             }
@@ -254,13 +278,23 @@ __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint
         float rscale = 1.0f;
         if (g.row_scale) rscale = g.row_scale[g.row_scale_idx ? g.row_scale_idx[p] : p];
         uint8_t *wrow = mine + ln * PITCH;
+        // per-row weight scales (FP8): output column n of register 4 rg + i is col_base (+ 32 nt) + 8 rg + 4 h + i
+        auto wscale = [&](const QView &b, int n) {
+            return *(const float *)(b.scales + e * b.s_mat + (size_t)(n < n_out ? n : n_out - 1) * b.s_row);
+        };
         if (GATE_UP) {
 #pragma unroll
             for (int rg = 0; rg < 4; ++rg) {
                 float v[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    v[i] = limited_swiglu(acc[mt][0][4 * rg + i], acc[mt][1][4 * rg + i], g.swiglu_limit) * rscale;
+                for (int i = 0; i < 4; ++i) {
+                    float gv = acc[mt][0][4 * rg + i], uv = acc[mt][1][4 * rg + i];
+                    if (Fmt::kRowScale) {
+                        gv *= wscale(g.b0, col_base + 8 * rg + 4 * h + i);
+                        uv *= wscale(g.b1, col_base + 8 * rg + 4 * h + i);
+                    }
+                    v[i] = limited_swiglu(gv, uv, g.swiglu_limit) * rscale;
+                }
                 *(uint2 *)(wrow + (8 * rg + 4 * h) * 2) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
             }
         } else {
@@ -270,7 +304,11 @@ __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint
                 for (int rg = 0; rg < 4; ++rg) {
                     float v[4];
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) v[i] = acc[mt][nt][4 * rg + i] * rscale;
+                    for (int i = 0; i < 4; ++i) {
+                        v[i] = acc[mt][nt][4 * rg + i];
+                        if (Fmt::kRowScale) v[i] *= wscale(g.b0, col_base + 32 * nt + 8 * rg + 4 * h + i);
+                        v[i] *= rscale;
+                    }
                     *(uint2 *)(wrow + (32 * nt + 8 * rg + 4 * h) * 2) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
                 }
             }
@@ -327,8 +365,7 @@ __global__ __launch_bounds__(kWideWaves * 64, 2) void qgemm_wide_kernel(GemmArgs
 }
 
 bool qgemm_wide_supports(const QView &b) {
-    const bool four_bit = (b.mode == DMOE_QUANT_AFFINE && b.bits == 4) || b.mode == DMOE_QUANT_MXFP4;
-    return four_bit && b.packed && b.cols % 64 == 0 && b.rows % 4 == 0;
+    return b.mode != DMOE_QUANT_NONE && b.packed && b.cols % 64 == 0 && b.rows % 4 == 0;
 }
 
 template <typename Fmt, bool GATE_UP>
@@ -362,6 +399,10 @@ int launch_qgemm_wide(const GemmArgs &g, hipStream_t st) {
     if (g.max_tiles == 0) return DMOE_OK;
     if (g.b0.mode == DMOE_QUANT_MXFP4)
         return g.gate_up ? launch_wide<FmtMxfp4, true>(g, st) : launch_wide<FmtMxfp4, false>(g, st);
+    if (g.b0.mode == DMOE_QUANT_FP8_ROW)
+        return g.gate_up ? launch_wide<FmtFp8Row, true>(g, st) : launch_wide<FmtFp8Row, false>(g, st);
+    if (g.b0.bits == 8)
+        return g.gate_up ? launch_wide<FmtAffine8, true>(g, st) : launch_wide<FmtAffine8, false>(g, st);
     return g.gate_up ? launch_wide<FmtAffine4, true>(g, st) : launch_wide<FmtAffine4, false>(g, st);
 }
 
