@@ -277,7 +277,7 @@ def describe(torch, wl, config, timing, U, counts, steps, warmup, counters):
     if rec:
         roof["counters_from"] = rec.get("source")
     launches = (["qgemm_skinny_kernel (gate/up and down tiles in one launch)"] if paired else ["qgemm_skinny_kernel"] if decode else
-                ["qgemm_wide_kernel"] if split else ["qgemm_mfma_kernel"])
+                ["qgemm_wide_kernel"])  # the benchmark's layers hold their weights in the packed resident layout
     if split:
         roof["rows_in_launch"] = k_rows
         roof["small_tile_launch_ms"] = stages[kern + "_small"]
