@@ -11,7 +11,7 @@ GEMM + limited SwiGLU -> grouped down GEMM -> weighted combine + shared expert, 
 --config selects the benchmark configuration (0..4, as listed in BASELINE.json); default 1: the 64-sequence decode
 step the headline metric is quoted on. The metric's other half - the fraction of the bf16 MFMA peak at the 8k-token
 ragged prefill, configuration 3 - is measured in the same run with the same procedure and reported under the key
-`prefill_c3` (switch off with --no-prefill).
+`prefill_c3`, and so are configurations 2 (`decode_c2`) and 4 (`mixed_c4`) (switch all three off with --no-prefill).
 
 Timing procedure, per configuration: a pre-run of at least --settle-ms of steps brings clocks and memory to their
 loaded state (reported as `settle`, separate from `warmup`); then W untimed warm-up steps; then --windows windows of
@@ -53,7 +53,7 @@ def cpu_baseline(wl, max_tokens, min_seconds=10.0, max_runs=5):
     """Time the oracle (route + MoE forward) on the first `max_tokens` tokens of the workload."""
     import numpy as np
     from oracle import oracle
-    from tests.helpers import bf16_bits, qmat
+    from oracle.oracle import bf16_bits, qmat
 
     n = min(wl.T, max_tokens)
     scores = wl.scores[:n].cpu().numpy()
@@ -260,15 +260,17 @@ def describe(torch, wl, config, timing, U, counts, steps, warmup, counters):
     by_bound = {"hbm": {"bound": "hbm", "achieved": hbm, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": hbm / HBM_PEAK_GBS},
                 "mfma": {"bound": "mfma", "achieved": mfma, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": mfma / MFMA_BF16_PEAK_TFLOPS}}
-    # decode is bound by HBM and the 4-bit prefill by the matrix core; the mixed batch (configuration 4, 8-bit weights,
-    # 2080 tokens) sits between the two: both are reported, the one with the larger fraction as the bound
-    if config == 4:
-        first = "hbm" if by_bound["hbm"]["frac"] >= by_bound["mfma"]["frac"] else "mfma"
-    else:
-        first = "hbm" if decode else "mfma"
+    # Which roofline bounds the launch follows from its arithmetic intensity against the machine balance (published
+    # peaks: 2500 TFLOP/s / 8000 GB/s = 312.5 flop per byte), both taken from the ALGORITHMIC flops and bytes: decode
+    # launches sit far below it (HBM), the 4-bit prefill far above (matrix core), the mixed batch of configuration 4
+    # (8-bit weights, 2080 tokens) below it at 130 flop per byte. The fraction of the other peak is reported as well.
+    intensity = k_flops / k_bytes
+    ridge = MFMA_BF16_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
+    first = "hbm" if intensity < ridge else "mfma"
     roof = dict(by_bound[first])
-    if config == 4:
-        roof["other_bound"] = by_bound["mfma" if first == "hbm" else "hbm"]
+    roof["other_bound"] = by_bound["mfma" if first == "hbm" else "hbm"]
+    roof["flop_per_byte"] = intensity
+    roof["fractions_use"] = "algorithmic bytes and flops of the launch (not the counted traffic)"
     rec = counters.get(f"c{config}", {}).get(kern, {})
     roof["traffic"] = rec.get("traffic_bytes")
     if "mfma_busy" in rec:
@@ -321,7 +323,7 @@ def main():
     ap.add_argument("--score-before-down", type=int, default=0, choices=[0, 1],
                     help="1: routing weight applied to the activation before the down projection (DSV4SwitchGLU.forward); "
                          "0: to the expert outputs (expert provider paths)")
-    ap.add_argument("--no-prefill", action="store_true", help="with --config 1: do not also time configuration 3")
+    ap.add_argument("--no-prefill", action="store_true", help="with --config 1: do not also time configurations 3, 2 and 4")
     ap.add_argument("--no-gate", action="store_true", help="do not also time the router (DSV4Gate.forward) in front of the step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-peaks", action="store_true", help="skip the library copy / GEMM reference measurements")
@@ -364,10 +366,15 @@ def main():
     torch.cuda.empty_cache()
 
     if args.config == 1 and not args.no_prefill:
-        # the metric's prefill half: configuration 3 with the same procedure, its own roofline block
-        wl3, timing3, U3, counts3 = run_config(torch, 3, args.steps, args.warmup, args.windows, args.settle_ms,
-                                               score_before_down=args.score_before_down)
-        result["prefill_c3"] = describe(torch, wl3, 3, timing3, U3, counts3, args.steps, args.warmup, counters)
+        # the metric's prefill half (configuration 3) and the two remaining configurations (2: MXFP4 decode with 51
+        # resident experts; 4: mixed batch, 8-bit routed + FP8 shared expert), each with the same procedure and its
+        # own roofline block
+        for key, cfg in (("prefill_c3", 3), ("decode_c2", 2), ("mixed_c4", 4)):
+            wl_n, timing_n, U_n, counts_n = run_config(torch, cfg, args.steps, args.warmup, args.windows, args.settle_ms,
+                                                       score_before_down=args.score_before_down)
+            result[key] = describe(torch, wl_n, cfg, timing_n, U_n, counts_n, args.steps, args.warmup, counters)
+            del wl_n
+            torch.cuda.empty_cache()
     if not args.no_gate:
         result["gate"] = time_gate(torch, args.steps, args.windows)
     print(json.dumps(result))

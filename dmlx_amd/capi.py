@@ -64,6 +64,7 @@ EXPORTS = [
     "dmoe_malloc", "dmoe_free", "dmoe_copy_to_device", "dmoe_copy_to_host",
     "dmoe_workspace_create", "dmoe_workspace_destroy", "dmoe_workspace_reserved",
     "dmoe_workspace_check", "dmoe_workspace_set_wait_limit", "dmoe_workspace_set_paired_launch", "dmoe_workspace_set_weight_cache",
+    "dmoe_workspace_weight_cache_invalidate", "dmoe_workspace_set_weight_cache_limit", "dmoe_workspace_weight_cache_stats",
     "dmoe_workspace_set_stage_timing", "dmoe_workspace_read_stage_times",
     "dmoe_topk_route", "dmoe_gate_route", "dmoe_remap_indices", "dmoe_expand_tokens",
     "dmoe_reduce_experts", "dmoe_smelt_build_mask", "dmoe_build_remap", "dmoe_preload_remap",
@@ -71,7 +72,7 @@ EXPORTS = [
     "dmoe_resident_weight_create", "dmoe_resident_weight_destroy", "dmoe_gather_qmm_resident",
     "dmoe_layer_create", "dmoe_layer_destroy", "dmoe_moe_forward",
     "dmoe_switch_glu_forward_no_scores", "dmoe_moe_layer_forward", "dmoe_moe_layer_forward_static",
-    "dmoe_debug_last_activations",
+    "dmoe_debug_last_activations", "dmoe_debug_dequantize_fused",
     "dmoe_gate_create", "dmoe_gate_destroy", "dmoe_gate_forward",
     "dmoe_layer_create_from_safetensors", "dmoe_layer_dims", "dmoe_batch_build", "dmoe_block_post",
 ]
@@ -131,6 +132,22 @@ class Workspace:
     def set_weight_cache(self, enabled):
         """gather_qmm keeps re-ordered resident copies of the stacks it sees (dmoe_workspace_set_weight_cache)"""
         check(lib().dmoe_workspace_set_weight_cache(self.h, int(enabled)))
+
+    def invalidate_weight_cache(self, qw=None):
+        """drop the cached copy of one stack (a QWeight), or every copy"""
+        if qw is None:
+            check(lib().dmoe_workspace_weight_cache_invalidate(self.h, None))
+        else:
+            c = qw.c()
+            check(lib().dmoe_workspace_weight_cache_invalidate(self.h, C.byref(c)))
+
+    def set_weight_cache_limit(self, max_bytes):
+        check(lib().dmoe_workspace_set_weight_cache_limit(self.h, C.c_size_t(max_bytes)))
+
+    def weight_cache_stats(self):
+        b, n = C.c_size_t(0), C.c_int(0)
+        check(lib().dmoe_workspace_weight_cache_stats(C.byref(b), C.byref(n), self.h))
+        return b.value, n.value
 
     def set_paired_launch(self, enabled):
         check(lib().dmoe_workspace_set_paired_launch(self.h, int(enabled)))
@@ -266,10 +283,12 @@ def pack(idx, E, ws):
     return out
 
 
-def dequantize(qw, mat_index=0):
+def dequantize(qw, mat_index=0, fused=False):
+    """dmoe_dequantize; fused=True: the same matrix through the prefill kernels' in-register decoder."""
     out = torch.empty((qw.rows, qw.cols), dtype=torch.bfloat16, device=qw.w.device)
     c = qw.c()
-    check(lib().dmoe_dequantize(_ptr(out), C.byref(c), mat_index, _stream()))
+    fn = lib().dmoe_debug_dequantize_fused if fused else lib().dmoe_dequantize
+    check(fn(_ptr(out), C.byref(c), mat_index, _stream()))
     return out
 
 

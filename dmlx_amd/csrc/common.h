@@ -71,6 +71,7 @@ struct Workspace {
     // layer.hip (weight_cache_find_or_add / weight_cache_clear).
     bool cache_weights = false;
     void *weight_cache = nullptr;
+    size_t cache_limit_bytes = (size_t)32 << 30; // copies beyond this many bytes push out the least recently used ones
     // gate/up and down of a decode step share one launch (down workgroups wait per tile for gate/up). Switched off by
     // dmoe_workspace_set_paired_launch, and by dmoe_workspace_check once a wait gave up: the two GEMMs then run as two
     // launches in a row, which wait for nothing.
@@ -90,6 +91,8 @@ int stage_flush(Workspace *w);
 int workspace_reserve(dmoe_workspace ws, size_t bytes, Workspace **out);
 // drops every cached resident copy of the workspace (layer.hip)
 void weight_cache_clear(Workspace *w);
+int weight_cache_invalidate(Workspace *w, const dmoe_qweight *qw);  // one stack's copy, or every copy (qw == null)
+int weight_cache_stats(Workspace *w, size_t *out_bytes, int *out_stacks);
 // the current device's workspace over the static device scratch (layer.hip); resolves its address on first use
 int static_workspace(Workspace **out);
 
@@ -108,6 +111,20 @@ inline T *at(Workspace *w, size_t off) {
 }
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// Dynamic-LDS limit of a kernel above 64 KiB: hipFuncSetAttribute belongs to (function, device), so every kernel
+// instantiation keeps one of these and raises its limit once per device. dmoe_init raises all of them for its device
+// (prepare_kernels), so that no launch made later - possibly under stream capture, possibly from another thread - has
+// host-side set-up left to do.
+constexpr int kMaxDevices = 64;
+struct LdsLimit {
+    unsigned long long raised = 0; // bit d: done on device d (read and written under lds_limit_mutex)
+};
+int raise_lds_limit(LdsLimit &state, const void *kernel, int bytes);
+// raise the limits of every kernel instantiation of the GEMM files on the current device
+int qgemm_wide_prepare();
+int qgemm_mfma_prepare();
+int qgemm_skinny_prepare();
 
 // ---- tile list produced by the pack kernels ----------------------------------------------------------
 // one entry per (expert segment, row tile): rows [row0, row0 + nrows) of the sorted row order

@@ -97,15 +97,48 @@ __global__ void dequant_kernel(uint16_t *__restrict__ out, QView q, int mat) {
     for (int p = 0; p < Fmt::kVals / 2; ++p) o[p] = pairs[p];
 }
 
+// The same matrix through the decoder that the matrix-core kernels run in registers (pair_meta / decode_pair), for
+// tests that compare it bit for bit with decode().
+template <typename Fmt>
+__global__ void dequant_fused_kernel(uint16_t *__restrict__ out, QView q, int mat) {
+    const int chunks_per_row = q.cols / Fmt::kVals;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)q.rows * chunks_per_row) return;
+    int row = (int)(i / chunks_per_row), c = (int)(i - (size_t)row * chunks_per_row);
+    int k0 = c * Fmt::kVals;
+    const uint8_t *wrow = q.w + (size_t)mat * q.w_mat + (size_t)row * q.w_row;
+    const uint8_t *srow = q.scales + (size_t)mat * q.s_mat + (size_t)row * q.s_row;
+    const uint8_t *brow = q.biases ? q.biases + (size_t)mat * q.s_mat + (size_t)row * q.s_row : nullptr;
+    uint4 raw = *(const uint4 *)(wrow + (size_t)c * 16);
+    const Meta m = Fmt::pair_meta(Fmt::load_meta(q, srow, brow, k0));
+    uint32_t pairs[Fmt::kVals / 2], st[Fmt::kPairState] = {};
+    Fmt::pair_state(st);
+#pragma unroll
+    for (int p = 0; p < Fmt::kVals / 2; ++p) Fmt::decode_pair(raw, m, p, pairs, st);
+    if (Fmt::kRowScale) {
+        float rs = *(const float *)srow;
+#pragma unroll
+        for (int p = 0; p < Fmt::kVals / 2; ++p)
+            pairs[p] = pack_bf16x2(bf16_bits_to_f32(pairs[p] & 0xffffu) * rs, bf16_bits_to_f32(pairs[p] >> 16) * rs);
+    }
+    uint32_t *o = (uint32_t *)(out + (size_t)row * q.cols + k0);
+#pragma unroll
+    for (int p = 0; p < Fmt::kVals / 2; ++p) o[p] = pairs[p];
+}
+
 struct DequantLaunch {
     uint16_t *out;
     QView q;
     int mat;
     hipStream_t st;
+    bool fused = false;
     template <typename Fmt>
     int operator()() {
         size_t total = (size_t)q.rows * (q.cols / Fmt::kVals);
-        hipLaunchKernelGGL(dequant_kernel<Fmt>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, out, q, mat);
+        if (fused)
+            hipLaunchKernelGGL(dequant_fused_kernel<Fmt>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, out, q, mat);
+        else
+            hipLaunchKernelGGL(dequant_kernel<Fmt>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, out, q, mat);
         DMOE_LAUNCH_CHECK();
         return DMOE_OK;
     }
@@ -115,7 +148,7 @@ struct DequantLaunch {
 
 using namespace dmoe;
 
-extern "C" int dmoe_dequantize(uint16_t *d_out, const dmoe_qweight *qw, int mat_index, dmoe_stream s) {
+static int dequantize_common(uint16_t *d_out, const dmoe_qweight *qw, int mat_index, bool fused, dmoe_stream s) {
     QView q;
     DMOE_TRY(make_qview(&q, qw, "dequantize"));
     DMOE_REQUIRE(d_out != nullptr, "dequantize: out is null");
@@ -126,5 +159,13 @@ extern "C" int dmoe_dequantize(uint16_t *d_out, const dmoe_qweight *qw, int mat_
         return DMOE_OK;
     }
     DMOE_REQUIRE(q.cols % 32 == 0, "dequantize: cols %d not a multiple of 32", q.cols);
-    return dispatch_format(q, DequantLaunch{d_out, q, mat_index, to_hip(s)});
+    return dispatch_format(q, DequantLaunch{d_out, q, mat_index, to_hip(s), fused});
+}
+
+extern "C" int dmoe_dequantize(uint16_t *d_out, const dmoe_qweight *qw, int mat_index, dmoe_stream s) {
+    return dequantize_common(d_out, qw, mat_index, false, s);
+}
+
+extern "C" int dmoe_debug_dequantize_fused(uint16_t *d_out, const dmoe_qweight *qw, int mat_index, dmoe_stream s) {
+    return dequantize_common(d_out, qw, mat_index, true, s);
 }

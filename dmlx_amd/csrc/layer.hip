@@ -394,23 +394,40 @@ static int shared_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
 struct CachedStack {
     dmoe_qweight key; // the caller's stack as passed (pointers, shape, format)
     QOwned owned;     // its re-ordered copy
+    size_t bytes = 0; // device bytes held by the copy
+    uint64_t last_use = 0;
 };
 struct WeightCache {
     std::vector<CachedStack *> items;
+    size_t bytes = 0;
+    uint64_t clock = 0;
 };
 static bool same_stack(const dmoe_qweight &a, const dmoe_qweight &b) {
     return a.w == b.w && a.scales == b.scales && a.biases == b.biases && a.n_mats == b.n_mats && a.rows == b.rows &&
            a.cols == b.cols && a.mode == b.mode && a.bits == b.bits && a.group_size == b.group_size;
 }
+static void drop_item(WeightCache *c, size_t i) {
+    CachedStack *it = c->items[i];
+    c->bytes -= it->bytes;
+    free_owned(it->owned);
+    delete it;
+    c->items.erase(c->items.begin() + (long)i);
+}
 void weight_cache_clear(Workspace *w) {
     WeightCache *c = (WeightCache *)w->weight_cache;
     if (!c) return;
-    for (CachedStack *it : c->items) {
-        free_owned(it->owned);
-        delete it;
-    }
+    while (!c->items.empty()) drop_item(c, c->items.size() - 1);
     delete c;
     w->weight_cache = nullptr;
+}
+// drops the copy of `qw` (null: every copy); kernels in flight may still read a copy, so the device is waited for
+int weight_cache_invalidate(Workspace *w, const dmoe_qweight *qw) {
+    WeightCache *c = (WeightCache *)w->weight_cache;
+    if (!c || c->items.empty()) return DMOE_OK;
+    DMOE_HIP(hipDeviceSynchronize());
+    for (size_t i = c->items.size(); i-- > 0;)
+        if (!qw || same_stack(c->items[i]->key, *qw)) drop_item(c, i);
+    return DMOE_OK;
 }
 // the cached resident view of `qw`, made on first sight (one re-ordering pass, waits for it)
 static int weight_cache_find_or_add(Workspace *w, const dmoe_qweight *qw, const QView **out, hipStream_t st) {
@@ -419,6 +436,7 @@ static int weight_cache_find_or_add(Workspace *w, const dmoe_qweight *qw, const 
     DMOE_REQUIRE(c != nullptr, "gather_qmm: out of host memory");
     for (CachedStack *it : c->items)
         if (same_stack(it->key, *qw)) {
+            it->last_use = ++c->clock;
             *out = &it->owned.view;
             return DMOE_OK;
         }
@@ -431,8 +449,32 @@ static int weight_cache_find_or_add(Workspace *w, const dmoe_qweight *qw, const 
         delete it;
         return rc;
     }
+    it->bytes = it->owned.view.packed ? packed_w_bytes(it->owned.view) + packed_meta_bytes(it->owned.view) : 0;
+    // over the byte limit: the least recently used copies go first (never the new one). Their kernels may still run.
+    if (w->cache_limit_bytes && c->bytes + it->bytes > w->cache_limit_bytes && !c->items.empty()) {
+        hipError_t e = hipDeviceSynchronize();
+        if (e != hipSuccess) {
+            free_owned(it->owned);
+            delete it;
+            return hip_fail(e, "hipDeviceSynchronize");
+        }
+        while (!c->items.empty() && c->bytes + it->bytes > w->cache_limit_bytes) {
+            size_t oldest = 0;
+            for (size_t i = 1; i < c->items.size(); ++i)
+                if (c->items[i]->last_use < c->items[oldest]->last_use) oldest = i;
+            drop_item(c, oldest);
+        }
+    }
+    it->last_use = ++c->clock;
+    c->bytes += it->bytes;
     c->items.push_back(it);
     *out = &it->owned.view;
+    return DMOE_OK;
+}
+int weight_cache_stats(Workspace *w, size_t *out_bytes, int *out_stacks) {
+    WeightCache *c = (WeightCache *)w->weight_cache;
+    if (out_bytes) *out_bytes = c ? c->bytes : 0;
+    if (out_stacks) *out_stacks = c ? (int)c->items.size() : 0;
     return DMOE_OK;
 }
 

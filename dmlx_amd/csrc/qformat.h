@@ -119,42 +119,34 @@ struct FmtAffine4 {
     }
     __device__ static __forceinline__ void decode_fast(const uint4 &raw, Meta m, uint32_t *out) { decode(raw, m, out); }
     // Values (2q, 2q+1) of the chunk only, for callers that spread the decode between other instructions; q must
-    // run upwards through a chunk. `m` must come from pair_meta() and `st` from pair_state(): code c becomes the f16
-    // number 1024 + c by OR-ing it into 0x6400, v_fma_mix_f32 takes that half-word straight into an f32 fma, and
-    // (1024 + c) * s + (b - 1024 s) is c * s + b rounded once, as decode() computes it. A code that sits four bits up
-    // in its half-word needs no shift either: OR-ed in place it reads 1024 + 16 c, and (1024 + 16 c) * (s / 16) +
-    // (b - 64 s) is the same value (s / 16 is exact, and so are both offsets for bf16 s and b). Per word of 8 codes:
-    // one shift, four masked pairs (codes i and i + 4 share a register; the magic is held in a register because
-    // v_and_or_b32 takes one literal), 8 fmas, 4 packs = 17 instructions, against 23 with byte planes and
-    // v_cvt_f32_ubyteN.
-    static constexpr int kPairState = 7;
+    // run upwards through a chunk. `m` must come from pair_meta() and `st` from pair_state(). A 4-bit code c masked
+    // out in place IS an f16 number: the bit pattern c is the subnormal c * 2^-24, and a code that sits four bits up
+    // in its half-word (pattern 16 c) is 16 c * 2^-24. v_fma_mix_f32 widens that half-word exactly inside an f32 fma,
+    // so (c * 2^-24) * (s * 2^24) + b, respectively (16 c * 2^-24) * (s * 2^20) + b, is c * s + b rounded ONCE: bit for
+    // bit what decode() computes with fmaf((float)c, s, b), for every bf16 scale and bias (the scaled s is exact up to
+    // |s| < 2^103). Per word of 8 codes: one shift, four masks (codes i and i + 4 share a register), 8 fmas, 4 packs
+    // = 17 instructions, against 23 with byte planes and v_cvt_f32_ubyteN.
+    static constexpr int kPairState = 6;
     __device__ static __forceinline__ Meta pair_meta(Meta m) {
-        m.b = fmaf(-1024.0f, m.s, m.b);
+        m.s *= 16777216.0f; // s * 2^24, exact
         return m;
     }
-    __device__ static __forceinline__ void pair_state(uint32_t *st) {
-        uint32_t magic = 0x64006400u;
-        asm volatile("" : "+v"(magic)); // opaque, so that it stays a register operand of v_and_or_b32
-        st[4] = magic;
-    }
+    __device__ static __forceinline__ void pair_state(uint32_t *) {}
     __device__ static __forceinline__ void decode_pair(const uint4 &raw, Meta m, int q, uint32_t *out, uint32_t *st) {
         typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
         const uint32_t w = (q / 4) == 0 ? raw.x : (q / 4) == 1 ? raw.y : (q / 4) == 2 ? raw.z : raw.w;
-        if (q == 0) { // scale and offset of the codes that stay four bits up
-            st[5] = __float_as_uint(m.s * 0.0625f);
-            st[6] = __float_as_uint(fmaf(960.0f, m.s, m.b)); // (b - 1024 s) + 960 s = b - 64 s
-        }
+        if (q == 0) st[5] = __float_as_uint(m.s * 0.0625f); // the scale of the codes that stay four bits up: s * 2^20
         if (q % 4 == 0) {
-            st[0] = (w & 0x000f000fu) | st[4]; // codes 0 | 4
-            st[1] = (w & 0x00f000f0u) | st[4]; // codes 1 | 5, sixteen-fold
+            st[0] = w & 0x000f000fu; // codes 0 | 4
+            st[1] = w & 0x00f000f0u; // codes 1 | 5, sixteen-fold
         } else if (q % 4 == 1) {
             const uint32_t w8 = w >> 8;
-            st[2] = (w8 & 0x000f000fu) | st[4]; // codes 2 | 6
-            st[3] = (w8 & 0x00f000f0u) | st[4]; // codes 3 | 7, sixteen-fold
+            st[2] = w8 & 0x000f000fu; // codes 2 | 6
+            st[3] = w8 & 0x00f000f0u; // codes 3 | 7, sixteen-fold
         }
         const f16x2_t a = __builtin_bit_cast(f16x2_t, st[(q % 2) * 2]), b = __builtin_bit_cast(f16x2_t, st[(q % 2) * 2 + 1]);
         const float va = (q % 4) < 2 ? (float)a.x : (float)a.y, vb = (q % 4) < 2 ? (float)b.x : (float)b.y;
-        out[q] = pack_bf16x2(fmaf(va, m.s, m.b), fmaf(vb, __uint_as_float(st[5]), __uint_as_float(st[6])));
+        out[q] = pack_bf16x2(fmaf(va, m.s, m.b), fmaf(vb, __uint_as_float(st[5]), m.b));
     }
 };
 

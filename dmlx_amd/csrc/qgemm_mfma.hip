@@ -324,6 +324,23 @@ bool qgemm_mfma_supports(const QView &b) {
     return b.mode != DMOE_QUANT_NONE && b.cols % (2 * vals) == 0 && b.cols % 64 == 0 && b.rows % 4 == 0;
 }
 
+template <typename Fmt, bool GATE_UP, bool PACKED>
+static int mfma_raise_limit() {
+    static LdsLimit limit; // per instantiation
+    return raise_lds_limit(limit, (const void *)qgemm_mfma_kernel<Fmt, GATE_UP, PACKED>, (int)MfmaGeom<Fmt>::kLdsBytes);
+}
+template <typename Fmt>
+static int mfma_prepare_format() {
+    DMOE_TRY((mfma_raise_limit<Fmt, true, false>()));
+    return mfma_raise_limit<Fmt, false, false>();
+}
+int qgemm_mfma_prepare() {
+    DMOE_TRY(mfma_prepare_format<FmtAffine4>());
+    DMOE_TRY(mfma_prepare_format<FmtAffine8>());
+    DMOE_TRY(mfma_prepare_format<FmtMxfp4>());
+    return mfma_prepare_format<FmtFp8Row>();
+}
+
 struct MfmaLaunch {
     const GemmArgs &g;
     hipStream_t st;
@@ -331,11 +348,7 @@ struct MfmaLaunch {
     int go() {
         auto kern = qgemm_mfma_kernel<Fmt, GATE_UP, PACKED>;
         const size_t lds = MfmaGeom<Fmt>::kLdsBytes;
-        static thread_local bool raised = false; // per instantiation: allow more than 64 KiB of dynamic LDS once
-        if (!raised) {
-            DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-            raised = true;
-        }
+        DMOE_TRY((mfma_raise_limit<Fmt, GATE_UP, PACKED>())); // done by dmoe_init for its device; a flag test otherwise
         const int cols_per_block = kMfmaWaves * (GATE_UP ? 32 : 64);
         dim3 grid((unsigned)ceil_div(g.b0.rows, cols_per_block), (unsigned)g.max_tiles), block(kMfmaWaves * 64);
         hipLaunchKernelGGL(kern, grid, block, lds, st, g);

@@ -102,7 +102,7 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
     // no barrier is involved).
     constexpr bool GROUPED = MBLK && RJT == 1;
     constexpr int LG = 4; // steps per 128-byte line = loads per group
-    constexpr int STAGES = GROUPED ? kSkinnyGroupedStages : RJT == 1 ? kSkinnyStages : kSkinnyStages / 2;
+    constexpr int STAGES = GROUPED ? kSkinnyGroupedStages : (RJT == 1 || !FACTORED) ? kSkinnyStages : kSkinnyStages / 2;
     constexpr int PRE = GROUPED ? STAGES : STAGES - 1; // stages requested before the first step is consumed
     constexpr int ROUND = MBLK && STAGES < 8 ? 8 : STAGES;  // steps per unrolled round (MBLK: whole blocks of entries)
     static_assert(ROUND % STAGES == 0 && (!MBLK || ROUND % 8 == 0), "rounds are whole turns of the ring");
@@ -611,6 +611,30 @@ static bool mlx_meta_blocks(const QView &b) {
            (!b.biases || ((uintptr_t)b.biases % 16) == 0);
 }
 
+template <typename Fmt, bool FACTORED, bool PACKED, bool MBLK>
+static int skinny_raise_limit() {
+    static LdsLimit limit; // per instantiation
+    return raise_lds_limit(limit, (const void *)qgemm_skinny_kernel<Fmt, FACTORED, PACKED, MBLK>, 150 * 1024);
+}
+// the instantiations SkinnyLaunch can pick for one format
+template <typename Fmt>
+static int skinny_prepare_format() {
+    constexpr bool can_factor = std::is_same<Fmt, FmtAffine4>::value;
+    constexpr bool has_entries = Fmt::kMetaEntryBytes != 0;
+    DMOE_TRY((skinny_raise_limit<Fmt, can_factor, true, false>()));
+    DMOE_TRY((skinny_raise_limit<Fmt, false, true, false>()));
+    DMOE_TRY((skinny_raise_limit<Fmt, can_factor, false, has_entries>()));
+    DMOE_TRY((skinny_raise_limit<Fmt, false, false, has_entries>()));
+    DMOE_TRY((skinny_raise_limit<Fmt, can_factor, false, false>()));
+    return skinny_raise_limit<Fmt, false, false, false>();
+}
+int qgemm_skinny_prepare() {
+    DMOE_TRY(skinny_prepare_format<FmtAffine4>());
+    DMOE_TRY(skinny_prepare_format<FmtAffine8>());
+    DMOE_TRY(skinny_prepare_format<FmtMxfp4>());
+    return skinny_prepare_format<FmtFp8Row>();
+}
+
 struct SkinnyLaunch {
     const GemmArgs &g;
     hipStream_t st;
@@ -619,11 +643,7 @@ struct SkinnyLaunch {
     int go() {
         auto kern = qgemm_skinny_kernel<Fmt, FACTORED, PACKED, MBLK>;
         const size_t lds = skinny_lds_bytes(g.b0) + (MBLK ? kSkinnyTurnBytes : 0);
-        static thread_local size_t allowed = 0; // per instantiation: raise the dynamic LDS limit once
-        if (lds > allowed) {
-            DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(150 * 1024)));
-            allowed = 150 * 1024;
-        }
+        DMOE_TRY((skinny_raise_limit<Fmt, FACTORED, PACKED, MBLK>())); // done by dmoe_init for its device; a flag test otherwise
         // 8 wavefronts per workgroup: 128 output columns of gate AND up, or 256 of a single projection
         auto blocks_x = [](const GemmArgs &a) { return ceil_div(a.b0.rows, (a.gate_up ? 1 : 2) * kSkinnyWaves * 32); };
         dim3 block(2 * kSkinnyWaves * 64);

@@ -369,13 +369,26 @@ bool qgemm_wide_supports(const QView &b) {
 }
 
 template <typename Fmt, bool GATE_UP>
+static int wide_raise_limit() {
+    static LdsLimit limit; // per instantiation
+    return raise_lds_limit(limit, (const void *)qgemm_wide_kernel<Fmt, GATE_UP>, (int)kWideLdsBytes);
+}
+template <typename Fmt>
+static int wide_prepare_format() {
+    DMOE_TRY((wide_raise_limit<Fmt, true>()));
+    return wide_raise_limit<Fmt, false>();
+}
+int qgemm_wide_prepare() {
+    DMOE_TRY(wide_prepare_format<FmtAffine4>());
+    DMOE_TRY(wide_prepare_format<FmtAffine8>());
+    DMOE_TRY(wide_prepare_format<FmtMxfp4>());
+    return wide_prepare_format<FmtFp8Row>();
+}
+
+template <typename Fmt, bool GATE_UP>
 static int launch_wide(const GemmArgs &g, hipStream_t st) {
     auto kern = qgemm_wide_kernel<Fmt, GATE_UP>;
-    static thread_local bool raised = false; // per instantiation: allow more than 64 KiB of dynamic LDS once
-    if (!raised) {
-        DMOE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLdsBytes));
-        raised = true;
-    }
+    DMOE_TRY((wide_raise_limit<Fmt, GATE_UP>())); // done by dmoe_init for its device; a flag test otherwise
     const int cols_per_block = kWideWaves * (GATE_UP ? 32 : 64);
     dim3 grid((unsigned)ceil_div(g.b0.rows, cols_per_block), (unsigned)((g.max_tiles + 7) / 8 * 8)), block(kWideWaves * 64);
     hipLaunchKernelGGL(kern, grid, block, kWideLdsBytes, st, g);

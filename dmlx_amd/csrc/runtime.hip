@@ -3,9 +3,24 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "common.h"
 
 namespace dmoe {
+
+static std::mutex lds_limit_mutex;
+
+int raise_lds_limit(LdsLimit &state, const void *kernel, int bytes) {
+    int dev = 0;
+    DMOE_HIP(hipGetDevice(&dev));
+    DMOE_REQUIRE(dev >= 0 && dev < kMaxDevices, "device index %d is out of range", dev);
+    std::lock_guard<std::mutex> lock(lds_limit_mutex);
+    if (state.raised >> dev & 1ull) return DMOE_OK;
+    DMOE_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+    state.raised |= 1ull << dev;
+    return DMOE_OK;
+}
 
 static thread_local char g_err[2048] = ""; // same size as the reference's mlx error buffer
 
@@ -54,6 +69,8 @@ int side_stream_ready(Workspace *w) {
 int stage_flush(Workspace *w) {
     StageTimer &t = w->timer;
     for (int i = 0; i < DMOE_STAGE_COUNT; ++i) {
+        // a stage whose start is recorded and whose stop is not keeps its slot: its ring is read at a later flush
+        if (t.open[i]) continue;
         for (int k = 0; k < t.pending[i]; ++k) {
             DMOE_HIP(hipEventSynchronize(t.stop[i][k]));
             float ms = 0.0f;
@@ -125,6 +142,11 @@ int dmoe_init(int device) {
     // resolve this device's copy of the static scratch now, so that the allocation-free entry point finds it ready
     Workspace *unused = nullptr;
     DMOE_TRY(static_workspace(&unused));
+    // and every GEMM kernel's dynamic-LDS limit: a first launch under stream capture or from another thread then has
+    // no host-side set-up left
+    DMOE_TRY(qgemm_wide_prepare());
+    DMOE_TRY(qgemm_mfma_prepare());
+    DMOE_TRY(qgemm_skinny_prepare());
     return DMOE_OK;
 }
 
@@ -300,6 +322,25 @@ int dmoe_workspace_set_weight_cache(dmoe_workspace ws, int enabled) {
     }
     w->cache_weights = enabled != 0;
     return DMOE_OK;
+}
+
+int dmoe_workspace_weight_cache_invalidate(dmoe_workspace ws, const dmoe_qweight *qw) {
+    Workspace *w = (Workspace *)ws.ctx;
+    DMOE_REQUIRE(w != nullptr, "workspace handle is null");
+    return weight_cache_invalidate(w, qw);
+}
+
+int dmoe_workspace_set_weight_cache_limit(dmoe_workspace ws, size_t max_bytes) {
+    Workspace *w = (Workspace *)ws.ctx;
+    DMOE_REQUIRE(w != nullptr, "workspace handle is null");
+    w->cache_limit_bytes = max_bytes;
+    return DMOE_OK;
+}
+
+int dmoe_workspace_weight_cache_stats(size_t *out_bytes, int *out_stacks, dmoe_workspace ws) {
+    Workspace *w = (Workspace *)ws.ctx;
+    DMOE_REQUIRE(w != nullptr, "workspace handle is null");
+    return weight_cache_stats(w, out_bytes, out_stacks);
 }
 
 int dmoe_workspace_set_paired_launch(dmoe_workspace ws, int enabled) {

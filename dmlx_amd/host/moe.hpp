@@ -66,6 +66,9 @@ class Context {
     // reported a time-out at synchronize() has already switched the workspace to two launches
     // gatherQmm on borrowed MLX-layout arrays: keep re-ordered resident copies of the stacks seen (see dmoe.h)
     void setWeightCache(bool enabled) const { check(dmoe_workspace_set_weight_cache(ws_, enabled ? 1 : 0)); }
+    // before a cached stack is freed or rewritten (null: every copy); the cap pushes out least recently used copies
+    void invalidateWeightCache(const dmoe_qweight *qw = nullptr) const { check(dmoe_workspace_weight_cache_invalidate(ws_, qw)); }
+    void setWeightCacheLimit(size_t max_bytes) const { check(dmoe_workspace_set_weight_cache_limit(ws_, max_bytes)); }
     void setPairedLaunch(bool enabled) const { check(dmoe_workspace_set_paired_launch(ws_, enabled ? 1 : 0)); }
 
   private:

@@ -55,6 +55,14 @@ pub const Context = struct {
     pub fn setWeightCache(self: Context, enabled: bool) Error!void {
         try check(c.dmoe_workspace_set_weight_cache(self.ws, @intFromBool(enabled)));
     }
+    /// before a cached stack is freed or rewritten while the cache is on (null: drop every copy)
+    pub fn invalidateWeightCache(self: Context, qw: ?*const c.dmoe_qweight) Error!void {
+        try check(c.dmoe_workspace_weight_cache_invalidate(self.ws, qw));
+    }
+    /// byte cap of the cached copies (0 = none); a new stack beyond it pushes out the least recently used ones
+    pub fn setWeightCacheLimit(self: Context, max_bytes: usize) Error!void {
+        try check(c.dmoe_workspace_set_weight_cache_limit(self.ws, max_bytes));
+    }
     /// decode steps: gate/up and down in one launch (default) or as two launches that wait for nothing; after `eval`
     /// reported a time-out the workspace is already on two launches
     pub fn setPairedLaunch(self: Context, enabled: bool) Error!void {

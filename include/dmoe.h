@@ -230,8 +230,19 @@ int dmoe_gather_qmm(uint16_t *d_out, const uint16_t *d_x, const dmoe_qweight *qw
  * dmoe_gather_qmm_resident does. A stack is recognised by its three pointers, shape and format: the caller promises
  * that the arrays behind cached pointers neither change nor are freed while the cache is on. Costs the stack's size
  * in HBM again. enabled = 0 (the default) drops every copy; so does dmoe_workspace_destroy. Same results either way.
- * No counterpart in the reference (its QuantizedWeight arrays live as long as the model). */
+ * No counterpart in the reference (its QuantizedWeight arrays live as long as the model).
+ *
+ * An allocator that recycles addresses can hand a freed stack's pointers to a NEW stack of the same shape; the cache
+ * cannot tell the two apart and would serve the old copy. A caller that frees or rewrites a stack while the cache is
+ * on calls dmoe_workspace_weight_cache_invalidate with that stack's descriptor first (qw = null drops every copy; it
+ * waits for the device, since kernels in flight may still read a copy). The copies are capped by bytes
+ * (dmoe_workspace_set_weight_cache_limit, default 32 GiB, 0 = no cap): a new stack that would exceed the cap pushes
+ * out the least recently used copies, which costs one wait for the device. dmoe_workspace_weight_cache_stats reports
+ * what is held. */
 int dmoe_workspace_set_weight_cache(dmoe_workspace ws, int enabled);
+int dmoe_workspace_weight_cache_invalidate(dmoe_workspace ws, const dmoe_qweight *qw);
+int dmoe_workspace_set_weight_cache_limit(dmoe_workspace ws, size_t max_bytes);
+int dmoe_workspace_weight_cache_stats(size_t *out_bytes, int *out_stacks, dmoe_workspace ws);
 
 /* The same call on a stack that was made resident once: mlx-zig's QuantizedWeight is a long-lived object (the w /
  * scales / biases Arrays of DSV4SwitchGLU live as long as the model, deepseek_v4.zig:687-717), and its counterpart
@@ -341,10 +352,16 @@ int dmoe_moe_layer_forward(uint16_t *d_out, uint32_t *d_out_indices, float *d_ou
  *   - a batch whose buffers do not fit is rejected with DMOE_ERR_INVALID and a message naming the size (at D = 4096,
  *     F = 2048, K = 6 with a folded shared expert: up to 195 tokens);
  *   - gate/up and down always run as two launches and a shared expert of another format runs after them on the same
- *     stream, so nothing waits inside a kernel and there is nothing to check afterwards; results are bit-identical;
+ *     stream, so nothing waits inside a kernel; results are bit-identical;
+ *   - there is no dmoe_workspace_check for this entry point and none is needed: the two conditions that check reports
+ *     cannot arise here. No kernel waits (see above), and the expert ids reach the packing step from the call's own
+ *     routing - a top-k over E_total scores, mapped through the remap that dmoe_layer_create validated - so they are
+ *     always inside the layer's range (the reference's remap gives the same guarantee, expert_preload.zig:141-149).
+ *     The flag words the packing kernels would count bad ids in sit in the static array and are never read;
  *   - every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race.
- * The array's address is resolved by dmoe_init on the device it selects, else by the first call on a device (do not
- * make that first call under stream capture). */
+ * The array's address and every kernel's launch attributes are set up by dmoe_init on the device it selects, else by
+ * the first call on a device (do not make that first call under stream capture). After that a call does no host-side
+ * set-up and can be captured into a HIP graph from any thread. */
 int dmoe_moe_layer_forward_static(uint16_t *d_out, uint32_t *d_out_indices, float *d_out_weights, dmoe_layer layer,
                                   const uint16_t *d_x, const float *d_scores, const float *d_bias,
                                   const uint8_t *d_resident_mask, int T, int E_total, int renorm, float route_scale,
@@ -423,6 +440,11 @@ int dmoe_batch_build(uint32_t *d_out_tokens, int32_t *d_out_positions, float *d_
 /* Inspection of the last dmoe_moe_forward / dmoe_switch_glu_forward_no_scores on this workspace:
  * the SwiGLU activations in flat (t*K+k) row order, bf16 [T*K, F]. For parity tests. */
 int dmoe_debug_last_activations(uint16_t *d_out, dmoe_layer layer, int T, dmoe_workspace ws, dmoe_stream s);
+
+/* dmoe_dequantize through the decoder that the prefill kernels run in registers between their matrix instructions
+ * (same arguments, same result layout). For parity tests: the fused decode must give the bits of dmoe_dequantize,
+ * i.e. of mlx_dequantize as called at deepseek_v4_loader.zig:129, for every scale and bias. */
+int dmoe_debug_dequantize_fused(uint16_t *d_out, const dmoe_qweight *qw, int mat_index, dmoe_stream s);
 
 #ifdef __cplusplus
 }

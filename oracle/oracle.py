@@ -110,6 +110,28 @@ class QMat:
                      self.mode, self.bits, self.group)
 
 
+def bf16_bits(t):
+    """A torch bf16 tensor (any device) -> numpy uint16 bit patterns."""
+    import torch
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def qmat(qw):
+    """A weight stack as the harness holds it (torch tensors `w`, `scales`, `biases` in MLX layout plus `rows`, `cols`,
+    `mode`, `bits`, `group_size`; the mode numbers are those of include/dmoe.h) -> QMat over numpy copies."""
+    w = qw.w.detach().cpu().contiguous()
+    if qw.mode == NONE:
+        return QMat(bf16_bits(w), None, None, qw.rows, qw.cols, NONE, 16, 0)
+    s = qw.scales.detach().cpu().contiguous()
+    b = None if qw.biases is None else qw.biases.detach().cpu().contiguous()
+    if qw.mode == FP8_ROW:
+        return QMat(w.numpy(), s.numpy(), None, qw.rows, qw.cols, FP8_ROW, 8, 0)
+    if qw.mode == MXFP4:
+        return QMat(w.numpy().view(np.uint32), s.numpy(), None, qw.rows, qw.cols, MXFP4, 4, 32)
+    return QMat(w.numpy().view(np.uint32), bf16_bits(s), None if b is None else bf16_bits(b),
+                qw.rows, qw.cols, AFFINE, qw.bits, qw.group_size)
+
+
 def topk_route(scores, K, normalize=True):
     s = _c(scores, np.float32)
     T, E = s.shape

@@ -2,36 +2,16 @@
 import numpy as np
 import torch
 
-from dmlx_amd import capi
 from oracle import oracle
+from oracle.oracle import bf16_bits, qmat  # noqa: F401  (re-exported: the tests import them from here)
 
 
 def to_np_u32(t):
     return t.detach().cpu().contiguous().numpy().view(np.uint32)
 
 
-def bf16_bits(t):
-    """torch bf16 tensor -> numpy uint16 bit patterns"""
-    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
-
-
 def bf16_to_f32(t):
     return t.detach().cpu().float().numpy()
-
-
-def qmat(qw):
-    """capi.QWeight (torch, any device) -> oracle.QMat (numpy)"""
-    w = qw.w.detach().cpu().contiguous()
-    if qw.mode == capi.QUANT_NONE:
-        return oracle.QMat(bf16_bits(w), None, None, qw.rows, qw.cols, oracle.NONE, 16, 0)
-    s = qw.scales.detach().cpu().contiguous()
-    b = None if qw.biases is None else qw.biases.detach().cpu().contiguous()
-    if qw.mode == capi.QUANT_FP8_ROW:
-        return oracle.QMat(w.numpy(), s.numpy(), None, qw.rows, qw.cols, oracle.FP8_ROW, 8, 0)
-    if qw.mode == capi.QUANT_MXFP4:
-        return oracle.QMat(w.numpy().view(np.uint32), s.numpy(), None, qw.rows, qw.cols, oracle.MXFP4, 4, 32)
-    return oracle.QMat(w.numpy().view(np.uint32), bf16_bits(s), None if b is None else bf16_bits(b),
-                       qw.rows, qw.cols, oracle.AFFINE, qw.bits, qw.group_size)
 
 
 def max_abs_rel(got, ref):
@@ -82,4 +62,34 @@ def dense_reference_f64(x_bits, idx, w, gate, up, down, limit=0.0, shared=None, 
         np.add.at(out, tok, y * w.reshape(-1)[pos].astype(np.float64)[:, None])
     if shared is not None:
         out += ffn(x, deq(shared[0], 0), deq(shared[1], 0), deq(shared[2], 0), shared_limit)
+    return out
+
+
+def dense_reference_f64_device(x, idx, w, gate, up, down, limit=0.0, shared=None, shared_limit=0.0, device="cuda"):
+    """dense_reference_f64 for whole prefill batches: the same float64 evaluation (no intermediate rounding), with the
+    matrix products done by torch on `device`. The weights are the ORACLE's dequantized values (oracle.dequantize_f32
+    on the CPU, one expert at a time, then copied over); nothing of the library under test takes part.
+    x: torch bf16 [T, D]; idx: numpy [T, K] slot ids; w: numpy f32 [T, K]. Returns a float64 tensor [T, D] on `device`."""
+    T, K = idx.shape
+    xd = x.to(device).to(torch.float64)
+
+    def deq(qm, m):
+        return torch.from_numpy(oracle.dequantize_f32(qm, m)).to(device).to(torch.float64)
+
+    def ffn(xr, g_, u_, d_, L):
+        g, u = xr @ g_.T, xr @ u_.T
+        if L > 0:
+            g, u = torch.clamp(g, max=L), torch.clamp(u, -L, L)
+        return (g / (1.0 + torch.exp(-g)) * u) @ d_.T
+
+    out = torch.zeros((T, down.rows), dtype=torch.float64, device=device)
+    flat = torch.from_numpy(idx.reshape(-1).astype(np.int64)).to(device)
+    wf = torch.from_numpy(w.reshape(-1).astype(np.float64)).to(device)
+    for e in np.unique(idx.reshape(-1)):
+        pos = torch.nonzero(flat == int(e)).reshape(-1)
+        tok = pos // K
+        y = ffn(xd[tok], deq(gate, int(e)), deq(up, int(e)), deq(down, int(e)), limit)
+        out.index_add_(0, tok, y * wf[pos][:, None])   # a token holds an expert at most once: no duplicate indices
+    if shared is not None:
+        out += ffn(xd, deq(shared[0], 0), deq(shared[1], 0), deq(shared[2], 0), shared_limit)
     return out

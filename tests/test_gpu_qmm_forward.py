@@ -56,11 +56,12 @@ def test_dequantize_bit_exact(dmoe, orc, fmt):
         qw.w[0, 0, :256] = torch.arange(256, dtype=torch.uint8, device="cuda")
     qm = qmat(qw)
     for m in range(3):
-        got = bf16_bits(dmoe.dequantize(qw, m))
         want = orc.dequantize(qm, m)
         nan = (want & 0x7FFF) > 0x7F80
-        np.testing.assert_array_equal(got[~nan], want[~nan])
-        assert ((got[nan] & 0x7FFF) > 0x7F80).all()
+        for fused in (False, True) if fmt != "bf16" else (False,):   # fused: the prefill kernels' in-register decoder
+            got = bf16_bits(dmoe.dequantize(qw, m, fused=fused))
+            np.testing.assert_array_equal(got[~nan], want[~nan], err_msg=f"{fmt} fused={fused}")
+            assert ((got[nan] & 0x7FFF) > 0x7F80).all()
 
 
 @pytest.mark.parametrize("fmt", FORMATS)
@@ -173,6 +174,51 @@ def test_gather_qmm_weight_cache_gives_the_resident_results(dmoe, orc, ws):
     assert max_abs_rel(plain.float().cpu().numpy(), want) < OUT_TOL
 
 
+def test_gather_qmm_weight_cache_invalidate_and_cap(dmoe, orc, ws):
+    """A stack rewritten in place keeps its pointers, so the cache cannot tell: it serves the old copy until the
+    caller invalidates that stack, after which the call sees the new bytes. The byte cap pushes out the least recently
+    used copies; results stay right throughout."""
+    g = torch.Generator(device="cuda").manual_seed(5)
+    qw = _stack("affine4", 4, 128, 512, 401)
+    other = _stack("mxfp4", 3, 128, 512, 402)
+    R = 16
+    x = torch.randn((R, qw.cols), generator=g, device="cuda").to(torch.bfloat16)
+    rhs = torch.randint(0, 3, (R,), generator=g, device="cuda", dtype=torch.int32)
+    ws.set_weight_cache(True)
+    try:
+        old = dmoe.gather_qmm(x, qw, rhs, ws)
+        dmoe.gather_qmm(x, other, rhs, ws)
+        assert ws.weight_cache_stats()[1] == 2
+        fresh = _stack("affine4", 4, 128, 512, 403)
+        qw.w.copy_(fresh.w), qw.scales.copy_(fresh.scales), qw.biases.copy_(fresh.biases)   # same addresses, new values
+        want_new = orc.gather_qmm(bf16_bits(x), qmat(qw), to_np_u32(rhs), None)
+        stale = dmoe.gather_qmm(x, qw, rhs, ws)
+        assert torch.equal(stale, old)                           # what the documentation warns about
+        ws.invalidate_weight_cache(qw)
+        assert ws.weight_cache_stats()[1] == 1                   # only that stack's copy went
+        got = dmoe.gather_qmm(x, qw, rhs, ws)
+        assert max_abs_rel(got.float().cpu().numpy(), want_new) < OUT_TOL
+        assert not torch.equal(got, old)
+        held, n = ws.weight_cache_stats()
+        assert n == 2 and held > 0
+        # cap below two copies: adding a third stack leaves only the most recent ones that fit
+        ws.set_weight_cache_limit(held)
+        third = _stack("affine8", 2, 128, 512, 404)
+        got3 = dmoe.gather_qmm(x, third, rhs % 2, ws)
+        want3 = orc.gather_qmm(bf16_bits(x), qmat(third), to_np_u32(rhs % 2), None)
+        assert max_abs_rel(got3.float().cpu().numpy(), want3) < OUT_TOL
+        held3, n3 = ws.weight_cache_stats()
+        assert held3 <= held and 1 <= n3 <= 2
+        again = dmoe.gather_qmm(x, qw, rhs, ws)                  # possibly re-made: same bits either way
+        assert torch.equal(again, got)
+        ws.invalidate_weight_cache()
+        assert ws.weight_cache_stats() == (0, 0)
+        ws.check()
+    finally:
+        ws.set_weight_cache_limit(32 << 30)
+        ws.set_weight_cache(False)
+
+
 @pytest.mark.parametrize("fmt", FORMATS)
 def test_gather_qmm_seeded_random_shapes(dmoe, orc, ws, fmt):
     """Twelve seeded shapes per format across both paths and both layouts: odd expert counts, weight rows that are
@@ -210,6 +256,78 @@ def test_gather_qmm_one_expert_takes_every_row(dmoe, orc, ws, fmt, R):
     got = dmoe.gather_qmm(x, qw, rhs, ws, None).float().cpu().numpy()
     want = orc.gather_qmm(bf16_bits(x), qmat(qw), to_np_u32(rhs), None)
     assert max_abs_rel(got, want) < OUT_TOL, (fmt, R, max_abs_rel(got, want))
+
+
+def _adversarial_affine(bits, n_mats, rows, cols, seed):
+    """Random codes with HAND-SET bf16 scales and biases: every group takes one of seven relations between the bias b
+    and the scale s that a min/max quantizer never produces together: b = 0, |b| = s / 256, b = +3 s, |b| = 100 s,
+    b = -7.5 s (the usual case, for contrast), b = -s, and a negative scale with a positive bias. Scales are
+    (1 + m / 128) 2^e with all eight significant bits in use."""
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    n_groups = cols // 64
+    codes = torch.randint(0, 2 ** bits, (n_mats, rows, cols), generator=g, device="cuda")
+    mant = torch.randint(0, 128, (n_mats, rows, n_groups), generator=g, device="cuda").float()
+    expo = torch.randint(-9, -5, (n_mats, rows, n_groups), generator=g, device="cuda").float()
+    s = ((1.0 + mant / 128.0) * torch.exp2(expo)).to(torch.bfloat16)
+    kind = (torch.arange(n_groups, device="cuda")[None, None, :] + torch.arange(rows, device="cuda")[None, :, None]) % 7
+    sf = s.float()
+    b = torch.zeros_like(sf)
+    b = torch.where(kind == 1, -sf / 256.0, b)
+    b = torch.where(kind == 2, 3.0 * sf, b)
+    b = torch.where(kind == 3, -100.0 * sf, b)
+    b = torch.where(kind == 4, -7.5 * sf, b)
+    b = torch.where(kind == 5, -sf, b)
+    s = torch.where(kind == 6, -sf, sf).to(torch.bfloat16)
+    b = torch.where(kind == 6, 11.0 * sf, b).to(torch.bfloat16)
+    return QWeight(Q._pack_codes(codes, bits), s, b, rows, cols, QUANT_AFFINE, bits, 64)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_affine_decode_on_adversarial_scales_and_biases(dmoe, orc, ws, bits):
+    """The in-kernel affine decode (prefill kernels: (1024 + c) s + (b - 1024 s) through an f16 magic number; decode
+    kernel: scales factored out of the matrix product) on scale / bias pairs for which b - 1024 s is NOT exactly
+    representable in f32, on zero and positive biases and on biases far above the scale. dmoe_dequantize must give
+    the oracle's bits; every GEMM path must stay within the output bar of the oracle; and the prefill and the decode
+    kernels, fed the same rows, must agree to two bf16 steps of the value (plus accumulation-order noise). Two, not
+    one: the prefill kernels multiply bf16-rounded weights (the values of dmoe_dequantize), the 4-bit decode kernel
+    factors the scale out of the matrix product and never rounds a weight, and where |b| = 100 |s| that rounding is a
+    fifth of a code step per weight."""
+    n_mats, rows, cols = 3, 128, 1024
+    qw = _adversarial_affine(bits, n_mats, rows, cols, 40 + bits)
+    qm = qmat(qw)
+    for m in range(n_mats):
+        want_bits = orc.dequantize(qm, m)
+        np.testing.assert_array_equal(bf16_bits(dmoe.dequantize(qw, m)), want_bits)
+        # the decoder fused into the prefill kernels: the same bits, also where b - 1024 s would not be representable
+        np.testing.assert_array_equal(bf16_bits(dmoe.dequantize(qw, m, fused=True)), want_bits)
+    g = torch.Generator(device="cuda").manual_seed(bits)
+    R = 8 * n_mats + 400                                  # prefill-sized: the matrix-core kernels
+    x = torch.randn((R, cols), generator=g, device="cuda").to(torch.bfloat16)
+    rhs = torch.randint(0, n_mats, (R,), generator=g, device="cuda", dtype=torch.int32)
+    want = orc.gather_qmm(bf16_bits(x), qm, to_np_u32(rhs), None)
+    res = dmoe.ResidentWeight(qw)
+    big = {"resident": res.gather_qmm(x, rhs, ws), "mlx": dmoe.gather_qmm(x, qw, rhs, ws)}
+    for name, got in big.items():
+        err = max_abs_rel(got.float().cpu().numpy(), want)
+        assert err < OUT_TOL, (bits, "prefill kernels", name, err)
+    # the same rows in decode-sized calls (8 rows per matrix at most): the weight-streaming kernel
+    step = 8 * n_mats
+    small = {"resident": [], "mlx": []}
+    for r0 in range(0, 3 * step, step):
+        small["resident"].append(res.gather_qmm(x[r0:r0 + step].contiguous(), rhs[r0:r0 + step].contiguous(), ws))
+        small["mlx"].append(dmoe.gather_qmm(x[r0:r0 + step].contiguous(), qw, rhs[r0:r0 + step].contiguous(), ws))
+    top = float(np.abs(want).max())
+    for name in small:
+        got = torch.cat(small[name]).float().cpu().numpy()
+        err = max_abs_rel(got, want[:3 * step])
+        assert err < OUT_TOL, (bits, "decode kernel", name, err)
+        ref = big[name][:3 * step].float().cpu().numpy()
+        gap = np.abs(got - ref)
+        allowed = np.maximum(np.abs(got), np.abs(ref)) * 2.0 ** -6 + 1e-3 * top
+        assert (gap <= allowed).all(), (bits, name, "prefill and decode kernels differ by more than two bf16 steps",
+                                        float((gap - allowed).max()))
+    res.close()
+    ws.check()
 
 
 def _route(dmoe, orc, wl):

@@ -389,6 +389,14 @@ def test_grouped_float64_reference_equals_the_row_by_row_one(orc):
     np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-14)
     clamped = dense_reference_f64(x_bits, idx, w, gate, up, down, 0.7, sh, 0.01)
     assert np.abs(clamped - want).max() > 1e-6      # the shared expert's own limit is applied
+    # the torch twin that the GPU tests use on whole prefill batches (run here on the CPU)
+    import torch
+    from tests.helpers import dense_reference_f64_device
+    x_t = torch.from_numpy(orc.bf16_to_f32(x_bits)).to(torch.bfloat16)
+    twin = dense_reference_f64_device(x_t, idx, w, gate, up, down, 0.7, sh, 0.0, device="cpu").numpy()
+    np.testing.assert_allclose(twin, want, rtol=1e-10, atol=1e-13)
+    twin_clamped = dense_reference_f64_device(x_t, idx, w, gate, up, down, 0.7, sh, 0.01, device="cpu").numpy()
+    np.testing.assert_allclose(twin_clamped, clamped, rtol=1e-10, atol=1e-13)
 
 
 # ---------------------------------------------------------------- batch builder --------------------------------

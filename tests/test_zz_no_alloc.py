@@ -77,3 +77,46 @@ def test_static_entry_point_allocates_nothing_and_rejects_large_batches(dmoe, ws
         assert torch.equal(again.view(torch.int16), want.view(torch.int16))
     finally:
         layer.close()
+
+
+@pytest.mark.parametrize("config,scale,T", [(1, 0.5, 48), (4, 0.125, 200)])
+def test_static_entry_point_under_graph_capture(dmoe, ws, config, scale, T):
+    """The callers this entry point is for include code under HIP graph capture: one static forward is captured
+    (after an eager call, so that nothing host-side is left to set up) and replayed on changing inputs, with eager
+    work and synchronizations between the replays; every replay must give the bits of the workspace entry point."""
+    wl = workloads.make(config, device="cuda", scale=scale)
+    T = min(T, wl.T)
+    layer = _layer(dmoe, wl)
+    try:
+        scores = wl.scores[:T].contiguous()
+        x_a = wl.x[:T].contiguous()
+        x_b = torch.roll(x_a, 1, dims=0).contiguous()
+        route = (wl.bias, wl.resident_mask, wl.renorm, wl.route_scale)
+        want_a = layer.layer_forward(x_a, scores, *route, ws).clone()
+        want_b = layer.layer_forward(x_b, scores, *route, ws).clone()
+        x_in = x_a.clone()
+        out = torch.empty((T, wl.D), dtype=torch.bfloat16, device="cuda")
+        layer.layer_forward(x_in, scores, *route, None, out=out)     # eager static call first
+        torch.cuda.synchronize()
+        assert torch.equal(out, want_a)
+        free0, _ = torch.cuda.mem_get_info()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            layer.layer_forward(x_in, scores, *route, None, out=out)
+        torch.cuda.synchronize()
+        for i, (x, want) in enumerate([(x_a, want_a), (x_b, want_b), (x_b, want_b), (x_a, want_a)]):
+            x_in.copy_(x)
+            out.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, want), f"config {config}: replay {i} of the captured static forward differs"
+            eager = layer.layer_forward(x, scores, *route, ws)        # eager work between the replays
+            torch.cuda.synchronize()
+            assert torch.equal(eager, want)
+        ws.check()
+        del graph
+        torch.cuda.synchronize()
+    finally:
+        layer.close()
