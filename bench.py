@@ -37,6 +37,7 @@ COPY_PROBE_BYTES = 256 << 20  # --copy-probe: bytes read (and written) by each c
 COUNTERS_FILE = os.path.join(ROOT, "profiles", "counters.json")   # written from the rocprofv3 --pmc summaries
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
+SMALL_PATH_AVG_ROWS = 16     # at most this many rows per resident expert on average: weight-streaming kernel (kSkinnyAvgRows in csrc/layer.hip)
 WIDE_TILE_ROWS = 128         # rows per tile of the library's matrix-core kernels (kMfmaWideTileM in csrc/common.h)
 
 
@@ -223,7 +224,7 @@ def describe(torch, wl, config, timing, U, counts, steps, warmup, counters):
     gate_up_w = (wl.gate.nbytes() + wl.up.nbytes()) // wl.E
     down_w = wl.down.nbytes() // wl.E
     kern = "gate_up" if stages["gate_up"] >= stages["down"] else "down"
-    decode = rows <= 8 * wl.E   # the library's own rule for the small-M path (8 rows per resident expert on average)
+    decode = rows <= SMALL_PATH_AVG_ROWS * wl.E   # the library's own rule for the small-M path
     # At decode sizes a shared expert of the routed experts' format rides in the routed launches as one more expert
     # with T rows (the library's rule: small-M path, same shape / mode / bits / group): its weights and rows count.
     sh = wl.shared
@@ -357,7 +358,7 @@ def main():
                         f"pre-run and {args.warmup} warm-up steps")
     if not args.no_peaks:
         result["roofline"]["measured_peaks"] = measured_peaks(torch)
-    decode = wl.T * wl.K <= 8 * wl.E
+    decode = wl.T * wl.K <= SMALL_PATH_AVG_ROWS * wl.E
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(wl, max_tokens=64 if decode else 256)
     else:

@@ -174,8 +174,11 @@ __global__ void combine_kernel(uint16_t *__restrict__ out, const uint16_t *__res
 
 // ---- forward -------------------------------------------------------------------------------------------
 
-// at or below this many rows per expert on average the skinny (weight-streaming) kernel runs every tile
-constexpr int kSkinnyAvgRows = 8;
+// At or below this many rows per expert on average the skinny (weight-streaming) kernel runs every tile. Measured on one
+// projection [128, 2048, 4096] with every expert live (TB/s of weight bytes, whole call): at 12 and 16 rows per expert
+// the weight-streaming kernel gives 4.1 / 4.0 against the matrix-core kernel's 3.5 / 3.6 (4-bit affine), 4.5 / 4.3 against
+// 4.4 / 4.3 (MXFP4), 5.3 / 5.3 against 5.2 / 5.2 (8-bit); at 24 and 32 rows the matrix-core kernel is level or ahead.
+constexpr int kSkinnyAvgRows = 16;
 constexpr int kSharedSkinnyRows = 64;
 
 static bool use_small_path(size_t rows, int n_experts, const QView &b) {

@@ -91,8 +91,10 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
     constexpr int KV = Fmt::kVals;   // values per 16-byte chunk
     constexpr int KSTEP = 2 * KV;    // reduction elements per step (both lane halves)
     constexpr int NJ = KV / 8;       // MFMAs (K = 16) per step
-    // depth of the weight ring: the large-tile copy keeps 16 accumulators per lane and takes a shallower ring to
-    // stay inside the same register budget (span boundaries stay whole ring rounds either way)
+    // depth of the weight ring: the large-tile copy of the factored 4-bit form keeps 16 accumulators AND 16 products
+    // per lane and takes a shallower ring to stay inside the same register budget (span boundaries stay whole ring
+    // rounds either way); the other formats have the registers for the full ring (32 rows per expert, 256 live
+    // experts, MXFP4: 4.2 -> 4.4 TB/s)
     // MLX layout, tiles of one row block (GROUPED): in the operand layout a wavefront's load would take 32 bytes out of
     // each of 32 rows (32 cache lines per instruction, a quarter of each used, the same lines again for the next three
     // steps; measured 2.7 TB/s at best). Instead lane l of load i fetches 16 bytes of row 8 i + l / 8, eight lanes
@@ -395,7 +397,7 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
             }
             // with 16 products per lane alive, letting the next step's matrix instructions start before this step's
             // scaling has finished would double them: keep the steps apart (other wavefronts fill the wait)
-            if (RJT > 1 || GROUPED) __builtin_amdgcn_sched_barrier(0);
+            if ((RJT > 1 && FACTORED) || GROUPED) __builtin_amdgcn_sched_barrier(0);
         };
 
         // GROUPED: ring stages j .. j+3 (one group as loaded) -> the chunks of its four steps in the operand layout

@@ -107,7 +107,7 @@ def test_gather_qmm_on_a_resident_stack(dmoe, orc, ws, fmt, R, n_mats, rows, col
     for use_lhs in (False, True):
         got = res.gather_qmm(x, rhs, ws, lhs if use_lhs else None)
         plain = dmoe.gather_qmm(x, qw, rhs, ws, lhs if use_lhs else None)
-        if R <= 8 * n_mats:
+        if R <= 16 * n_mats:   # both calls on the weight-streaming kernel
             assert torch.equal(got, plain), (fmt, use_lhs)
         else:
             # one bf16 step of the largest output at most (2^-7 of its value)
@@ -229,7 +229,7 @@ def test_gather_qmm_seeded_random_shapes(dmoe, orc, ws, fmt):
         n_mats = int(rng.integers(1, 13))
         rows = 4 * int(rng.integers(2, 81)) if case % 3 else 32 * int(rng.integers(1, 9))
         cols = 128 * int(rng.integers(1, 13)) if fmt == "affine4g128" else 64 * int(rng.integers(1, 25))
-        R = int(rng.integers(1, 40)) if case % 2 else int(rng.integers(8 * n_mats + 1, 8 * n_mats + 600))
+        R = int(rng.integers(1, 40)) if case % 2 else int(rng.integers(16 * n_mats + 1, 16 * n_mats + 600))
         qw = _stack(fmt, n_mats, rows, cols, 100 + case)
         g = torch.Generator(device="cuda").manual_seed(case)
         x = torch.randn((R + 2, cols), generator=g, device="cuda").to(torch.bfloat16)
@@ -301,7 +301,7 @@ def test_affine_decode_on_adversarial_scales_and_biases(dmoe, orc, ws, bits):
         # the decoder fused into the prefill kernels: the same bits, also where b - 1024 s would not be representable
         np.testing.assert_array_equal(bf16_bits(dmoe.dequantize(qw, m, fused=True)), want_bits)
     g = torch.Generator(device="cuda").manual_seed(bits)
-    R = 8 * n_mats + 400                                  # prefill-sized: the matrix-core kernels
+    R = 16 * n_mats + 400                                 # prefill-sized: the matrix-core kernels
     x = torch.randn((R, cols), generator=g, device="cuda").to(torch.bfloat16)
     rhs = torch.randint(0, n_mats, (R,), generator=g, device="cuda", dtype=torch.int32)
     want = orc.gather_qmm(bf16_bits(x), qm, to_np_u32(rhs), None)
@@ -389,10 +389,12 @@ def test_c0_small_layer_full_size(dmoe, orc, ws):
     layer.close()
 
 
-@pytest.mark.parametrize("config,scale", [(1, 0.125), (1, 0.5), (2, 0.125), (2, 0.5), (3, 0.125), (4, 0.125)])
+@pytest.mark.parametrize("config,scale", [(1, 0.0625), (1, 0.125), (1, 0.5), (2, 0.0625), (2, 0.125), (2, 0.5), (3, 0.125),
+                                          (4, 0.125)])
 def test_configs_reduced_size(dmoe, orc, ws, config, scale):
-    """Configurations 1-4 with E, D, F shrunk (same formats, routing rules and raggedness). Scale 0.5 keeps
-    the decode configurations on the small-M kernel, 0.125 puts them on the MFMA kernel."""
+    """Configurations 1-4 with E, D, F shrunk (same formats, routing rules and raggedness). Scales 0.5 and 0.125 keep
+    the decode configurations on the small-M kernel (at most 16 rows per expert on average), 0.0625 (16 experts) puts
+    them on the MFMA kernel."""
     wl = workloads.make(config, scale=scale)
     _check_layer(dmoe, orc, ws, wl)
 
