@@ -46,33 +46,6 @@ __device__ uint32_t block_excl_scan(uint32_t v, uint32_t *total, uint32_t *sm /*
     return sm[wave] + incl - v;
 }
 
-// the same for a 64-bit value (several small counters packed into one word scan together); sm64 holds kPackWaves + 1 words
-__device__ uint64_t block_excl_scan64(uint64_t v, uint64_t *total, uint64_t *sm64) {
-    const int lane = lane_id(), wave = (int)(threadIdx.x >> 6);
-    uint64_t incl = v;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        uint64_t o = (uint64_t)__shfl_up((long long)incl, off, 64);
-        if (lane >= off) incl += o;
-    }
-    __syncthreads(); // sm64 may still be read from a previous call
-    if (lane == 63) sm64[wave] = incl;
-    __syncthreads();
-    if (wave == 0) {
-        uint64_t t = lane < kPackWaves ? sm64[lane] : 0ull, ti = t;
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            uint64_t o = (uint64_t)__shfl_up((long long)ti, off, 64);
-            if (lane >= off) ti += o;
-        }
-        if (lane < kPackWaves) sm64[lane] = ti - t;
-        if (lane == 63) sm64[kPackWaves] = ti;
-    }
-    __syncthreads();
-    *total = sm64[kPackWaves];
-    return sm64[wave] + incl - v;
-}
-
 // lanes of this wavefront that hold the same expert id (only among `active` lanes)
 __device__ __forceinline__ uint64_t match_expert(uint32_t e, bool active, int nbits) {
     uint64_t peers = __ballot(active);
@@ -125,40 +98,18 @@ __device__ uint32_t emit_segments(uint32_t count, int e, int E, size_t n, int ti
             t.flags = kTileDense;
             o.tiles[j] = t;
         }
-        // Order of the list = order in which the GEMM launches start their workgroups. A tile's run time grows with its
-        // rows (in steps of 32), and a launch ends with a tail as long as its last workgroups, so the long tiles go
-        // first and the short ones last:
-        //   class 0  every tile above kPackSmallTileRows rows of an expert that fills at least one whole tile, in expert
-        //            order (an expert's tiles stay together: they share its weights through the L2), then
-        //   class c  the single tiles of the other experts by falling size, c = 1 + (4 - quarter), quarter = the number of
-        //            started quarters of tile_m the tile holds (4, 3, 2, 1), then
-        //   class 5  the tiles of at most kPackSmallTileRows rows (on the prefill path another kernel takes those).
-        // On the decode path a tile above 8 rows takes about twice as long as a small one (it restages its activations
-        // on the way). (Moving the last, partial tile of an expert away from its full tiles measured 2-3 % slower at
-        // prefill: it then finds none of the expert's weights in L2.)
+        // Tiles above kPackSmallTileRows rows first, then the rest, each group in expert order. On the decode path a
+        // large tile takes about twice as long as a small one (it restages its activations on the way), so the few
+        // of them start with the launch instead of stretching its tail. (Splitting further - full tiles of all experts
+        // first, then the partial ones - measured 2-3 % slower at prefill: a partial tile then runs far from its
+        // expert's full tiles and finds none of the weights in L2.)
         const uint32_t tm = (uint32_t)tile_m;
         const uint32_t nt = (count + tm - 1) / tm;
         const uint32_t last_rows = count - (nt ? (nt - 1) * tm : 0);           // rows of the expert's last tile
         const uint32_t n_big = nt == 0 ? 0 : (nt - 1) + (last_rows > kPackSmallTileRows ? 1u : 0u);
-        const uint32_t quarter = (tm + 3) / 4;
-        // class of this expert's tiles above kPackSmallTileRows rows (all of them share it)
-        const uint32_t cls = nt > 1 || count == tm ? 0u : 1u + (4u - (count + quarter - 1) / quarter);
-        // Two scans: the tiles of class 0 (an expert can have hundreds), and - one 64-bit word - the five counters of
-        // the other classes, each 0 or 1 per expert and at most 1024 in total: 12 bits apiece.
-        uint32_t total0;
-        const uint32_t base0 = block_excl_scan(cls == 0 ? n_big : 0u, &total0, sm);
-        const uint32_t small_here = nt - n_big; // 0 or 1
-        const uint64_t word = ((cls >= 1 && cls <= 4 && n_big) ? 1ull << (12 * (cls - 1)) : 0ull) | ((uint64_t)small_here << 48);
-        uint64_t total_w;
-        const uint64_t base_w = block_excl_scan64(word, &total_w, (uint64_t *)sm);
-        uint32_t pos_cls = base0, run = total0;
-#pragma unroll
-        for (uint32_t c = 1; c <= 4; ++c) {
-            if (c == cls) pos_cls = run + (uint32_t)(base_w >> (12 * (c - 1)) & 0xfffu);
-            run += (uint32_t)(total_w >> (12 * (c - 1)) & 0xfffu);
-        }
-        const uint32_t small_base = (uint32_t)(base_w >> 48 & 0xfffu);
-        const uint32_t total_big = run, total_small = (uint32_t)(total_w >> 48 & 0xfffu);
+        uint32_t total_big, total_small;
+        const uint32_t big_base = block_excl_scan(n_big, &total_big, sm);
+        const uint32_t small_base = block_excl_scan(nt - n_big, &total_small, sm);
         for (uint32_t j = 0; j < nt; ++j) {
             Tile t;
             t.expert = (uint32_t)e;
@@ -166,7 +117,7 @@ __device__ uint32_t emit_segments(uint32_t count, int e, int E, size_t n, int ti
             uint32_t left = count - j * tm;
             t.nrows = left < tm ? left : tm;
             t.flags = 0;
-            const uint32_t pos = j < n_big ? pos_cls + j : total_big + small_base;
+            const uint32_t pos = j < n_big ? big_base + j : total_big + small_base;
             o.tiles[nt_dense + pos] = t;
         }
         const uint32_t tf = total_big + total_small;
@@ -217,7 +168,7 @@ __device__ __forceinline__ void pack_fused_body(const PackOut &o, uint32_t e, bo
 __global__ __launch_bounds__(kPackThreads) void pack_fused_kernel(PackOut o, const uint32_t *__restrict__ idx,
                                                                   uint32_t n, int K, int E, int tile_m) {
     extern __shared__ uint32_t pack_sm[]; // hist[kPackWaves][E]
-    __shared__ __attribute__((aligned(8))) uint32_t scan_sm[2 * (kPackWaves + 1)]; // also scanned as 64-bit words
+    __shared__ uint32_t scan_sm[kPackWaves + 1];
     const bool active = threadIdx.x < n;
     const uint32_t e = active ? idx[threadIdx.x] : 0u;
     pack_fused_body(o, e, active, n, K, E, tile_m, pack_sm, scan_sm);
@@ -253,7 +204,7 @@ __global__ __launch_bounds__(kScatterWaves * 64) void pack_hist_kernel(uint32_t 
 
 __global__ __launch_bounds__(kPackThreads) void pack_scan_kernel(PackOut o, uint32_t *__restrict__ cnt,
                                                                  size_t n, int E, int n_sub, int tile_m) {
-    __shared__ __attribute__((aligned(8))) uint32_t scan_sm[2 * (kPackWaves + 1)]; // also scanned as 64-bit words
+    __shared__ uint32_t scan_sm[kPackWaves + 1];
     const int tid = (int)threadIdx.x;
     uint32_t count = 0;
     if (tid < E) {
