@@ -34,7 +34,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 COPY_PROBE_BYTES = 256 << 20  # --copy-probe: bytes read (and written) by each calibration copy
-COUNTERS_FILE = os.path.join(ROOT, "profiles", "counters.json")   # written from the rocprofv3 --pmc summaries
+COUNTERS_FILE = os.path.join(ROOT, "profiles", "counters.json")   # written by dmlx_amd/rocprof_summary.py from rocprofv3 --pmc output
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 SMALL_PATH_AVG_ROWS = 16     # at most this many rows per resident expert on average: weight-streaming kernel (kSkinnyAvgRows in csrc/layer.hip)
@@ -277,6 +277,8 @@ def describe(torch, wl, config, timing, U, counts, steps, warmup, counters):
     if "mfma_busy" in rec:
         roof["mfma_busy"] = rec["mfma_busy"]              # SQ_VALU_MFMA_BUSY_CYCLES / (SIMDs x kernel cycles)
         roof["valu_per_mfma"] = rec.get("valu_per_mfma")  # other vector instructions per MFMA
+    if "wait_share" in rec:
+        roof["wait_share"] = rec["wait_share"]            # SQ_WAIT_INST_ANY / SQ_WAVE_CYCLES
     if rec:
         roof["counters_from"] = rec.get("source")
     launches = (["qgemm_skinny_kernel (gate/up and down tiles in one launch)"] if paired else ["qgemm_skinny_kernel"] if decode else

@@ -83,23 +83,10 @@ def read_counters(dirs):
     return agg
 
 
-def counters(args):
-    agg = read_counters(args.dirs)
-    out = [f"# {args.title}", "", "commands (one MI355X, one rocprofv3 run each):", ""] + [f"    {c}" for c in args.command] + [
-        "", "Per dispatch, over all dispatches of the kernel in the runs (pre-run, warm-up, timed and stage-timed windows).",
-        "FETCH_SIZE / WRITE_SIZE are KiB; COPY = the runtime's device-copy kernel; its largest dispatches are the 256 MiB copies of --copy-probe, the scale of",
-        "those two counters; SQ_ACTIVE_* / SQ_WAIT_* / SQ_WAVE_CYCLES count units of four cycles; GRBM_GUI_ACTIVE is summed",
-        "over the 8 XCDs.", "",
-        f"{'kernel':52s} {'workgroups':>10s} {'counter':30s} {'n':>5s} {'avg':>16s} {'min':>16s} {'max':>16s}"]
-    for (k, wgs, c), v in sorted(agg.items()):
-        out.append(f"{k[:50]:52s} {wgs:10d} {c:30s} {len(v):5d} {sum(v) / len(v):16.1f} {min(v):16.1f} {max(v):16.1f}")
-    print("\n".join(out))
+def derived(agg, kernel, min_workgroups=0):
+    """The figures bench.py quotes for one kernel, from the counters that are present."""
 
-
-def to_json(args):
-    agg = read_counters(args.dirs)
-
-    def avg(counter, kernel=None, copy=False):
+    def avg(counter, copy=False):
         vals = []
         for (k, wgs, c), v in agg.items():
             if c != counter:
@@ -107,31 +94,61 @@ def to_json(args):
             if copy:
                 if k == "COPY":
                     vals += v
-            elif kernel in k and wgs >= args.min_workgroups:
+            elif kernel in k and wgs >= min_workgroups:
                 vals += v
         if copy and vals:   # the --copy-probe copies are the largest device copies of a run: those within 2 % of the top
             vals = [x for x in vals if x >= 0.98 * max(vals)]
         return sum(vals) / len(vals) if vals else None
 
     rec = {}
-    fetch, write = avg("FETCH_SIZE", args.kernel), avg("WRITE_SIZE", args.kernel)
+    fetch, write = avg("FETCH_SIZE"), avg("WRITE_SIZE")
     if fetch is not None and write is not None:
         cf, cw = avg("FETCH_SIZE", copy=True), avg("WRITE_SIZE", copy=True)
-        if not cf or not cw:
-            sys.exit("no --copy-probe copies in the counter runs: FETCH_SIZE / WRITE_SIZE cannot be scaled")
-        f_scale, w_scale = COPY_BYTES / cf, COPY_BYTES / cw     # bytes per counter unit
-        rec["traffic_bytes"] = int(round(fetch * f_scale + write * w_scale))
-        rec["fetch_scale"] = round(f_scale / 1024, 3)           # in units of KiB: 2.0 = the counter reads half the bytes
-        rec["write_scale"] = round(w_scale / 1024, 3)
-    busy, gui = avg("SQ_VALU_MFMA_BUSY_CYCLES", args.kernel), avg("GRBM_GUI_ACTIVE", args.kernel)
+        if cf and cw:
+            f_scale, w_scale = COPY_BYTES / cf, COPY_BYTES / cw     # bytes per counter unit
+            rec["traffic_bytes"] = int(round(fetch * f_scale + write * w_scale))
+            rec["fetch_scale"] = round(f_scale / 1024, 3)           # in KiB: 2.0 = the counter reads half the bytes
+            rec["write_scale"] = round(w_scale / 1024, 3)
+    busy, gui = avg("SQ_VALU_MFMA_BUSY_CYCLES"), avg("GRBM_GUI_ACTIVE")
     if busy is not None and gui:
         rec["mfma_busy"] = round(busy / (N_SIMD * gui / N_XCD), 3)
-    valu, mfma = avg("SQ_INSTS_VALU", args.kernel), avg("SQ_INSTS_MFMA", args.kernel)
+    valu, mfma = avg("SQ_INSTS_VALU"), avg("SQ_INSTS_MFMA")
     if valu is not None and mfma:
         rec["valu_per_mfma"] = round((valu - mfma) / mfma, 2)
-    wait, wave = avg("SQ_WAIT_INST_ANY", args.kernel), avg("SQ_WAVE_CYCLES", args.kernel)
+    wait, wave = avg("SQ_WAIT_INST_ANY"), avg("SQ_WAVE_CYCLES")
     if wait is not None and wave:
         rec["wait_share"] = round(wait / wave, 3)
+    return rec
+
+
+def counters(args):
+    agg = read_counters(args.dirs)
+    out = [f"# {args.title}", "", "commands (one MI355X, one rocprofv3 run each):", ""] + [f"    {c}" for c in args.command] + [
+        "", "Per dispatch, over all dispatches of the kernel in the runs (pre-run, warm-up, timed and stage-timed windows); kernels",
+        f"whose name contains '{args.kernels}'. FETCH_SIZE / WRITE_SIZE are KiB; COPY = the runtime's device-copy kernel, whose",
+        "largest dispatches are the 256 MiB copies of --copy-probe (the scale of those two counters); SQ_ACTIVE_* / SQ_WAIT_* /",
+        "SQ_WAVE_CYCLES count units of four cycles; GRBM_GUI_ACTIVE is summed over the 8 XCDs.", "",
+        f"{'kernel':52s} {'workgroups':>10s} {'counter':30s} {'n':>5s} {'avg':>16s} {'min':>16s} {'max':>16s}"]
+    names = []
+    for (k, wgs, c), v in sorted(agg.items()):
+        if args.kernels not in k and not (k == "COPY" and max(v) >= 1024 and c in ("FETCH_SIZE", "WRITE_SIZE")):
+            continue
+        out.append(f"{k[:50]:52s} {wgs:10d} {c:30s} {len(v):5d} {sum(v) / len(v):16.1f} {min(v):16.1f} {max(v):16.1f}")
+        if k != "COPY" and (k, wgs) not in names:
+            names.append((k, wgs))
+    out += ["", "Derived per kernel and launch size (what profiles/counters.json holds): traffic_bytes = FETCH_SIZE x fetch_scale +",
+            "WRITE_SIZE x write_scale (scales = bytes of a --copy-probe copy / its counter reading, in KiB); mfma_busy =",
+            "SQ_VALU_MFMA_BUSY_CYCLES / (1024 SIMDs x GRBM_GUI_ACTIVE / 8); valu_per_mfma = (SQ_INSTS_VALU - SQ_INSTS_MFMA) /",
+            "SQ_INSTS_MFMA; wait_share = SQ_WAIT_INST_ANY / SQ_WAVE_CYCLES.", ""]
+    for k, wgs in names:
+        sub = {key: v for key, v in agg.items() if key[0] == "COPY" or (key[0] == k and key[1] == wgs)}
+        out.append(f"{k[:50]:52s} {wgs:10d} {json.dumps(derived(sub, k))}")
+    print("\n".join(out))
+
+
+def to_json(args):
+    agg = read_counters(args.dirs)
+    rec = derived(agg, args.kernel, args.min_workgroups)
     if not rec:
         sys.exit(f"no counters of a kernel matching {args.kernel!r} in {args.dirs}")
     rec["source"] = args.source
@@ -160,6 +177,7 @@ def main():
         p.add_argument("dirs", nargs="+")
         p.add_argument("--title", required=True)
         p.add_argument("--command", action="append", default=[])
+        p.add_argument("--kernels", default="gemm", help="counters: list only kernels whose name contains this")
     p = sub.add_parser("json")
     p.add_argument("config", type=int)
     p.add_argument("stage")
