@@ -120,3 +120,33 @@ def test_prefill_configs_every_row_against_float64(dmoe, orc, ws, config):
     assert err < OUT_TOL, (wl.name, "kernels against float64 over every row", err)
     assert float(row_err.max()) < ROW_TOL, (wl.name, "per-row error over every row", worst, float(row_err[worst]))
     layer.close()
+
+
+def test_prefill_full_size_is_linear_in_the_routing_weights_and_blind_to_the_order_of_k(dmoe, ws):
+    """Size-independent properties at the full 8192-token ragged prefill (no oracle needed). With the routing weight
+    applied in the combine (the provider form), doubling every weight doubles the f32 sum before its one rounding, so
+    the bf16 output doubles EXACTLY; a zero weight removes that expert's term exactly (the row is still computed); and
+    rotating each token's K (index, weight) pairs permutes the packed rows inside their segments without changing any
+    token's set of experts, so the outputs may differ only by the f32 summation order of the combine: one bf16 step."""
+    wl = workloads.make(3)
+    layer = _layer(dmoe, wl)
+    idx, w = dmoe.gate_route(wl.scores, wl.bias, wl.resident_mask, wl.K, wl.renorm, wl.route_scale)
+    out = layer.forward(wl.x, idx, w, ws).clone()
+    twice = layer.forward(wl.x, idx, (2.0 * w).contiguous(), ws)
+    assert torch.equal((2.0 * out.float()).to(torch.bfloat16), twice), "doubling the routing weights must double the output bits exactly"
+    # drop the last column's weight: the same as a forward over the first K - 1 columns' terms
+    w_cut = w.clone()
+    w_cut[:, -1] = 0.0
+    cut = layer.forward(wl.x, idx, w_cut, ws).float()
+    y = layer.forward_no_scores(wl.x, idx, ws).float()                # [T, K, D] expert outputs, bf16-rounded
+    want_cut = (y[:, :-1] * w[:, :-1, None]).sum(dim=1)
+    scale = float(want_cut.abs().max())
+    assert float((cut - want_cut).abs().max()) <= 2.0 ** -7 * scale, "zero weight must remove exactly that expert's term"
+    # rotate the K columns of every token
+    idx_r, w_r = torch.roll(idx, 1, dims=1).contiguous(), torch.roll(w, 1, dims=1).contiguous()
+    rot = layer.forward(wl.x, idx_r, w_r, ws).float()
+    gap = (rot - out.float()).abs()
+    allowed = torch.maximum(rot.abs(), out.float().abs()) * 2.0 ** -7 + 1e-6 * float(out.float().abs().max())
+    assert bool((gap <= allowed).all()), float((gap - allowed).max())
+    ws.check()
+    layer.close()

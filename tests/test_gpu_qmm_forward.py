@@ -550,6 +550,22 @@ def test_layer_seeded_random_shapes(dmoe, orc, ws, fmt):
         _check_layer(dmoe, orc, ws, wl)
 
 
+@pytest.mark.parametrize("fmt,T", [("affine4", 24), ("affine4", 330), ("mxfp4", 330)])
+def test_layer_with_a_hidden_size_that_is_not_a_power_of_two(dmoe, orc, ws, fmt, T):
+    """D = 7168 (112 reduction steps of 64: not a multiple of the kernels' ring rounds, unroll trips or span counts), F =
+    2048, 16 experts top-4 with a shared expert: the decode kernel at 24 tokens (6 rows per expert, partial last round),
+    the matrix-core kernels at 330 (82 rows per expert, 28 whole trips of the activation ring)."""
+    D, F, E, K = 7168, 2048, 16, 4
+    g = torch.Generator(device="cuda").manual_seed(7000 + T)
+    x = torch.randn((T, D), generator=g, device="cuda").to(torch.bfloat16)
+    scores = torch.sigmoid(torch.randn((T, E), generator=g, device="cuda"))
+    shared = (_stack(fmt, 1, F, D, 711), _stack(fmt, 1, F, D, 712), _stack(fmt, 1, D, F, 713))
+    wl = workloads.Workload(f"D=7168 {fmt} T={T}", T, D, F, E, E, K, x, scores, None, None, None, True, 2.5,
+                            _stack(fmt, E, F, D, 701), _stack(fmt, E, F, D, 702), _stack(fmt, E, D, F, 703), shared,
+                            swiglu_limit=7.0)
+    _check_layer(dmoe, orc, ws, wl)
+
+
 def test_forward_edge_cases(dmoe, orc, ws):
     wl = workloads.make(1, scale=0.125)
     layer = dmoe.Layer(wl.D, wl.F, wl.K, wl.gate, wl.up, wl.down, swiglu_limit=wl.swiglu_limit, shared=wl.shared)
