@@ -146,6 +146,56 @@ def time_gate(torch, steps, windows):
     return out
 
 
+def time_gather_qmm(torch, steps, windows):
+    """The leaf operator on its own (quantize_mod.gatherQmm, call shape deepseek_v4.zig:976): the gate and the down
+    projection of configuration 1 with that step's routing (384 rows over the live experts), three ways of holding the
+    weights: the caller's MLX-layout arrays as they are (dmoe_gather_qmm), the same call with the workspace's opt-in
+    cache of re-ordered copies, and a stack made resident once (dmoe_gather_qmm_resident). GB/s of the live experts'
+    weight bytes over the whole call (packing launch included)."""
+    from dmlx_amd import capi, workloads
+
+    wl = workloads.make(1, device="cuda")
+    ws = capi.Workspace()
+    idx, _ = capi.gate_route(wl.scores, wl.bias, None, wl.K, wl.renorm, wl.route_scale)
+    rhs = idx.reshape(-1).contiguous()
+    live = int(torch.unique(rhs).numel())
+    x_d = wl.x.repeat_interleave(wl.K, 0).contiguous()
+    g = torch.Generator(device="cuda").manual_seed(2)
+    x_f = torch.randn((x_d.shape[0], wl.F), generator=g, device="cuda").to(torch.bfloat16)
+    out = []
+    for name, q, x in (("gate_proj [E, F, D]", wl.gate, x_d), ("down_proj [E, D, F]", wl.down, x_f)):
+        per = q.nbytes() // q.n_mats
+        res = capi.ResidentWeight(q)
+        calls = {"mlx_layout": lambda: capi.gather_qmm(x, q, rhs, ws),
+                 "resident": lambda: res.gather_qmm(x, rhs, ws)}
+        row = {"projection": name, "rows": int(rhs.numel()), "live_experts": live, "weight_bytes": live * per}
+        for key in ("mlx_layout", "resident", "mlx_layout_cached"):
+            if key == "mlx_layout_cached":
+                ws.set_weight_cache(True)
+                fn = calls["mlx_layout"]
+            else:
+                fn = calls[key]
+            for _ in range(steps):
+                fn()
+            torch.cuda.synchronize()
+            ms = []
+            for _ in range(windows):
+                t0 = time.perf_counter()
+                for _ in range(steps):
+                    fn()
+                torch.cuda.synchronize()
+                ms.append((time.perf_counter() - t0) * 1e3 / steps)
+            m = statistics.median(ms)
+            row[key] = {"ms": m, "GBs": live * per / (m * 1e-3) / 1e9, "frac_of_hbm_peak": live * per / (m * 1e-3) / 1e9 / HBM_PEAK_GBS}
+            if key == "mlx_layout_cached":
+                ws.set_weight_cache(False)
+        res.close()
+        out.append(row)
+    ws.check()
+    ws.close()
+    return out
+
+
 def run_config(torch, config, steps, warmup, windows, settle_ms, copy_probe=False, score_before_down=False):
     """Builds configuration `config`, times it as the module docstring says and returns (workload, timing, analysis
     inputs). The layer and its workspace are released before returning."""
@@ -327,7 +377,7 @@ def main():
                     help="1: routing weight applied to the activation before the down projection (DSV4SwitchGLU.forward); "
                          "0: to the expert outputs (expert provider paths)")
     ap.add_argument("--no-prefill", action="store_true", help="with --config 1: do not also time configurations 3, 2 and 4")
-    ap.add_argument("--no-gate", action="store_true", help="do not also time the router (DSV4Gate.forward) in front of the step")
+    ap.add_argument("--no-gate", action="store_true", help="do not also time the router (DSV4Gate.forward) in front of the step and the gatherQmm leaf operator")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-peaks", action="store_true", help="skip the library copy / GEMM reference measurements")
     ap.add_argument("--copy-probe", action="store_true",
@@ -380,6 +430,7 @@ def main():
             torch.cuda.empty_cache()
     if not args.no_gate:
         result["gate"] = time_gate(torch, args.steps, args.windows)
+        result["gather_qmm"] = time_gather_qmm(torch, args.steps, args.windows)
     print(json.dumps(result))
 
 
