@@ -151,6 +151,10 @@ struct PackOut {
     // optional device counter: +1 for every expert id >= E met (such a row is packed under expert E - 1 so that every
     // access stays in bounds; the host learns about it from dmoe_workspace_check)
     uint32_t *bad_ids = nullptr;
+    // optional map applied to every id before it is packed (global expert id -> resident slot; an id outside the
+    // table maps to slot 0 like an expert that is not loaded)
+    const int32_t *remap = nullptr;
+    uint32_t n_remap = 0;
 };
 
 inline int pack_max_tiles(size_t n, int E, int tile_m) {

@@ -185,7 +185,7 @@ static bool use_small_path(size_t rows, int n_experts, const QView &b) {
     return qgemm_skinny_supports(b) && rows <= (size_t)kSkinnyAvgRows * (size_t)n_experts;
 }
 struct FwdLayout {
-    size_t slot_idx, order, inv, token, sorted_e, counts, offsets, live, n_live, tiles, n_tiles, tile_done, scratch;
+    size_t order, inv, token, sorted_e, counts, offsets, live, n_live, tiles, n_tiles, tile_done, scratch;
     size_t h, y, sh_h, sh_y, total;
     int max_tiles, tile_m;
     bool small;
@@ -203,7 +203,6 @@ static FwdLayout forward_layout(const Layer *L, int T, bool with_shared = true) 
     f.fold = with_shared && f.small && L->shared_folded;
     const size_t rows = n + (f.fold ? (size_t)T : 0); // sorted rows of the GEMMs
     f.max_tiles = pack_max_tiles(n, L->E, f.tile_m) + (f.fold ? ceil_div(T, f.tile_m) : 0);
-    f.slot_idx = b.take(n * 4);
     f.order = b.take(rows * 4);
     f.inv = b.take(n * 4);
     f.token = b.take(rows * 4);
@@ -251,7 +250,8 @@ static int run_gemm(const GemmArgs &g, bool small, hipStream_t st, int small_row
 
 // routed experts on slot ids: fills ws->y ([T*K, D] bf16 in flat (t,k) order) or `y_out` when given
 static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, const uint16_t *d_x,
-                          const uint32_t *d_slots, const float *d_scores, int T, uint16_t *y_out, hipStream_t st) {
+                          const uint32_t *d_ids, bool remap, const float *d_scores, int T, uint16_t *y_out,
+                          hipStream_t st) {
     size_t n = (size_t)T * L->K;
     PackOut po;
     po.order = at<uint32_t>(w, f.order);
@@ -272,7 +272,11 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     po.tile_done = at<uint32_t>(w, f.tile_done);
     po.n_done = (uint32_t)f.max_tiles;
     po.bad_ids = w->flags + 1;
-    DMOE_TRY(launch_pack(po, d_slots, n, L->K, L->E, f.tile_m, at<void>(w, f.scratch), st));
+    if (remap) { // global expert ids -> resident slots, inside the packing kernels
+        po.remap = L->remap;
+        po.n_remap = (uint32_t)L->n_total;
+    }
+    DMOE_TRY(launch_pack(po, d_ids, n, L->K, L->E, f.tile_m, at<void>(w, f.scratch), st));
     DMOE_TRY(stage_end(w, DMOE_STAGE_PACK, st));
 
     GemmArgs gu;
@@ -623,14 +627,8 @@ static int forward_common(uint16_t *d_out, uint16_t *y_out, Layer *L, const uint
     Workspace *w = nullptr;
     DMOE_TRY(workspace_reserve(ws, f.total, &w));
     w->last_with_shared = with_shared && !y_out;
-    const uint32_t *slots = d_indices;
-    size_t n = (size_t)T * L->K;
     DMOE_TRY(stage_begin(w, DMOE_STAGE_PACK, st));
-    if (apply_remap && L->remap) {
-        uint32_t *sl = at<uint32_t>(w, f.slot_idx);
-        DMOE_TRY(dmoe_remap_indices(sl, L->remap, d_indices, n, L->n_total, s));
-        slots = sl;
-    }
+    const bool remap = apply_remap && L->remap;
     // The shared expert does not depend on the routing: it runs on the workspace's side stream, forked
     // here and joined before the combine, so its two small dense GEMMs overlap pack and the routed GEMMs.
     // The routed launches are enqueued first: they are the critical path, and the host has all of their run
@@ -642,7 +640,7 @@ static int forward_common(uint16_t *d_out, uint16_t *y_out, Layer *L, const uint
         DMOE_TRY(side_stream_ready(w));
         DMOE_HIP(hipEventRecord(w->fork, st));
     }
-    DMOE_TRY(routed_forward(L, w, f, d_x, slots, d_scores, T, y_out, st));
+    DMOE_TRY(routed_forward(L, w, f, d_x, d_indices, remap, d_scores, T, y_out, st));
     if (side_shared) {
         DMOE_HIP(hipStreamWaitEvent(w->side, w->fork, 0));
         DMOE_TRY(stage_begin(w, DMOE_STAGE_SHARED, w->side));

@@ -57,6 +57,12 @@ __device__ __forceinline__ uint64_t match_expert(uint32_t e, bool active, int nb
     return peers;
 }
 
+// the id as it is packed: through the optional slot map
+__device__ __forceinline__ uint32_t packed_id(const PackOut &o, uint32_t e) {
+    if (!o.remap) return e;
+    return e < o.n_remap ? (uint32_t)o.remap[e] : 0u;
+}
+
 __device__ __forceinline__ int log2_ceil(int E) {
     int b = 0;
     while ((1 << b) < E) ++b;
@@ -170,15 +176,14 @@ __global__ __launch_bounds__(kPackThreads) void pack_fused_kernel(PackOut o, con
     extern __shared__ uint32_t pack_sm[]; // hist[kPackWaves][E]
     __shared__ uint32_t scan_sm[kPackWaves + 1];
     const bool active = threadIdx.x < n;
-    const uint32_t e = active ? idx[threadIdx.x] : 0u;
+    const uint32_t e = active ? packed_id(o, idx[threadIdx.x]) : 0u;
     pack_fused_body(o, e, active, n, K, E, tile_m, pack_sm, scan_sm);
 }
 
 // ---- three launches, any n --------------------------------------------------------------------------------
-__global__ __launch_bounds__(kScatterWaves * 64) void pack_hist_kernel(uint32_t *__restrict__ cnt,
+__global__ __launch_bounds__(kScatterWaves * 64) void pack_hist_kernel(PackOut o, uint32_t *__restrict__ cnt,
                                                                        const uint32_t *__restrict__ idx,
-                                                                       size_t n, int E, int n_sub,
-                                                                       uint32_t *__restrict__ bad_ids) {
+                                                                       size_t n, int E, int n_sub) {
     extern __shared__ uint32_t pack_sm[]; // hist[kScatterWaves][E]
     const int tid = (int)threadIdx.x, lane = lane_id(), wave = tid >> 6;
     for (int i = tid; i < kScatterWaves * E; i += kScatterWaves * 64) pack_sm[i] = 0;
@@ -188,9 +193,9 @@ __global__ __launch_bounds__(kScatterWaves * 64) void pack_hist_kernel(uint32_t 
         for (int g = 0; g < kSubGroups; ++g) {
             size_t i = (size_t)sub * kSubRows + (size_t)g * 64 + lane;
             if (i < n) {
-                uint32_t e = idx[i];
+                uint32_t e = packed_id(o, idx[i]);
                 if (e >= (uint32_t)E) { // counted here once; the scatter kernel clamps the same way
-                    if (bad_ids) atomicAdd(bad_ids, 1u);
+                    if (o.bad_ids) atomicAdd(o.bad_ids, 1u);
                     e = (uint32_t)E - 1;
                 }
                 atomicAdd(&pack_sm[wave * E + e], 1u);
@@ -243,7 +248,7 @@ __global__ __launch_bounds__(kScatterWaves * 64) void pack_scatter_kernel(PackOu
     for (int g = 0; g < kSubGroups; ++g) {
         size_t i = (size_t)sub * kSubRows + (size_t)g * 64 + lane;
         const bool active = wave_on && i < n;
-        uint32_t e = active ? idx[i] : 0u;
+        uint32_t e = active ? packed_id(o, idx[i]) : 0u;
         if (active && e >= (uint32_t)E) e = (uint32_t)E - 1;
         uint64_t peers = match_expert(e, active, nbits);
         uint32_t base = 0, rank = 0;
@@ -283,7 +288,7 @@ int launch_pack(const PackOut &o, const uint32_t *d_idx, size_t n, int K, int E,
     int n_sub = (int)((n + kSubRows - 1) / kSubRows);
     dim3 grid((unsigned)ceil_div(n_sub, kScatterWaves)), block(kScatterWaves * 64);
     size_t lds = sizeof(uint32_t) * (size_t)kScatterWaves * E;
-    hipLaunchKernelGGL(pack_hist_kernel, grid, block, lds, st, cnt, d_idx, n, E, n_sub, o.bad_ids);
+    hipLaunchKernelGGL(pack_hist_kernel, grid, block, lds, st, o, cnt, d_idx, n, E, n_sub);
     DMOE_LAUNCH_CHECK();
     hipLaunchKernelGGL(pack_scan_kernel, dim3(1), dim3(kPackThreads), 0, st, o, cnt, n, E, n_sub, tile_m);
     DMOE_LAUNCH_CHECK();
