@@ -19,31 +19,50 @@ constexpr int kSubRows = 64 * kSubGroups;       // 256 rows per sub-chunk
 constexpr int kScatterWaves = 4;                // wavefronts per block in the multi-launch path
 constexpr uint32_t kPackSmallTileRows = 8;      // tiles of at most this many rows go behind the larger ones in the tile list
 
-// exclusive scan of one value per thread across a 1024-thread block; *total gets the block sum
-__device__ uint32_t block_excl_scan(uint32_t v, uint32_t *total, uint32_t *sm /*[kPackWaves + 1]*/) {
-    const int lane = lane_id(), wave = (int)(threadIdx.x >> 6);
-    uint32_t incl = v;
+// one step of a wavefront-wide prefix sum: v += the value `CTRL` selects (0 where it selects nothing or the row is masked)
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t scan_dpp_step(uint32_t v) {
+    return v + (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+// inclusive prefix sum inside each row of 16 lanes
+__device__ __forceinline__ uint32_t row_incl_scan(uint32_t v) {
+    v = scan_dpp_step<0x111, 0xf>(v); // row_shr:1
+    v = scan_dpp_step<0x112, 0xf>(v); // row_shr:2
+    v = scan_dpp_step<0x114, 0xf>(v); // row_shr:4
+    v = scan_dpp_step<0x118, 0xf>(v); // row_shr:8
+    return v;
+}
+// inclusive prefix sum over the 64 lanes (all of them active)
+__device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v) {
+    v = row_incl_scan(v);
+    v = scan_dpp_step<0x142, 0xa>(v); // row_bcast:15 into rows 1 and 3: the total of the row before
+    v = scan_dpp_step<0x143, 0xc>(v); // row_bcast:31 into rows 2 and 3: the total of rows 0 and 1
+    return v;
+}
+
+// exclusive scans of NV values per thread across a 1024-thread block in one pass; total[k] gets the block sums.
+// One barrier: every wavefront adds up the 16 wavefront totals for itself. `sm` holds kPackWaves * NV words that nothing
+// else touches (a kernel scans once).
+template <int NV>
+__device__ __forceinline__ void block_excl_scan(const uint32_t (&v)[NV], uint32_t (&excl)[NV], uint32_t (&total)[NV],
+                                                uint32_t *sm) {
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    uint32_t incl[NV];
 #pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        uint32_t o = (uint32_t)__shfl_up((int)incl, off, 64);
-        if (lane >= off) incl += o;
+    for (int k = 0; k < NV; ++k) {
+        incl[k] = wave_incl_scan(v[k]);
+        if (lane == 63) sm[wave * NV + k] = incl[k];
     }
-    __syncthreads(); // sm may still be read from a previous call
-    if (lane == 63) sm[wave] = incl;
     __syncthreads();
-    if (wave == 0) {
-        uint32_t t = lane < kPackWaves ? sm[lane] : 0u, ti = t;
 #pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            uint32_t o = (uint32_t)__shfl_up((int)ti, off, 64);
-            if (lane >= off) ti += o;
-        }
-        if (lane < kPackWaves) sm[lane] = ti - t;
-        if (lane == 63) sm[kPackWaves] = ti;
+    for (int k = 0; k < NV; ++k) {
+        const uint32_t t = row_incl_scan(lane < kPackWaves ? sm[lane * NV + k] : 0u); // lanes 0..15 = one row
+        const uint32_t upto = (uint32_t)__builtin_amdgcn_readlane((int)t, wave);      // wavefronts 0..wave
+        const uint32_t mine = (uint32_t)__builtin_amdgcn_readlane((int)incl[k], 63);  // this wavefront's total
+        total[k] = (uint32_t)__builtin_amdgcn_readlane((int)t, kPackWaves - 1);
+        excl[k] = upto - mine + incl[k] - v[k];
     }
-    __syncthreads();
-    *total = sm[kPackWaves];
-    return sm[wave] + incl - v;
 }
 
 // lanes of this wavefront that hold the same expert id (only among `active` lanes)
@@ -71,24 +90,32 @@ __device__ __forceinline__ int log2_ceil(int E) {
 
 // phase 2 body shared by the fused and the stand-alone scan kernel. `count` is this thread's expert total.
 __device__ uint32_t emit_segments(uint32_t count, int e, int E, size_t n, int tile_m, const PackOut &o,
-                                  uint32_t *sm) {
-    uint32_t total;
-    uint32_t off = block_excl_scan(count, &total, sm);
+                                  uint32_t *sm /*[4 * kPackWaves]*/) {
+    // Tiles above kPackSmallTileRows rows first, then the rest, each group in expert order. On the decode path a
+    // large tile takes about twice as long as a small one (it restages its activations on the way), so the few
+    // of them start with the launch instead of stretching its tail. (Splitting further - full tiles of all experts
+    // first, then the partial ones - measured 2-3 % slower at prefill: a partial tile then runs far from its
+    // expert's full tiles and finds none of the weights in L2.)
+    const uint32_t tm = tile_m > 0 ? (uint32_t)tile_m : 1u;
+    const uint32_t nt = tile_m > 0 ? (count + tm - 1) / tm : 0u;
+    const uint32_t last_rows = count - (nt ? (nt - 1) * tm : 0);           // rows of the expert's last tile
+    const uint32_t n_big = nt == 0 ? 0 : (nt - 1) + (last_rows > kPackSmallTileRows ? 1u : 0u);
+    // everything below depends on the expert's count only: segment start, rank among the live experts, first large
+    // and first small tile come out of one scan
+    const uint32_t in[4] = {count, count > 0 ? 1u : 0u, n_big, nt - n_big};
+    uint32_t ex[4], tot[4];
+    block_excl_scan<4>(in, ex, tot, sm);
+    const uint32_t off = ex[0];
     if (e < E) {
         if (o.counts) o.counts[e] = count;
         if (o.offsets) o.offsets[e] = off;
     }
     if (e == 0 && o.offsets) o.offsets[E] = (uint32_t)n;
-    if (o.live || o.n_live) {
-        uint32_t lt;
-        uint32_t lb = block_excl_scan(count > 0 ? 1u : 0u, &lt, sm);
-        if (count > 0 && o.live) o.live[lb] = (uint32_t)e;
-        if (e == 0 && o.n_live) *o.n_live = lt;
-    }
+    if (count > 0 && o.live) o.live[ex[1]] = (uint32_t)e;
+    if (e == 0 && o.n_live) *o.n_live = tot[1];
     for (uint32_t i = threadIdx.x; i < o.n_done; i += blockDim.x) o.tile_done[i] = 0;
     // the folded always-on expert: identity rows behind the routed ones, its tiles ahead of the routed tiles
-    const uint32_t dense_m = tile_m > 0 ? (uint32_t)tile_m : 1u;
-    const uint32_t nt_dense = (o.dense_rows + dense_m - 1) / dense_m;
+    const uint32_t nt_dense = (o.dense_rows + tm - 1) / tm;
     for (uint32_t i = threadIdx.x; i < o.dense_rows; i += blockDim.x) {
         o.order[n + i] = (uint32_t)n + i;
         if (o.token) o.token[n + i] = i;
@@ -98,24 +125,13 @@ __device__ uint32_t emit_segments(uint32_t count, int e, int E, size_t n, int ti
         for (uint32_t j = threadIdx.x; j < nt_dense; j += blockDim.x) {
             Tile t;
             t.expert = o.dense_expert;
-            t.row0 = (uint32_t)n + j * dense_m;
-            uint32_t left = o.dense_rows - j * dense_m;
-            t.nrows = left < dense_m ? left : dense_m;
+            t.row0 = (uint32_t)n + j * tm;
+            uint32_t left = o.dense_rows - j * tm;
+            t.nrows = left < tm ? left : tm;
             t.flags = kTileDense;
             o.tiles[j] = t;
         }
-        // Tiles above kPackSmallTileRows rows first, then the rest, each group in expert order. On the decode path a
-        // large tile takes about twice as long as a small one (it restages its activations on the way), so the few
-        // of them start with the launch instead of stretching its tail. (Splitting further - full tiles of all experts
-        // first, then the partial ones - measured 2-3 % slower at prefill: a partial tile then runs far from its
-        // expert's full tiles and finds none of the weights in L2.)
-        const uint32_t tm = (uint32_t)tile_m;
-        const uint32_t nt = (count + tm - 1) / tm;
-        const uint32_t last_rows = count - (nt ? (nt - 1) * tm : 0);           // rows of the expert's last tile
-        const uint32_t n_big = nt == 0 ? 0 : (nt - 1) + (last_rows > kPackSmallTileRows ? 1u : 0u);
-        uint32_t total_big, total_small;
-        const uint32_t big_base = block_excl_scan(n_big, &total_big, sm);
-        const uint32_t small_base = block_excl_scan(nt - n_big, &total_small, sm);
+        const uint32_t total_big = tot[2];
         for (uint32_t j = 0; j < nt; ++j) {
             Tile t;
             t.expert = (uint32_t)e;
@@ -123,11 +139,10 @@ __device__ uint32_t emit_segments(uint32_t count, int e, int E, size_t n, int ti
             uint32_t left = count - j * tm;
             t.nrows = left < tm ? left : tm;
             t.flags = 0;
-            const uint32_t pos = j < n_big ? big_base + j : total_big + small_base;
+            const uint32_t pos = j < n_big ? ex[2] + j : total_big + ex[3];
             o.tiles[nt_dense + pos] = t;
         }
-        const uint32_t tf = total_big + total_small;
-        if (e == 0 && o.n_tiles) *o.n_tiles = nt_dense + tf;
+        if (e == 0 && o.n_tiles) *o.n_tiles = nt_dense + tot[2] + tot[3];
     }
     return off;
 }
@@ -174,7 +189,7 @@ __device__ __forceinline__ void pack_fused_body(const PackOut &o, uint32_t e, bo
 __global__ __launch_bounds__(kPackThreads) void pack_fused_kernel(PackOut o, const uint32_t *__restrict__ idx,
                                                                   uint32_t n, int K, int E, int tile_m) {
     extern __shared__ uint32_t pack_sm[]; // hist[kPackWaves][E]
-    __shared__ uint32_t scan_sm[kPackWaves + 1];
+    __shared__ uint32_t scan_sm[4 * kPackWaves];
     const bool active = threadIdx.x < n;
     const uint32_t e = active ? packed_id(o, idx[threadIdx.x]) : 0u;
     pack_fused_body(o, e, active, n, K, E, tile_m, pack_sm, scan_sm);
@@ -209,7 +224,7 @@ __global__ __launch_bounds__(kScatterWaves * 64) void pack_hist_kernel(PackOut o
 
 __global__ __launch_bounds__(kPackThreads) void pack_scan_kernel(PackOut o, uint32_t *__restrict__ cnt,
                                                                  size_t n, int E, int n_sub, int tile_m) {
-    __shared__ uint32_t scan_sm[kPackWaves + 1];
+    __shared__ uint32_t scan_sm[4 * kPackWaves];
     const int tid = (int)threadIdx.x;
     uint32_t count = 0;
     if (tid < E) {
