@@ -87,7 +87,8 @@ def cpu_baseline(wl, max_tokens, min_seconds=10.0, max_runs=5):
 
 def measured_peaks(torch):
     """What simple library kernels reach on this GPU, reported next to the published peaks: a device-to-device copy
-    (read + written bytes per second) and a square bf16 GEMM through torch (hipBLASLt)."""
+    (read + written bytes per second), a square bf16 GEMM through torch (hipBLASLt) and a loop of matrix instructions
+    alone."""
     out = {}
     n = 1 << 30
     src = torch.empty(n, dtype=torch.uint8, device="cuda")
@@ -105,6 +106,25 @@ def measured_peaks(torch):
         e1.record()
         torch.cuda.synchronize()
         out[name] = work / (e0.elapsed_time(e1) / 10 * 1e-3)
+    # the matrix cores alone: the library's loop of bf16 matrix instructions on operands in registers (no loads, no
+    # LDS, no decode), on all-zero and on random operands. The gap between the two is power: the prefill kernels'
+    # ceiling on real data is the second figure, not the published peak the roofline fraction is quoted against.
+    from dmlx_amd import capi
+    iters = 20000
+    g = torch.Generator(device="cuda").manual_seed(2)
+    rnd = torch.randn((capi.MFMA_LOOP_OPERANDS,), generator=g, device="cuda")
+    rnd[:capi.MFMA_LOOP_OPERANDS // 3] *= 0.02          # the weight fragments, scaled like the benchmark's weights
+    sink = torch.empty((capi.MFMA_LOOP_OUT,), dtype=torch.float32, device="cuda")
+    for name, ops in (("mfma_loop_zero_operands_TFLOPs", torch.zeros_like(rnd).to(torch.bfloat16)),
+                      ("mfma_loop_random_operands_TFLOPs", rnd.to(torch.bfloat16))):
+        for _ in range(3):
+            capi.mfma_loop(ops, iters, sink)
+        e0.record()
+        for _ in range(5):
+            capi.mfma_loop(ops, iters, sink)
+        e1.record()
+        torch.cuda.synchronize()
+        out[name] = capi.MFMA_LOOP_FLOP_PER_ITER * iters / 1e12 / (e0.elapsed_time(e1) / 5 * 1e-3)
     return out
 
 

@@ -72,7 +72,7 @@ EXPORTS = [
     "dmoe_resident_weight_create", "dmoe_resident_weight_destroy", "dmoe_gather_qmm_resident",
     "dmoe_layer_create", "dmoe_layer_destroy", "dmoe_moe_forward",
     "dmoe_switch_glu_forward_no_scores", "dmoe_moe_layer_forward", "dmoe_moe_layer_forward_static",
-    "dmoe_debug_last_activations", "dmoe_debug_dequantize_fused",
+    "dmoe_debug_last_activations", "dmoe_debug_dequantize_fused", "dmoe_debug_mfma_loop",
     "dmoe_gate_create", "dmoe_gate_destroy", "dmoe_gate_forward",
     "dmoe_layer_create_from_safetensors", "dmoe_layer_dims", "dmoe_batch_build", "dmoe_block_post",
 ]
@@ -289,6 +289,20 @@ def dequantize(qw, mat_index=0, fused=False):
     c = qw.c()
     fn = lib().dmoe_debug_dequantize_fused if fused else lib().dmoe_dequantize
     check(fn(_ptr(out), C.byref(c), mat_index, _stream()))
+    return out
+
+
+MFMA_LOOP_OPERANDS = 49152            # DMOE_MFMA_LOOP_OPERANDS
+MFMA_LOOP_OUT = 131072                # DMOE_MFMA_LOOP_OUT
+MFMA_LOOP_FLOP_PER_ITER = 2147483648.0
+
+
+def mfma_loop(operands, iters, out=None):
+    """dmoe_debug_mfma_loop: one launch of the matrix-instruction loop on `operands` (bf16 [MFMA_LOOP_OPERANDS])."""
+    assert operands.dtype == torch.bfloat16 and operands.numel() == MFMA_LOOP_OPERANDS and operands.is_contiguous()
+    if out is None:
+        out = torch.empty((MFMA_LOOP_OUT,), dtype=torch.float32, device=operands.device)
+    check(lib().dmoe_debug_mfma_loop(_ptr(out), _ptr(operands), int(iters), _stream()))
     return out
 
 

@@ -446,6 +446,17 @@ int dmoe_debug_last_activations(uint16_t *d_out, dmoe_layer layer, int T, dmoe_w
  * i.e. of mlx_dequantize as called at deepseek_v4_loader.zig:129, for every scale and bias. */
 int dmoe_debug_dequantize_fused(uint16_t *d_out, const dmoe_qweight *qw, int mat_index, dmoe_stream s);
 
+/* Calibration for the benchmark (no counterpart in the reference): ONE launch of a loop of bf16 matrix instructions
+ * (v_mfma_f32_32x32x16_bf16) on operands held in registers, 512 workgroups of 4 wavefronts, `iters` iterations of 32
+ * instructions per wavefront: DMOE_MFMA_LOOP_FLOP_PER_ITER floating-point operations per iteration and launch. What
+ * the matrix cores sustain with nothing else running depends on the operand values (power), so the caller chooses them:
+ * d_operands = DMOE_MFMA_LOOP_OPERANDS bf16 values (24 fragments x 256 lanes x 8), d_out = DMOE_MFMA_LOOP_OUT floats
+ * (one checksum per lane, so that the loop is not removed). The caller times the launch. */
+#define DMOE_MFMA_LOOP_OPERANDS 49152
+#define DMOE_MFMA_LOOP_OUT 131072
+#define DMOE_MFMA_LOOP_FLOP_PER_ITER 2147483648.0 /* 512 x 4 wavefronts x 32 instructions x 2*32*32*16 */
+int dmoe_debug_mfma_loop(float *d_out, const uint16_t *d_operands, int iters, dmoe_stream s);
+
 #ifdef __cplusplus
 }
 #endif

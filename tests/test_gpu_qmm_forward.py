@@ -591,3 +591,18 @@ def test_forward_edge_cases(dmoe, orc, ws):
     with pytest.raises(dmoe.DmoeError):
         dmoe.Layer(wl.D, wl.F + 8, wl.K, wl.gate, wl.up, wl.down)
     layer.close()
+
+
+def test_mfma_calibration_loop_counts_what_it_claims(dmoe):
+    """The benchmark's matrix-core calibration (dmoe_debug_mfma_loop) reports flops as iterations x a constant: with
+    every operand 1.0 each of a lane's 128 accumulators grows by 16 per instruction and 64 per iteration, so the lane
+    checksum must be 128 x 64 x iters exactly, i.e. the loop really issues 32 instructions of k = 16 per iteration."""
+    ones = torch.ones((dmoe.MFMA_LOOP_OPERANDS,), dtype=torch.bfloat16, device="cuda")
+    for iters in (1, 3):
+        out = dmoe.mfma_loop(ones, iters)
+        torch.cuda.synchronize()
+        assert out.shape == (dmoe.MFMA_LOOP_OUT,)
+        assert torch.equal(out, torch.full_like(out, 128.0 * 64.0 * iters))
+    assert dmoe.MFMA_LOOP_FLOP_PER_ITER == 512 * 4 * 32 * 2.0 * 32 * 32 * 16
+    with pytest.raises(dmoe.DmoeError, match="iters"):
+        dmoe.mfma_loop(ones, 0)
