@@ -87,8 +87,8 @@ def cpu_baseline(wl, max_tokens, min_seconds=10.0, max_runs=5):
 
 def measured_peaks(torch):
     """What simple library kernels reach on this GPU, reported next to the published peaks: a device-to-device copy
-    (read + written bytes per second), a square bf16 GEMM through torch (hipBLASLt) and a loop of matrix instructions
-    alone."""
+    (read + written bytes per second), a square bf16 GEMM through torch (hipBLASLt), a loop of matrix instructions
+    alone and a kernel that only reads."""
     out = {}
     n = 1 << 30
     src = torch.empty(n, dtype=torch.uint8, device="cuda")
@@ -125,6 +125,24 @@ def measured_peaks(torch):
         e1.record()
         torch.cuda.synchronize()
         out[name] = capi.MFMA_LOOP_FLOP_PER_ITER * iters / 1e12 / (e0.elapsed_time(e1) / 5 * 1e-3)
+    # a kernel that only reads (2 GiB, far beyond the memory-side cache): what the decode launch's weight streaming
+    # could reach at most. Few workgroups with long private streams do best; the best of three grid sizes is reported.
+    del dst, a, b
+    big = torch.empty(2 << 30, dtype=torch.uint8, device="cuda")
+    big.fill_(1)
+    best = 0.0
+    for wgs in (256, 512, 8192):
+        for _ in range(3):
+            nbytes = capi.read_stream(big, wgs)
+        e0.record()
+        for _ in range(10):
+            capi.read_stream(big, wgs)
+        e1.record()
+        torch.cuda.synchronize()
+        rate = nbytes / 1e9 / (e0.elapsed_time(e1) / 10 * 1e-3)
+        if rate > best:
+            best, out["read_stream_workgroups"] = rate, wgs
+    out["read_stream_GBs"] = best
     return out
 
 

@@ -72,7 +72,7 @@ EXPORTS = [
     "dmoe_resident_weight_create", "dmoe_resident_weight_destroy", "dmoe_gather_qmm_resident",
     "dmoe_layer_create", "dmoe_layer_destroy", "dmoe_moe_forward",
     "dmoe_switch_glu_forward_no_scores", "dmoe_moe_layer_forward", "dmoe_moe_layer_forward_static",
-    "dmoe_debug_last_activations", "dmoe_debug_dequantize_fused", "dmoe_debug_mfma_loop",
+    "dmoe_debug_last_activations", "dmoe_debug_dequantize_fused", "dmoe_debug_mfma_loop", "dmoe_debug_read_stream",
     "dmoe_gate_create", "dmoe_gate_destroy", "dmoe_gate_forward",
     "dmoe_layer_create_from_safetensors", "dmoe_layer_dims", "dmoe_batch_build", "dmoe_block_post",
 ]
@@ -304,6 +304,17 @@ def mfma_loop(operands, iters, out=None):
         out = torch.empty((MFMA_LOOP_OUT,), dtype=torch.float32, device=operands.device)
     check(lib().dmoe_debug_mfma_loop(_ptr(out), _ptr(operands), int(iters), _stream()))
     return out
+
+
+def read_stream(src, workgroups, sink=None):
+    """dmoe_debug_read_stream: one launch that reads `src` (any contiguous tensor); returns the bytes it reads."""
+    assert src.is_contiguous()
+    if sink is None:
+        sink = torch.empty((4 * workgroups,), dtype=torch.int32, device=src.device)
+    n = C.c_size_t(0)
+    check(lib().dmoe_debug_read_stream(C.byref(n), _ptr(sink), _ptr(src), C.c_size_t(src.numel() * src.element_size()),
+                                       int(workgroups), _stream()))
+    return n.value
 
 
 class ResidentWeight:

@@ -457,6 +457,14 @@ int dmoe_debug_dequantize_fused(uint16_t *d_out, const dmoe_qweight *qw, int mat
 #define DMOE_MFMA_LOOP_FLOP_PER_ITER 2147483648.0 /* 512 x 4 wavefronts x 32 instructions x 2*32*32*16 */
 int dmoe_debug_mfma_loop(float *d_out, const uint16_t *d_operands, int iters, dmoe_stream s);
 
+/* Calibration for the benchmark (no counterpart in the reference): ONE launch of a kernel that only reads. `workgroups`
+ * workgroups of 4 wavefronts; every wavefront streams a private contiguous part of d_src [bytes] with 16-byte loads,
+ * eight per lane in flight, with the streaming hint of the decode kernel's weight loads, and stores one checksum word
+ * into d_sink [4 * workgroups]. Whole 8 KiB chunks per wavefront only: *out_bytes_read gets the bytes one launch reads
+ * (<= bytes). The caller times the launch; a source larger than the 256 MiB memory-side cache measures HBM. */
+int dmoe_debug_read_stream(size_t *out_bytes_read, uint32_t *d_sink, const void *d_src, size_t bytes, int workgroups,
+                           dmoe_stream s);
+
 #ifdef __cplusplus
 }
 #endif

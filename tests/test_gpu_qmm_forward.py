@@ -606,3 +606,21 @@ def test_mfma_calibration_loop_counts_what_it_claims(dmoe):
     assert dmoe.MFMA_LOOP_FLOP_PER_ITER == 512 * 4 * 32 * 2.0 * 32 * 32 * 16
     with pytest.raises(dmoe.DmoeError, match="iters"):
         dmoe.mfma_loop(ones, 0)
+
+
+def test_read_stream_calibration_reads_what_it_reports(dmoe):
+    """dmoe_debug_read_stream reports the bytes one launch reads: whole 8 KiB chunks per wavefront, never past the
+    buffer, and each wavefront's checksum is the XOR of exactly its own part."""
+    wgs, chunk = 3, 8192
+    n = 4 * wgs * 2 * chunk + 5000                       # two chunks per wavefront and a ragged rest that is not read
+    src = torch.randint(0, 2 ** 31 - 1, (n // 4,), dtype=torch.int32, device="cuda")
+    sink = torch.zeros((4 * wgs,), dtype=torch.int32, device="cuda")
+    got = dmoe.read_stream(src, wgs, sink)
+    torch.cuda.synchronize()
+    assert got == 4 * wgs * 2 * chunk
+    per_wave = src[: got // 4].view(4 * wgs, -1).cpu().numpy()
+    import numpy as np
+    want = np.bitwise_xor.reduce(per_wave, axis=1)
+    assert np.array_equal(sink.cpu().numpy(), want)
+    with pytest.raises(dmoe.DmoeError, match="less than one"):
+        dmoe.read_stream(src[:1024], wgs, sink)
