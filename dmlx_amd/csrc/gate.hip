@@ -27,6 +27,8 @@ namespace dmoe {
 
 constexpr int kGateSeg = 128;   // reduction elements per partial sum
 constexpr int kGateTokens = 8;  // tokens per wavefront
+constexpr int kGateTokensFew = 2; // ... for batches of at most kGateFewTokens tokens: four times the wavefronts, each a quarter as long
+constexpr int kGateFewTokens = 256;
 constexpr int kGateWaves = 4;
 
 struct Gate {
@@ -51,16 +53,16 @@ __global__ void gate_repack_kernel(uint4 *__restrict__ dst, const uint16_t *__re
 // partial[(t * n_out_seg + s) * E + e]: SPLIT -> a workgroup takes `segs_per_wave` consecutive segments (grid.z =
 // group of segments) and stores every segment sum, n_out_seg = n_seg; otherwise it walks all segments and stores
 // their left-to-right sum, n_out_seg = 1.
-template <bool SPLIT>
+template <bool SPLIT, int TOK>
 __global__ __launch_bounds__(kGateWaves * 64) void gate_logits_kernel(float *__restrict__ partial,
                                                                       const uint16_t *__restrict__ x,
                                                                       const uint4 *__restrict__ wgp, int T, int D,
                                                                       int E, int n_seg, int segs_per_wave) {
-    __shared__ __attribute__((aligned(16))) float xs[kGateTokens][kGateSeg]; // the tokens' segment, widened to f32
+    __shared__ __attribute__((aligned(16))) float xs[TOK][kGateSeg]; // the tokens' segment, widened to f32
     const int tid = (int)threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int e = ((int)blockIdx.x * kGateWaves + wave) * 64 + lane;
-    const int t0 = (int)blockIdx.y * kGateTokens;
+    const int t0 = (int)blockIdx.y * TOK;
     const bool e_on = e < E;
     const int ec = e_on ? e : E - 1;
     const int seg0 = SPLIT ? (int)blockIdx.z * segs_per_wave : 0;
@@ -68,9 +70,9 @@ __global__ __launch_bounds__(kGateWaves * 64) void gate_logits_kernel(float *__r
     // staging: thread -> (token tid / 32, four elements at (tid % 32) * 4); surplus tokens repeat the last one
     const int st_tok = tid >> 5, st_k = (tid & 31) * 4;
     const uint16_t *st_src = x + (size_t)(t0 + st_tok < T ? t0 + st_tok : T - 1) * D;
-    float total[kGateTokens];
+    float total[TOK];
 #pragma unroll
-    for (int i = 0; i < kGateTokens; ++i) total[i] = 0.0f;
+    for (int i = 0; i < TOK; ++i) total[i] = 0.0f;
     for (int seg = seg0; seg < seg1; ++seg) {
         const int k_begin = seg * kGateSeg, k_end = k_begin + kGateSeg < D ? k_begin + kGateSeg : D;
         // all weight pieces of the segment are requested before the first is used (one memory round trip per
@@ -83,17 +85,17 @@ __global__ __launch_bounds__(kGateWaves * 64) void gate_logits_kernel(float *__r
             wq[j] = wgp[(size_t)(k >> 3) * E + ec];
         }
         float4 xv = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (k_begin + st_k < k_end) { // D is a multiple of 8, so four elements are in or out together
+        if (st_tok < TOK && k_begin + st_k < k_end) { // D is a multiple of 8, so four elements are in or out together
             const uint2 v = *(const uint2 *)(st_src + k_begin + st_k);
             xv = make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16),
                              __uint_as_float(v.y & 0xffff0000u));
         }
         __syncthreads(); // the previous segment has been consumed
-        *(float4 *)&xs[st_tok][st_k] = xv;
+        if (st_tok < TOK) *(float4 *)&xs[st_tok][st_k] = xv;
         __syncthreads();
-        float part[kGateTokens];
+        float part[TOK];
 #pragma unroll
-        for (int i = 0; i < kGateTokens; ++i) part[i] = 0.0f;
+        for (int i = 0; i < TOK; ++i) part[i] = 0.0f;
 #pragma unroll
         for (int j = 0; j < kPieces; ++j) {
             if (k_begin + 8 * j >= k_end) continue; // uniform
@@ -103,7 +105,7 @@ __global__ __launch_bounds__(kGateWaves * 64) void gate_logits_kernel(float *__r
             wf[4] = __uint_as_float(wq[j].z << 16); wf[5] = __uint_as_float(wq[j].z & 0xffff0000u);
             wf[6] = __uint_as_float(wq[j].w << 16); wf[7] = __uint_as_float(wq[j].w & 0xffff0000u);
 #pragma unroll
-            for (int i = 0; i < kGateTokens; ++i) {
+            for (int i = 0; i < TOK; ++i) {
                 // every lane reads the same address: LDS broadcasts
                 const float4 xa = *(const float4 *)&xs[i][8 * j], xb = *(const float4 *)&xs[i][8 * j + 4];
                 part[i] = fmaf(xa.x, wf[0], part[i]);
@@ -117,7 +119,7 @@ __global__ __launch_bounds__(kGateWaves * 64) void gate_logits_kernel(float *__r
             }
         }
 #pragma unroll
-        for (int i = 0; i < kGateTokens; ++i) {
+        for (int i = 0; i < TOK; ++i) {
             if (SPLIT) {
                 if (e_on && t0 + i < T) partial[((size_t)(t0 + i) * n_seg + seg) * E + e] = part[i];
             } else {
@@ -127,7 +129,7 @@ __global__ __launch_bounds__(kGateWaves * 64) void gate_logits_kernel(float *__r
     }
     if (SPLIT || !e_on) return;
 #pragma unroll
-    for (int i = 0; i < kGateTokens; ++i)
+    for (int i = 0; i < TOK; ++i)
         if (t0 + i < T) partial[(size_t)(t0 + i) * E + e] = total[i];
 }
 
@@ -190,7 +192,7 @@ __device__ __forceinline__ float det_logf(float x) {
 // round trip through memory; `scores` is written only when the caller wants them. Lane l owns experts l, l + 64, ...
 // (EPL of them). Softmax: the sum is taken as one partial per lane (its experts in increasing order), folded by
 // halves (lane i += lane i + 32, 16, .. 1).
-template <int EPL, bool ROUTE>
+template <int EPL, bool ROUTE, bool SPLIT>
 __global__ __launch_bounds__(kGateWaves * 64) void gate_scores_kernel(float *__restrict__ scores,
                                                                       const float *__restrict__ partial, int T,
                                                                       int E, int n_seg, int scoring,
@@ -204,23 +206,36 @@ __global__ __launch_bounds__(kGateWaves * 64) void gate_scores_kernel(float *__r
     if (t >= T) return;
     float v[EPL];
     float mx = -__builtin_inff();
+    // SPLIT (the matmul kernel stored every segment's sum): the segment sums of all of the lane's experts are requested
+    // 64 at a time (one memory round trip per batch, not one per expert and eight segments) and added per expert in
+    // segment order. Otherwise there is one sum per expert (n_seg == 1).
+    constexpr int SB = SPLIT ? 64 / EPL : 1;
+    const float *const p = partial + (size_t)t * n_seg * E;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) v[i] = 0.0f;
+    for (int s0 = 0; s0 < n_seg; s0 += SB) {
+        float q[EPL][SB];
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) {
+            const int e = lane + 64 * i;
+            const int ec = e < E ? e : E - 1;
+#pragma unroll
+            for (int j = 0; j < SB; ++j) q[i][j] = s0 + j < n_seg ? p[(size_t)(s0 + j) * E + ec] : 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < EPL; ++i)
+#pragma unroll
+            for (int j = 0; j < SB; ++j)
+                if (s0 + j < n_seg) v[i] = v[i] + q[i][j];
+    }
 #pragma unroll
     for (int i = 0; i < EPL; ++i) {
         const int e = lane + 64 * i;
-        v[i] = 0.0f;
         if (e < E) {
-            const float *p = partial + (size_t)t * n_seg * E + e;
-            float total = 0.0f;
-            for (int s0 = 0; s0 < n_seg; s0 += 8) { // eight loads in flight, added in order
-                float q[8];
-#pragma unroll
-                for (int j = 0; j < 8; ++j) q[j] = p[(size_t)(s0 + j < n_seg ? s0 + j : n_seg - 1) * E];
-#pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    if (s0 + j < n_seg) total = total + q[j];
-            }
-            v[i] = bf16_bits_to_f32(f32_to_bf16_bits(total));
+            v[i] = bf16_bits_to_f32(f32_to_bf16_bits(v[i]));
             mx = v[i] > mx ? v[i] : mx;
+        } else {
+            v[i] = 0.0f;
         }
     }
     if (scoring == DMOE_SCORE_SOFTMAX) {
@@ -264,6 +279,12 @@ __global__ __launch_bounds__(kGateWaves * 64) void gate_scores_kernel(float *__r
             out_w[(size_t)t * K + lane] = w;
         }
     }
+}
+
+template <int EPL, bool ROUTE, typename... Args>
+static void launch_scores(bool split, dim3 grid, dim3 block, hipStream_t st, Args... args) {
+    if (split) hipLaunchKernelGGL((gate_scores_kernel<EPL, ROUTE, true>), grid, block, 0, st, args...);
+    else hipLaunchKernelGGL((gate_scores_kernel<EPL, ROUTE, false>), grid, block, 0, st, args...);
 }
 
 // Hash routing (deepseek_v4.zig:619-636, then :655-678): the experts of a token come from a table indexed by its
@@ -383,7 +404,8 @@ int dmoe_gate_forward(uint32_t *d_out_indices, float *d_out_weights, float *d_ou
     const int n_seg = ceil_div(G->D, kGateSeg);
     // Few tokens: the segments are spread over several wavefronts so that the launch has about four wavefronts per
     // SIMD; the segment sums then travel through scratch (T * E * n_seg floats) to the scoring kernel.
-    const size_t waves_whole = (size_t)ceil_div(T, kGateTokens) * ceil_div(G->E, 64);
+    const int tok = T <= kGateFewTokens ? kGateTokensFew : kGateTokens;
+    const size_t waves_whole = (size_t)ceil_div(T, tok) * ceil_div(G->E, 64);
     int groups = (int)std::min<size_t>((size_t)n_seg, (4096 + waves_whole - 1) / waves_whole);
     const int segs_per_wave = ceil_div(n_seg, groups);
     groups = ceil_div(n_seg, segs_per_wave);
@@ -398,21 +420,27 @@ int dmoe_gate_forward(uint32_t *d_out_indices, float *d_out_weights, float *d_ou
     float *partial = at<float>(w, o_part);
     float *scores = d_out_scores ? d_out_scores : at<float>(w, o_scores);
     dim3 block(kGateWaves * 64);
-    dim3 grid((unsigned)ceil_div(G->E, kGateWaves * 64), (unsigned)ceil_div(T, kGateTokens), (unsigned)groups);
+    dim3 grid((unsigned)ceil_div(G->E, kGateWaves * 64), (unsigned)ceil_div(T, tok), (unsigned)groups);
     DMOE_REQUIRE(grid.y <= 65535u, "gate_forward: too many tokens for one launch (T=%d)", T);
-    if (split) hipLaunchKernelGGL(gate_logits_kernel<true>, grid, block, 0, st, partial, d_x, (const uint4 *)G->wgp, T, G->D, G->E, n_seg, segs_per_wave);
-    else hipLaunchKernelGGL(gate_logits_kernel<false>, grid, block, 0, st, partial, d_x, (const uint4 *)G->wgp, T, G->D, G->E, n_seg, segs_per_wave);
+    if (split && tok == kGateTokensFew)
+        hipLaunchKernelGGL((gate_logits_kernel<true, kGateTokensFew>), grid, block, 0, st, partial, d_x, (const uint4 *)G->wgp, T, G->D, G->E, n_seg, segs_per_wave);
+    else if (split)
+        hipLaunchKernelGGL((gate_logits_kernel<true, kGateTokens>), grid, block, 0, st, partial, d_x, (const uint4 *)G->wgp, T, G->D, G->E, n_seg, segs_per_wave);
+    else if (tok == kGateTokensFew)
+        hipLaunchKernelGGL((gate_logits_kernel<false, kGateTokensFew>), grid, block, 0, st, partial, d_x, (const uint4 *)G->wgp, T, G->D, G->E, n_seg, segs_per_wave);
+    else
+        hipLaunchKernelGGL((gate_logits_kernel<false, kGateTokens>), grid, block, 0, st, partial, d_x, (const uint4 *)G->wgp, T, G->D, G->E, n_seg, segs_per_wave);
     DMOE_LAUNCH_CHECK();
     // the reference renormalises for every scoring function except softmax (:663)
     const int normalize = G->scoring != DMOE_SCORE_SOFTMAX ? 1 : 0;
     const dim3 sgrid((unsigned)ceil_div(T, kGateWaves));
     if (hash) { // hash layer with token ids: the table replaces the top-k (:619-636)
         if (G->E <= 256)
-            hipLaunchKernelGGL((gate_scores_kernel<4, false>), sgrid, block, 0, st, scores, partial, T, G->E, n_out_seg, G->scoring,
-                               nullptr, nullptr, nullptr, nullptr, 0, 0, 1.0f);
+            launch_scores<4, false>(split, sgrid, block, st, scores, partial, T, G->E, n_out_seg, G->scoring, nullptr, nullptr,
+                                    nullptr, nullptr, 0, 0, 1.0f);
         else
-            hipLaunchKernelGGL((gate_scores_kernel<16, false>), sgrid, block, 0, st, scores, partial, T, G->E, n_out_seg, G->scoring,
-                               nullptr, nullptr, nullptr, nullptr, 0, 0, 1.0f);
+            launch_scores<16, false>(split, sgrid, block, st, scores, partial, T, G->E, n_out_seg, G->scoring, nullptr, nullptr,
+                                     nullptr, nullptr, 0, 0, 1.0f);
         DMOE_LAUNCH_CHECK();
         hipLaunchKernelGGL(gate_hash_route_kernel, dim3((unsigned)ceil_div(T, 256)), dim3(256), 0, st, d_out_indices,
                            d_out_weights, scores, G->tid2eid, d_input_ids, T, G->E, G->K, G->vocab, normalize, G->route_scale);
@@ -422,11 +450,11 @@ int dmoe_gate_forward(uint32_t *d_out_indices, float *d_out_weights, float *d_ou
     // scoring and selection in one launch; the scores leave the registers only if the caller asked for them
     DMOE_REQUIRE(G->K >= 1 && G->K <= G->E && G->K <= 64, "gate_forward: K=%d must satisfy 1 <= K <= min(E,64)", G->K);
     if (G->E <= 256)
-        hipLaunchKernelGGL((gate_scores_kernel<4, true>), sgrid, block, 0, st, d_out_scores, partial, T, G->E, n_out_seg, G->scoring,
-                           d_out_indices, d_out_weights, G->bias, G->mask, G->K, normalize, G->route_scale);
+        launch_scores<4, true>(split, sgrid, block, st, d_out_scores, partial, T, G->E, n_out_seg, G->scoring, d_out_indices,
+                               d_out_weights, G->bias, G->mask, G->K, normalize, G->route_scale);
     else
-        hipLaunchKernelGGL((gate_scores_kernel<16, true>), sgrid, block, 0, st, d_out_scores, partial, T, G->E, n_out_seg, G->scoring,
-                           d_out_indices, d_out_weights, G->bias, G->mask, G->K, normalize, G->route_scale);
+        launch_scores<16, true>(split, sgrid, block, st, d_out_scores, partial, T, G->E, n_out_seg, G->scoring, d_out_indices,
+                                d_out_weights, G->bias, G->mask, G->K, normalize, G->route_scale);
     DMOE_LAUNCH_CHECK();
     return DMOE_OK;
 }
