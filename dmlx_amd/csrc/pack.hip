@@ -228,9 +228,9 @@ __global__ __launch_bounds__(kPackThreads) void pack_scan_kernel(PackOut o, uint
     const int tid = (int)threadIdx.x;
     uint32_t count = 0;
     if (tid < E) {
-        // exclusive scan down this expert's column of sub-chunk counts, eight independent loads at a time (one
+        // exclusive scan down this expert's column of sub-chunk counts, 32 independent loads at a time (one
         // dependent load per sub-chunk made this loop the longest part of packing a prefill batch)
-        constexpr int kBatch = 8;
+        constexpr int kBatch = 32;
         for (int s0 = 0; s0 < n_sub; s0 += kBatch) {
             uint32_t c[kBatch];
 #pragma unroll
