@@ -30,6 +30,10 @@ constexpr int kGateTokens = 8;  // tokens per wavefront
 constexpr int kGateTokensFew = 2; // ... for batches of at most kGateFewTokens tokens: four times the wavefronts, each a quarter as long
 constexpr int kGateFewTokens = 256;
 constexpr int kGateWaves = 4;
+#ifndef DMOE_GATE_MFMA_MIN_TILES
+#define DMOE_GATE_MFMA_MIN_TILES 640
+#endif
+constexpr size_t kGateMfmaMinTiles = DMOE_GATE_MFMA_MIN_TILES; // 32 x 32 output tiles from which the matrix-core kernel is the faster one
 
 struct Gate {
     int device = 0;
@@ -131,6 +135,156 @@ __global__ __launch_bounds__(kGateWaves * 64) void gate_logits_kernel(float *__r
 #pragma unroll
     for (int i = 0; i < TOK; ++i)
         if (t0 + i < T) partial[(size_t)(t0 + i) * E + e] = total[i];
+}
+
+// The same sums on the f32 matrix core, for batches large enough to fill it. v_mfma_f32_32x32x2_f32 adds its two
+// products to the accumulator one after the other, each with one rounding: D = fma(a1, b1, fma(a0, b0, C)), bit for
+// bit what two fmaf calls give (checked on the device against the C library over 20 480 outputs of 64-instruction
+// chains, operands of both signs and of magnitudes six decades apart). A chain of these instructions over a
+// segment's 128 elements, started from C = 0, is therefore the segment sum exactly as gate_logits_kernel and the CPU
+// restatement form it, at twice the vector ALU's rate (the vector path has no packed fp32 here).
+// Wavefront = 32 tokens x NB blocks of 32 experts, the whole reduction; lane (i = lane % 32, kk = lane / 32) feeds
+// element kk of every pair of reduction elements for token i (A) and expert i of each block (B). Operands come
+// straight from global memory, 16 bytes = 8 elements per lane and row, kGateMfmaAhead chunks ahead in registers
+// (one wavefront per SIMD: nothing else hides the latency); both lane halves load the same 16 bytes and pick the
+// even or the odd elements. No LDS, no barrier.
+constexpr int kGateMfmaAhead = 4;
+template <int NB>
+__global__ __launch_bounds__(kGateWaves * 64) void gate_logits_mfma_kernel(float *__restrict__ logits,
+                                                                           const uint16_t *__restrict__ x,
+                                                                           const uint4 *__restrict__ wgp, int T, int D,
+                                                                           int E) {
+    const int tid = (int)threadIdx.x, lane = tid & 63, i = lane & 31, kk = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int t0 = (int)blockIdx.y * 32;
+    const int e0 = ((int)blockIdx.x * kGateWaves + wave) * 32 * NB;
+    if (e0 >= E) return; // the whole wavefront is past the last expert
+    const uint4 *const xrow = (const uint4 *)(x + (size_t)(t0 + i < T ? t0 + i : T - 1) * D);
+    int ec[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) ec[b] = e0 + 32 * b + i < E ? e0 + 32 * b + i : E - 1;
+    const int n_chunks = D >> 3;
+    constexpr int CPS = kGateSeg / 8; // chunks per segment
+    static_assert(CPS % kGateMfmaAhead == 0, "a segment is a whole number of turns of the ring");
+    const uint32_t sh = kk ? 0u : 16u; // element kk of a dword: the low half moves up, the high half stays
+    uint4 xr[kGateMfmaAhead], wr[kGateMfmaAhead][NB];
+#pragma unroll
+    for (int j = 0; j < kGateMfmaAhead; ++j) {
+        const int c = j < n_chunks ? j : n_chunks - 1;
+        xr[j] = xrow[c];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) wr[j][b] = wgp[(size_t)c * E + ec[b]];
+    }
+    f32x16_t total[NB], part[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) total[b][r] = 0.0f;
+    // the four pairs of one chunk: element kk of every dword
+    auto pairs = [&](const uint4 &xv, const uint4 (&wv)[NB]) {
+        const uint32_t xd[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const float a = __uint_as_float((xd[p] << sh) & 0xffff0000u);
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const uint32_t wd = p == 0 ? wv[b].x : p == 1 ? wv[b].y : p == 2 ? wv[b].z : wv[b].w;
+                part[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, __uint_as_float((wd << sh) & 0xffff0000u), part[b], 0, 0, 0);
+            }
+        }
+    };
+    auto segment_done = [&]() {
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                total[b][r] = total[b][r] + part[b][r];
+                part[b][r] = 0.0f;
+            }
+    };
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) part[b][r] = 0.0f;
+    // Whole segments: straight-line code, the ring slot of every chunk known at compile time. The operands of chunk
+    // c + 1 are widened to f32 between the matrix instructions of chunk c, into registers of their own (widening in
+    // place, right in front of each matrix instruction, measured 5 % slower). What keeps the chain from the bare
+    // instruction rate (28 ns per instruction measured, 150 TFLOP/s on the whole chip) are the load instructions: each
+    // costs the wavefront about 30 ns of issue whatever the look-ahead (4, 8 or 16 chunks measure the same; without
+    // the loads the kernel runs at the bare rate), which is why a wavefront takes two expert blocks per activation
+    // chunk once there is work for more than two wavefronts per SIMD. Fetching a pair of chunks per load (one per lane
+    // half, exchanged with v_permlane32_swap) halves the loads but costs the same again in swaps.
+    const int n_whole = n_chunks / CPS;
+    auto widen = [&](uint32_t d) { return __uint_as_float((d << sh) & 0xffff0000u); };
+    float fa[4], fb[NB][4];
+    {
+        const uint32_t xd[4] = {xr[0].x, xr[0].y, xr[0].z, xr[0].w};
+#pragma unroll
+        for (int p = 0; p < 4; ++p) fa[p] = widen(xd[p]);
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const uint32_t wd[4] = {wr[0][b].x, wr[0][b].y, wr[0][b].z, wr[0][b].w};
+#pragma unroll
+            for (int p = 0; p < 4; ++p) fb[b][p] = widen(wd[p]);
+        }
+    }
+    for (int seg = 0; seg < n_whole; ++seg) {
+#pragma unroll
+        for (int j = 0; j < CPS; ++j) {
+            const int c = seg * CPS + j;
+            constexpr int A = kGateMfmaAhead;
+            const uint4 xn = xr[(j + 1) % A];
+            const uint32_t xd[4] = {xn.x, xn.y, xn.z, xn.w};
+            float na[4], nb[NB][4];
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+#pragma unroll
+                for (int b = 0; b < NB; ++b) part[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[p], fb[b][p], part[b], 0, 0, 0);
+                na[p] = widen(xd[p]);
+#pragma unroll
+                for (int b = 0; b < NB; ++b) {
+                    const uint4 wn = wr[(j + 1) % A][b];
+                    nb[b][p] = widen(p == 0 ? wn.x : p == 1 ? wn.y : p == 2 ? wn.z : wn.w);
+                }
+                __builtin_amdgcn_sched_barrier(0); // keeps the widening between the matrix instructions
+            }
+            // slot j % A was widened during the chunk before: request the chunk that will use it next (the barriers keep
+            // the request HERE; left alone, the compiler sinks every load to just in front of its first use)
+            const int cn = c + A < n_chunks ? c + A : n_chunks - 1; // the last ones are not used
+            xr[j % A] = xrow[cn];
+#pragma unroll
+            for (int b = 0; b < NB; ++b) wr[j % A][b] = wgp[(size_t)cn * E + ec[b]];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                fa[p] = na[p];
+#pragma unroll
+                for (int b = 0; b < NB; ++b) fb[b][p] = nb[b][p];
+            }
+        }
+        segment_done();
+    }
+    // a short last segment (D not a multiple of 128): its few chunks are fetched as they are used
+    if (n_whole * CPS < n_chunks) {
+        for (int c = n_whole * CPS; c < n_chunks; ++c) {
+            const uint4 xv = xrow[c];
+            uint4 wv[NB];
+#pragma unroll
+            for (int b = 0; b < NB; ++b) wv[b] = wgp[(size_t)c * E + ec[b]];
+            pairs(xv, wv);
+        }
+        segment_done();
+    }
+    // accumulator r of lane (i, kk) is token 8 (r / 4) + 4 kk + r % 4, expert i of its block
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        const int e = e0 + 32 * b + i;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int t = t0 + 8 * (r >> 2) + 4 * kk + (r & 3);
+            if (e < E && t < T) logits[(size_t)t * E + e] = total[b][r];
+        }
+    }
 }
 
 // exp(x) from IEEE operations only: Cody-Waite reduction by ln 2 in two parts, the degree-5 polynomial of the
@@ -409,7 +563,12 @@ int dmoe_gate_forward(uint32_t *d_out_indices, float *d_out_weights, float *d_ou
     int groups = (int)std::min<size_t>((size_t)n_seg, (4096 + waves_whole - 1) / waves_whole);
     const int segs_per_wave = ceil_div(n_seg, groups);
     groups = ceil_div(n_seg, segs_per_wave);
-    const bool split = groups > 1;
+    // enough 32-token x 32-expert tiles for one wavefront on most SIMDs of the chip: the matrix-core kernel (whole
+    // sums); two tiles per wavefront once there are more than two wavefronts per SIMD
+    const size_t mfma_tiles = (size_t)ceil_div(T, 32) * ceil_div(G->E, 32);
+    const bool mfma = mfma_tiles >= kGateMfmaMinTiles;
+    const int mfma_nb = mfma_tiles > 2048 ? 2 : 1;
+    const bool split = groups > 1 && !mfma;
     const int n_out_seg = split ? n_seg : 1;
     Bump b;
     const size_t o_part = b.take(sizeof(float) * (size_t)T * G->E * n_out_seg);
@@ -422,7 +581,11 @@ int dmoe_gate_forward(uint32_t *d_out_indices, float *d_out_weights, float *d_ou
     dim3 block(kGateWaves * 64);
     dim3 grid((unsigned)ceil_div(G->E, kGateWaves * 64), (unsigned)ceil_div(T, tok), (unsigned)groups);
     DMOE_REQUIRE(grid.y <= 65535u, "gate_forward: too many tokens for one launch (T=%d)", T);
-    if (split && tok == kGateTokensFew)
+    if (mfma) {
+        const dim3 mgrid((unsigned)ceil_div(G->E, kGateWaves * 32 * mfma_nb), (unsigned)ceil_div(T, 32));
+        if (mfma_nb == 2) hipLaunchKernelGGL(gate_logits_mfma_kernel<2>, mgrid, block, 0, st, partial, d_x, (const uint4 *)G->wgp, T, G->D, G->E);
+        else hipLaunchKernelGGL(gate_logits_mfma_kernel<1>, mgrid, block, 0, st, partial, d_x, (const uint4 *)G->wgp, T, G->D, G->E);
+    } else if (split && tok == kGateTokensFew)
         hipLaunchKernelGGL((gate_logits_kernel<true, kGateTokensFew>), grid, block, 0, st, partial, d_x, (const uint4 *)G->wgp, T, G->D, G->E, n_seg, segs_per_wave);
     else if (split)
         hipLaunchKernelGGL((gate_logits_kernel<true, kGateTokens>), grid, block, 0, st, partial, d_x, (const uint4 *)G->wgp, T, G->D, G->E, n_seg, segs_per_wave);

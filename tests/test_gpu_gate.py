@@ -31,6 +31,8 @@ def _case(seed, T, D, E, with_bias, with_mask, spread):
     (4200, 256, 128, 6, True, False),    # many tokens: a wavefront walks all segments itself
     (1100, 4096, 256, 6, True, False),   # the prefill shape of configurations 3 / 4
     (900, 520, 300, 5, False, True),     # more than 256 experts, short last segment
+    (6200, 520, 300, 5, False, True),    # enough tiles for the f32 matrix-core kernel: ragged tokens and experts, short last segment
+    (12345, 256, 128, 6, True, False),   # the same kernel, whole segments, a partial last token tile
 ])
 def test_gate_forward_bit_exact(dmoe, orc, ws, func, T, D, E, K, with_bias, with_mask):
     x, wg, bias, mask = _case(7 + func, T, D, E, with_bias, with_mask, spread=2.0)
@@ -46,6 +48,21 @@ def test_gate_forward_bit_exact(dmoe, orc, ws, func, T, D, E, K, with_bias, with
     # without the inspection output the routing is the same
     idx2, w2 = gate.forward(x, ws)
     assert torch.equal(idx2, idx) and torch.equal(w2, w)
+    gate.close()
+
+
+def test_gate_prefill_full_size_bit_exact(dmoe, orc, ws):
+    """The router of the 8192-token prefill (f32 matrix-core kernel, one 32 x 32 tile per wavefront) at full size: logits
+    after scoring, selected experts and weights bit for bit against the CPU restatement, whose sums are fmaf chains."""
+    T, D, E, K = 8192, 4096, 256, 6
+    x, wg, bias, _ = _case(31, T, D, E, True, False, spread=2.0)
+    gate = dmoe.Gate(wg, K, 2, route_scale=1.5, bias=bias)
+    idx, w, scores = gate.forward(x, ws, want_scores=True)
+    want_scores = orc.gate_scores_det(orc.gate_logits(bf16_bits(x), bf16_bits(wg)), 2)
+    np.testing.assert_array_equal(scores.cpu().numpy().view(np.uint32), want_scores.view(np.uint32))
+    want_idx, want_w = orc.gate_route(want_scores, bias.cpu().numpy(), None, K, True, 1.5)
+    np.testing.assert_array_equal(to_np_u32(idx), want_idx)
+    np.testing.assert_array_equal(w.cpu().numpy().view(np.uint32), want_w.view(np.uint32))
     gate.close()
 
 
