@@ -33,6 +33,7 @@ def _case(seed, T, D, E, with_bias, with_mask, spread):
     (900, 520, 300, 5, False, True),     # more than 256 experts, short last segment
     (6200, 520, 300, 5, False, True),    # enough tiles for the f32 matrix-core kernel: ragged tokens and experts, short last segment
     (12345, 256, 128, 6, True, False),   # the same kernel, whole segments, a partial last token tile
+    (9000, 392, 300, 6, True, True),     # more than 2048 tiles: two expert blocks per wavefront, the last block partly past E
 ])
 def test_gate_forward_bit_exact(dmoe, orc, ws, func, T, D, E, K, with_bias, with_mask):
     x, wg, bias, mask = _case(7 + func, T, D, E, with_bias, with_mask, spread=2.0)
