@@ -120,3 +120,28 @@ def test_gate_rejects_bad_arguments(dmoe):
         dmoe.Gate(wg[:, :60].contiguous(), 2, 1)   # dim not a multiple of 8
     with pytest.raises(dmoe.DmoeError):
         dmoe.Gate(wg, 2, 7)            # unknown scoring function
+
+
+@pytest.mark.parametrize("T", [40, 6200])
+def test_gate_logits_tiny_and_huge_magnitudes(dmoe, orc, ws, T):
+    """Both matmul kernels (vector ALU for 40 tokens, f32 matrix core for 6200) on operands whose sums overflow to
+    infinity (both signs) next to operands whose products are f32 denormals: the scores must still be the oracle's
+    bits. (Logits that small all score like 0, so this checks that tiny operands produce nothing else - no NaN, no
+    stray value - not how the hardware rounds denormals; the overflowing sums do tell saturation from infinity.)"""
+    D, E = 256, 300
+    g = torch.Generator(device="cuda").manual_seed(17)
+    sign = lambda *s: torch.where(torch.rand(s, generator=g, device="cuda") < 0.5, -1.0, 1.0)
+    x = torch.full((T, D), 2.0 ** -90, device="cuda") * sign(T, D) * (1 + torch.rand((T, D), generator=g, device="cuda"))
+    wg = torch.full((E, D), 2.0 ** -50, device="cuda") * sign(E, D) * (1 + torch.rand((E, D), generator=g, device="cuda"))
+    x[1::2] = x[1::2] * 2.0 ** 150          # every second token: products near 2^10, still ordinary numbers
+    x[3::8] = 2.0 ** 100                    # some tokens against ...
+    wg[5::16] = 2.0 ** 27                   # ... some experts: 256 products of 2^127 overflow the sum
+    x, wg = x.to(torch.bfloat16), wg.to(torch.bfloat16)
+    logits = orc.gate_logits(bf16_bits(x), bf16_bits(wg))
+    assert np.isinf(logits).any() and (np.abs(logits[np.isfinite(logits)]) < 2.0 ** -126).any(), "the case must reach both ends"
+    for func in (1, 2):
+        gate = dmoe.Gate(wg, 4, func)
+        _, _, scores = gate.forward(x, ws, want_scores=True)
+        want = orc.gate_scores_det(logits, func)
+        np.testing.assert_array_equal(scores.cpu().numpy().view(np.uint32), want.view(np.uint32))
+        gate.close()
