@@ -336,14 +336,26 @@ template <typename Fmt, bool GATE_UP>
 __global__ __launch_bounds__(kWideWaves * 64, 2) void qgemm_wide_kernel(GemmArgs g) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t wide_lds[]; // [kWideRing][128 rows][128 bytes], swizzled
     Tile t;
-    // Workgroups go to the eight XCDs round-robin in launch order. All column strips of a tile are given to ONE XCD
-    // (tile = 8 * (k / strips) + xcd for the k-th workgroup of that XCD), so the tile's activations are fetched into one
-    // L2 instead of eight; gridDim.y is a multiple of 8, which makes this a permutation of the grid. (Also giving an XCD
-    // runs of 2..16 consecutive tiles of the list, their workgroups of one strip started back to back so that the tiles
-    // of an expert could share its weights through that L2, measured 0.5 % to 15 % slower the longer the run.)
-    const uint32_t nx = gridDim.x, b = blockIdx.y * nx + blockIdx.x, k = b >> 3;
-    const uint32_t slot = (k / nx) * 8u + (b & 7u);
-    const int strip = (int)(k % nx);
+    // Workgroups go to the eight XCDs round-robin in launch order; gridDim.y is a multiple of 8, which makes the maps
+    // below permutations of the grid. XCD x = (tile class x / 2, strip half x % 2): it takes every fourth tile of the
+    // list and one half of the tile's column strips, a tile's strips back to back. A tile's activations then enter two
+    // L2s instead of eight, and consecutive tiles of an expert find the half of its weights they need in the L2 they
+    // run on. Same box, against all strips of a tile on one XCD (the map before, kept for strip counts that are odd):
+    // C3 step -0.7 % (down launch -1.6 %), C4 step -1.7 % (gate/up launch -2.4 %); four strip groups x two tile classes
+    // -0.6 % / -1.3 %, eight strip groups (an XCD = two strips of every tile) +0.8 % / -0.9 %. (Giving an XCD runs of
+    // 2..16 consecutive tiles with ALL their strips, so that the tiles of an expert could share its weights through
+    // that L2, measured 0.5 % to 15 % slower the longer the run: an expert's weights do not fit one L2.)
+    const uint32_t nx = gridDim.x, b = blockIdx.y * nx + blockIdx.x, k = b >> 3, xcd = b & 7u;
+    uint32_t slot;
+    int strip;
+    if (nx % 2u == 0u) {
+        const uint32_t half = nx / 2u;
+        slot = 4u * (k / half) + (xcd >> 1);
+        strip = (int)((xcd & 1u) * half + k % half);
+    } else {
+        slot = (k / nx) * 8u + xcd;
+        strip = (int)(k % nx);
+    }
     if (g.tiles) {
         const uint32_t n_tiles = *g.n_tiles;
         t = g.tiles[slot < (uint32_t)g.max_tiles ? slot : 0u];
