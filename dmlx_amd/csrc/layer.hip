@@ -1,5 +1,6 @@
 // Resident MoE layer: weights held in HBM, and the forward pass
-//   remap -> pack -> grouped gate/up + limited SwiGLU -> grouped down -> weighted sum over k (+ shared).
+//   pack (slot map of Smelt layers applied as the ids are read) -> grouped gate/up + limited SwiGLU -> grouped down ->
+//   weighted sum over k (+ shared).
 // Also dmoe_gather_qmm, the leaf operator, built from the same pack + grouped-GEMM kernels.
 #include <string.h>
 
