@@ -239,6 +239,7 @@ int launch_gemm_bf16(const GemmArgs &g, hipStream_t st);
 int qgemm_skinny_tile_m(const QView &b);  // rows per tile to build tile lists with for the skinny path
 bool qgemm_mfma_supports(const QView &b);
 bool qgemm_wide_supports(const QView &b);
+bool qgemm_wide_bf16_supports(const QView &b); // unquantized weights in the packed resident layout (launch_qgemm_wide takes them too)
 // tile size to build tile lists with for the MFMA path of this weight matrix
 inline int qgemm_mfma_tile_m(const QView &b) { return qgemm_wide_supports(b) ? kMfmaWideTileM : kMfmaTileM; }
 

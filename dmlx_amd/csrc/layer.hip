@@ -182,8 +182,9 @@ __global__ void combine_kernel(uint16_t *__restrict__ out, const uint16_t *__res
 constexpr int kSkinnyAvgRows = 16;
 constexpr int kSharedSkinnyRows = 64;
 
+static bool few_rows(size_t rows, int n_experts) { return rows <= (size_t)kSkinnyAvgRows * (size_t)n_experts; }
 static bool use_small_path(size_t rows, int n_experts, const QView &b) {
-    return qgemm_skinny_supports(b) && rows <= (size_t)kSkinnyAvgRows * (size_t)n_experts;
+    return qgemm_skinny_supports(b) && few_rows(rows, n_experts);
 }
 struct FwdLayout {
     size_t order, inv, token, sorted_e, counts, offsets, live, n_live, tiles, n_tiles, tile_done, scratch;
@@ -238,8 +239,14 @@ static int prefill_small_rows(const QView &b0, const QView &b1) {
     // threshold measured on the same prefill: 8 rows 2.62 ms, 16 rows 2.63, 32 rows 2.64, 4 rows 2.67, no split 2.70
     return std::min(kPrefillSmallRows, std::min(qgemm_skinny_tile_m(b0), qgemm_skinny_tile_m(b1)));
 }
-static int run_gemm(const GemmArgs &g, bool small, hipStream_t st, int small_rows = 0) {
-    if (g.b0.mode == DMOE_QUANT_NONE) return launch_gemm_bf16(g, st);
+// `few` = few rows per expert (only read for unquantized weights; the quantized formats have `small`)
+static int run_gemm(const GemmArgs &g, bool small, hipStream_t st, int small_rows = 0, bool few = false) {
+    if (g.b0.mode == DMOE_QUANT_NONE) {
+        // prefill sizes on resident weights: the matrix-core kernel with activations through LDS
+        const bool wide = !few && qgemm_wide_bf16_supports(g.b0) && (!g.gate_up || qgemm_wide_bf16_supports(g.b1)) &&
+                          g.tile_m % 32 == 0 && g.tile_m <= kMfmaWideTileM;
+        return wide ? launch_qgemm_wide(g, st) : launch_gemm_bf16(g, st);
+    }
     if (small) return launch_qgemm_skinny(g, st);
     if (small_rows <= 0 || !g.tiles) return launch_qgemm_mfma(g, st);
     GemmArgs big = g, rest = g;
@@ -360,10 +367,11 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
         return DMOE_OK;
     }
     DMOE_TRY(stage_begin(w, DMOE_STAGE_GATE_UP, st));
-    DMOE_TRY(run_gemm(gu, f.small, st));
+    const bool few = few_rows(n, L->E);
+    DMOE_TRY(run_gemm(gu, f.small, st, 0, few));
     DMOE_TRY(stage_end(w, DMOE_STAGE_GATE_UP, st));
     DMOE_TRY(stage_begin(w, DMOE_STAGE_DOWN, st));
-    DMOE_TRY(run_gemm(dn, f.small, st));
+    DMOE_TRY(run_gemm(dn, f.small, st, 0, few));
     DMOE_TRY(stage_end(w, DMOE_STAGE_DOWN, st));
     return DMOE_OK;
 }
@@ -385,7 +393,7 @@ static int shared_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     gu.max_tiles = ceil_div(T, tile_m);
     gu.tile_m = tile_m;
     gu.swiglu_limit = L->shared_swiglu_limit;
-    DMOE_TRY(run_gemm(gu, small, st));
+    DMOE_TRY(run_gemm(gu, small, st, 0, T <= kSharedSkinnyRows));
     GemmArgs dn;
     dn.b0 = L->sdown.view;
     dn.a = at<uint16_t>(w, f.sh_h);
@@ -394,7 +402,7 @@ static int shared_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     dn.dense_rows = T;
     dn.max_tiles = ceil_div(T, tile_m);
     dn.tile_m = tile_m;
-    DMOE_TRY(run_gemm(dn, small, st));
+    DMOE_TRY(run_gemm(dn, small, st, 0, T <= kSharedSkinnyRows));
     return DMOE_OK;
 }
 
@@ -782,7 +790,7 @@ static int gather_qmm_view(uint16_t *d_out, const uint16_t *d_x, const QView &v,
     g.n_tiles = po.n_tiles;
     g.max_tiles = max_tiles;
     g.tile_m = tile_m;
-    return run_gemm(g, small, st, small ? 0 : prefill_small_rows(v, v));
+    return run_gemm(g, small, st, small ? 0 : prefill_small_rows(v, v), few_rows((size_t)R, v.n_mats));
 }
 
 int dmoe_gather_qmm(uint16_t *d_out, const uint16_t *d_x, const dmoe_qweight *qw, const uint32_t *d_lhs_indices,

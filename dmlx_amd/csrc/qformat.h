@@ -338,6 +338,39 @@ struct FmtFp8Row {
     }
 };
 
+// Unquantized bf16 weights seen as a "format" by the prefill kernel: a 16-byte chunk is eight values, i.e. exactly one
+// matrix-instruction operand, and decoding is the identity. Not part of dispatch_format (which walks the quantized modes).
+struct FmtBf16 {
+    static constexpr int kVals = 8;
+    static constexpr int kMetaEntryBytes = 0;
+    static constexpr int kDecodeOps = 0;
+    static constexpr bool kRowScale = false;
+    __device__ static __forceinline__ void load_meta_raw(const QView &, const uint8_t *, const uint8_t *, int, uint32_t *sb) {
+        sb[0] = 0u;
+        sb[1] = 0u;
+    }
+    __device__ static __forceinline__ size_t packed_meta_base(const QView &, size_t, int) { return 0; }
+    __device__ static __forceinline__ uint32_t packed_meta_lane(const QView &, int, int) { return 0u; }
+    __device__ static __forceinline__ uint32_t packed_meta_step(const QView &, int) { return 0u; }
+    __device__ static __forceinline__ void load_meta_at(const uint8_t *, uint32_t *sb) { sb[0] = 0u; }
+    __device__ static __forceinline__ Meta meta_from_raw(const uint32_t *) {
+        Meta m;
+        m.s = 1.0f;
+        m.b = 0.0f;
+        return m;
+    }
+    __device__ static __forceinline__ Meta meta_from_packed(const uint32_t *sb) { return meta_from_raw(sb); }
+    __device__ static __forceinline__ void decode_fast(const uint4 &raw, Meta, uint32_t *out /*[4]*/) {
+        out[0] = raw.x, out[1] = raw.y, out[2] = raw.z, out[3] = raw.w;
+    }
+    static constexpr int kPairState = 1;
+    __device__ static __forceinline__ Meta pair_meta(Meta m) { return m; }
+    __device__ static __forceinline__ void pair_state(uint32_t *) {}
+    __device__ static __forceinline__ void decode_pair(const uint4 &raw, Meta, int q, uint32_t *out, uint32_t *) {
+        out[q] = q == 0 ? raw.x : q == 1 ? raw.y : q == 2 ? raw.z : raw.w;
+    }
+};
+
 // dispatch a callable templated on the format: f.template operator()<Fmt>()
 template <typename F>
 inline int dispatch_format(const QView &q, F &&f) {

@@ -58,13 +58,14 @@ __device__ __forceinline__ void wide_tile(const GemmArgs &g, const Tile &t, uint
     // and ring, decode and the double-buffered decoded operands advance by chunk steps.
     constexpr int KV = Fmt::kVals, KSTEP = 64, NJ = 4, NT = 2;
     constexpr int CH = 32 / KV;           // chunk steps per step
-    static_assert(CH == 1 || CH == 2, "chunks of 32 or 16 values");
+    static_assert(CH == 1 || CH == 2 || CH == 4, "chunks of 32, 16 or 8 values");
     constexpr int NJC = NJ / CH;          // MFMA groups per chunk step
     constexpr int NUC = NJC * MT * NT;    // units (MFMAs) per chunk step
     constexpr int NPC = NT * (KV / 2);    // packed pairs to decode per chunk step
     // chunk steps held in registers (twice as many for tiles of at most 64 rows moved the 8-bit mixed batch by nothing)
-    constexpr int WRC = kWideWRing * CH;
-    static_assert(kWideRing % kWideWRing == 0, "ring slots must line up across trips");
+    // (unquantized weights: four chunk steps per step, so one step's worth keeps the ring at the 8-bit formats' size)
+    constexpr int WRC = CH == 4 ? CH : kWideWRing * CH;
+    static_assert(kWideRing % kWideWRing == 0 && (kWideRing * CH) % WRC == 0, "ring slots must line up across trips");
     const int tid = (int)threadIdx.x, lane = tid & 63, ln = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int cols = g.b0.cols, n_out = g.b0.rows;
@@ -391,6 +392,7 @@ static int wide_prepare_format() {
     return wide_raise_limit<Fmt, false>();
 }
 int qgemm_wide_prepare() {
+    DMOE_TRY(wide_prepare_format<FmtBf16>());
     DMOE_TRY(wide_prepare_format<FmtAffine4>());
     DMOE_TRY(wide_prepare_format<FmtAffine8>());
     DMOE_TRY(wide_prepare_format<FmtMxfp4>());
@@ -408,9 +410,13 @@ static int launch_wide(const GemmArgs &g, hipStream_t st) {
     return DMOE_OK;
 }
 
+bool qgemm_wide_bf16_supports(const QView &b) {
+    return b.mode == DMOE_QUANT_NONE && b.packed && b.cols % 64 == 0 && b.rows % 32 == 0 && ((uintptr_t)b.w % 16) == 0;
+}
+
 int launch_qgemm_wide(const GemmArgs &g, hipStream_t st) {
-    DMOE_REQUIRE(qgemm_wide_supports(g.b0), "wide MFMA GEMM: unsupported weight format or shape (rows=%d cols=%d)",
-                 g.b0.rows, g.b0.cols);
+    DMOE_REQUIRE(qgemm_wide_supports(g.b0) || qgemm_wide_bf16_supports(g.b0),
+                 "wide MFMA GEMM: unsupported weight format or shape (rows=%d cols=%d)", g.b0.rows, g.b0.cols);
     DMOE_REQUIRE(g.tile_m > 0 && g.tile_m <= kMfmaWideTileM && g.tile_m % 32 == 0, "wide MFMA GEMM: bad tile size %d",
                  g.tile_m);
     DMOE_REQUIRE(g.max_tiles >= 0 && g.max_tiles <= 65528, "wide MFMA GEMM: %d tiles exceed the grid limit", g.max_tiles);
@@ -422,6 +428,8 @@ int launch_qgemm_wide(const GemmArgs &g, hipStream_t st) {
                          g.b1.bits == g.b0.bits && g.b1.group == g.b0.group && g.b1.packed == g.b0.packed,
                      "wide MFMA GEMM: gate and up projections differ in shape or format");
     if (g.max_tiles == 0) return DMOE_OK;
+    if (g.b0.mode == DMOE_QUANT_NONE)
+        return g.gate_up ? launch_wide<FmtBf16, true>(g, st) : launch_wide<FmtBf16, false>(g, st);
     if (g.b0.mode == DMOE_QUANT_MXFP4)
         return g.gate_up ? launch_wide<FmtMxfp4, true>(g, st) : launch_wide<FmtMxfp4, false>(g, st);
     if (g.b0.mode == DMOE_QUANT_FP8_ROW)
