@@ -242,6 +242,7 @@ static int prefill_small_rows(const QView &b0, const QView &b1) {
 // `few` = few rows per expert (only read for unquantized weights; the quantized formats have `small`)
 static int run_gemm(const GemmArgs &g, bool small, hipStream_t st, int small_rows = 0, bool few = false) {
     if (g.b0.mode == DMOE_QUANT_NONE) {
+        if (small) return launch_qgemm_skinny(g, st); // few rows per expert on resident weights: the weight-streaming kernel
         // prefill sizes on resident weights: the matrix-core kernel with activations through LDS
         const bool wide = !few && qgemm_wide_bf16_supports(g.b0) && (!g.gate_up || qgemm_wide_bf16_supports(g.b1)) &&
                           g.tile_m % 32 == 0 && g.tile_m <= kMfmaWideTileM;

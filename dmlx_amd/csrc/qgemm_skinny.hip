@@ -578,6 +578,7 @@ __global__ __launch_bounds__(2 * kSkinnyWaves * 64) void qgemm_skinny_kernel(Gem
 }
 
 static int skinny_vals(const QView &b) {
+    if (b.mode == DMOE_QUANT_NONE) return 8;
     return (b.mode == DMOE_QUANT_AFFINE && b.bits == 4) || b.mode == DMOE_QUANT_MXFP4 ? 32 : 16;
 }
 static size_t skinny_lds_bytes(const QView &b) {
@@ -595,7 +596,9 @@ int qgemm_skinny_tile_m(const QView &b) {
 }
 
 bool qgemm_skinny_supports(const QView &b) {
-    return b.mode != DMOE_QUANT_NONE && b.cols % (2 * skinny_vals(b)) == 0 && skinny_lds_bytes(b) <= 150 * 1024;
+    // unquantized weights: resident (re-ordered) stacks only, whole 32-row blocks
+    if (b.mode == DMOE_QUANT_NONE && !(b.packed && b.rows % 32 == 0 && ((uintptr_t)b.w % 16) == 0)) return false;
+    return b.cols % (2 * skinny_vals(b)) == 0 && skinny_lds_bytes(b) <= 150 * 1024;
 }
 
 // rows of scales (and biases) that are 16-byte aligned and a whole number of 16-byte blocks long
@@ -631,6 +634,7 @@ static int skinny_prepare_format() {
     return skinny_raise_limit<Fmt, false, false, false>();
 }
 int qgemm_skinny_prepare() {
+    DMOE_TRY((skinny_raise_limit<FmtBf16, false, true, false>()));
     DMOE_TRY(skinny_prepare_format<FmtAffine4>());
     DMOE_TRY(skinny_prepare_format<FmtAffine8>());
     DMOE_TRY(skinny_prepare_format<FmtMxfp4>());
@@ -697,6 +701,7 @@ int launch_qgemm_skinny_pair(const GemmArgs &gu, const GemmArgs &dn, hipStream_t
                  "skinny GEMM pair: gate and up projections differ in shape or format");
     SkinnyLaunch l{gu, st};
     l.second = &dn;
+    if (gu.b0.mode == DMOE_QUANT_NONE) return l.template go<FmtBf16, false, true>();
     return dispatch_format(gu.b0, l);
 }
 
@@ -711,6 +716,7 @@ int launch_qgemm_skinny(const GemmArgs &g, hipStream_t st) {
                          g.b1.bits == g.b0.bits && g.b1.group == g.b0.group && g.b1.packed == g.b0.packed,
                      "skinny GEMM: gate and up projections differ in shape or format");
     if (g.max_tiles == 0) return DMOE_OK;
+    if (g.b0.mode == DMOE_QUANT_NONE) return SkinnyLaunch{g, st}.template go<FmtBf16, false, true>();
     return dispatch_format(g.b0, SkinnyLaunch{g, st});
 }
 
