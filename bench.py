@@ -235,6 +235,58 @@ def time_gather_qmm(torch, steps, windows):
     return out
 
 
+def time_float_arm(torch, steps, windows):
+    """The same step on UNQUANTIZED (bf16) experts, the `is_quantized == false` arm of dispatchGatherMm
+    (deepseek_v4.zig:978, ops.gatherMm): configurations 1 and 3 with their seeded routing, the routed experts replaced
+    by bf16 matrices drawn like the quantized ones (no shared expert). Decode: GB/s of the live experts' weights over
+    the whole step; prefill: TFLOP/s of the three GEMMs over the whole step."""
+    from dmlx_amd import capi, workloads
+
+    out = []
+    for config in (1, 3):
+        wl = workloads.make(config, device="cuda")
+        del wl.gate, wl.up, wl.down
+        wl.shared = None
+        torch.cuda.empty_cache()
+        gate, up, down = workloads._experts(wl.E, wl.D, wl.F, "bf16", workloads._gen(90 + config, "cuda"), "cuda")
+        layer = capi.Layer(wl.D, wl.F, wl.K, gate, up, down, swiglu_limit=wl.swiglu_limit,
+                           score_before_down=wl.score_before_down, shared=None, remap=wl.remap)
+        del gate, up, down      # the layer holds its own resident copy
+        torch.cuda.empty_cache()
+        ws = capi.Workspace(1 << 30)
+        res = torch.empty((wl.T, wl.D), dtype=torch.bfloat16, device="cuda")
+        step = lambda: layer.layer_forward(wl.x, wl.scores, wl.bias, wl.resident_mask, wl.renorm, wl.route_scale, ws, out=res)
+        _, idx, _ = layer.layer_forward(wl.x, wl.scores, wl.bias, wl.resident_mask, wl.renorm, wl.route_scale, ws,
+                                        want_routing=True)
+        live = int(torch.unique(idx).numel())
+        for _ in range(max(steps, 20)):
+            step()
+        torch.cuda.synchronize()
+        ms = []
+        for _ in range(windows):
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                step()
+            torch.cuda.synchronize()
+            ms.append((time.perf_counter() - t0) * 1e3 / steps)
+        ws.check()
+        m = statistics.median(ms)
+        wbytes = live * 3 * wl.D * wl.F * 2
+        flops = 2.0 * wl.T * wl.K * 3 * wl.D * wl.F
+        row = {"workload": f"shapes and routing of configuration {config}, bf16 experts, no shared expert", "tokens": wl.T, "live_experts": live,
+               "ms_per_step": m, "weight_bytes": wbytes, "flops": flops}
+        if config == 1:
+            row.update({"GBs": wbytes / (m * 1e-3) / 1e9, "frac_of_hbm_peak": wbytes / (m * 1e-3) / 1e9 / HBM_PEAK_GBS})
+        else:
+            row.update({"TFLOPs": flops / (m * 1e-3) / 1e12, "frac_of_mfma_peak": flops / (m * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS})
+        out.append(row)
+        layer.close()
+        ws.close()
+        del layer, ws, wl
+        torch.cuda.empty_cache()
+    return out
+
+
 def run_config(torch, config, steps, warmup, windows, settle_ms, copy_probe=False, score_before_down=False):
     """Builds configuration `config`, times it as the module docstring says and returns (workload, timing, analysis
     inputs). The layer and its workspace are released before returning."""
@@ -416,7 +468,7 @@ def main():
                     help="1: routing weight applied to the activation before the down projection (DSV4SwitchGLU.forward); "
                          "0: to the expert outputs (expert provider paths)")
     ap.add_argument("--no-prefill", action="store_true", help="with --config 1: do not also time configurations 3, 2 and 4")
-    ap.add_argument("--no-gate", action="store_true", help="do not also time the router (DSV4Gate.forward) in front of the step and the gatherQmm leaf operator")
+    ap.add_argument("--no-gate", action="store_true", help="do not also time the router (DSV4Gate.forward) in front of the step, the gatherQmm leaf operator and the step on unquantized experts")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-peaks", action="store_true", help="skip the library copy / GEMM reference measurements")
     ap.add_argument("--copy-probe", action="store_true",
@@ -470,6 +522,7 @@ def main():
     if not args.no_gate:
         result["gate"] = time_gate(torch, args.steps, args.windows)
         result["gather_qmm"] = time_gather_qmm(torch, args.steps, args.windows)
+        result["float_arm"] = time_float_arm(torch, args.steps, args.windows)
     print(json.dumps(result))
 
 
