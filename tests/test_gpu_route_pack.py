@@ -140,9 +140,11 @@ def test_pack_bit_exact(dmoe, orc, ws, T, K, E):
     np.testing.assert_array_equal(to_np_u32(got["live"])[:n_live], uniq)
 
 
-def test_expand_reduce_match_oracle(dmoe, orc):
+@pytest.mark.parametrize("T,K,D", [(37, 6, 200),      # rows of whole 16-byte pieces: the vector kernels
+                                   (5, 3, 37),        # ragged rows: one element per thread
+                                   (300, 8, 4100)])   # f32 rows in pieces, bf16 rows ragged (4100 = 4 * 1025)
+def test_expand_reduce_match_oracle(dmoe, orc, T, K, D):
     rng = np.random.default_rng(9)
-    T, K, D = 37, 6, 200
     x = rng.standard_normal((T, D)).astype(np.float32)
     w = rng.random((T, K)).astype(np.float32)
     ex = dmoe.expand_tokens(_dev(x), K)
