@@ -350,7 +350,7 @@ int dmoe_moe_layer_forward(uint16_t *d_out, uint32_t *d_out_indices, float *d_ou
  * until the process ends), so the call makes no hipMalloc / hipFree and creates no stream or event. Differences from
  * dmoe_moe_layer_forward:
  *   - a batch whose buffers do not fit is rejected with DMOE_ERR_INVALID and a message naming the size (at D = 4096,
- *     F = 2048, K = 6 with a folded shared expert: up to 195 tokens);
+ *     F = 2048, K = 6 with a folded shared expert: up to 194 tokens);
  *   - gate/up and down always run as two launches and a shared expert of another format runs after them on the same
  *     stream, so nothing waits inside a kernel; results are bit-identical;
  *   - there is no dmoe_workspace_check for this entry point and none is needed: the two conditions that check reports
