@@ -56,13 +56,15 @@ __global__ void remap_kernel(uint32_t *__restrict__ out, const int32_t *__restri
     out[i] = e < n_total ? (uint32_t)remap[e] : 0u;
 }
 
-// out[(t*K+k), :] = x[t, :], 16 bytes per thread
+// out[(t*K+k), :] = x[t, :]: one thread per 16 bytes of x, read once and stored K times
 __global__ void expand_kernel(uint4 *__restrict__ out, const uint4 *__restrict__ x, size_t row_vecs,
-                              int K, size_t total_vecs) {
+                              int K, size_t in_vecs) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= total_vecs) return;
-    size_t row = i / row_vecs, c = i - row * row_vecs;
-    out[i] = x[(row / (size_t)K) * row_vecs + c];
+    if (i >= in_vecs) return;
+    const size_t t = i / row_vecs, c = i - t * row_vecs;
+    const uint4 v = x[i];
+    uint4 *o = out + t * (size_t)K * row_vecs + c;
+    for (int k = 0; k < K; ++k) o[(size_t)k * row_vecs] = v;
 }
 __global__ void expand_kernel_bytes(uint8_t *__restrict__ out, const uint8_t *__restrict__ x,
                                     size_t row_bytes, int K, size_t total) {
@@ -156,7 +158,7 @@ int dmoe_expand_tokens(void *d_out, const void *d_x, int T, int D, int K, int el
     DMOE_REQUIRE(d_out && d_x, "expand: null pointer");
     size_t row_bytes = (size_t)D * elem_size;
     if (row_bytes % 16 == 0 && ((uintptr_t)d_out % 16 == 0) && ((uintptr_t)d_x % 16 == 0)) {
-        size_t rv = row_bytes / 16, total = rv * (size_t)T * K;
+        size_t rv = row_bytes / 16, total = rv * (size_t)T;
         hipLaunchKernelGGL(expand_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, to_hip(s),
                            (uint4 *)d_out, (const uint4 *)d_x, rv, K, total);
     } else {
