@@ -210,6 +210,9 @@ struct GemmArgs {
     // a launch serves the tiles with min_rows <= nrows <= max_rows of the list (prefill: the matrix-core kernels take the
     // large tiles, the weight-streaming kernel the small ones)
     int min_rows = 0, max_rows = 0x7fffffff;
+    // weight-streaming kernel, launches of a handful of tiles: the reduction of a tile split over two groups of
+    // wavefronts (see qgemm_skinny_ksplit_ok: packed layout, tiles of at most 8 rows)
+    int ksplit = 0;
     // Paired launch (gate/up and down of a decode step in ONE launch): the workgroups of a gate/up tile add 1 to
     // tile_done[tile] after their stores, a down workgroup of that tile waits for tile_done_target before it reads h.
     uint32_t *tile_done = nullptr;
@@ -236,6 +239,7 @@ bool qgemm_skinny_supports(const QView &b);
 // unquantized bf16 weights (DMOE_QUANT_NONE): one kernel for every size
 bool gemm_bf16_supports(const QView &b);
 int launch_gemm_bf16(const GemmArgs &g, hipStream_t st);
+bool qgemm_skinny_ksplit_ok(const QView &b); // the shape allows GemmArgs::ksplit
 int qgemm_skinny_tile_m(const QView &b);  // rows per tile to build tile lists with for the skinny path
 bool qgemm_mfma_supports(const QView &b);
 bool qgemm_wide_supports(const QView &b);

@@ -180,6 +180,11 @@ __global__ void combine_kernel(uint16_t *__restrict__ out, const uint16_t *__res
 // the weight-streaming kernel gives 4.1 / 4.0 against the matrix-core kernel's 3.5 / 3.6 (4-bit affine), 4.5 / 4.3 against
 // 4.4 / 4.3 (MXFP4), 5.3 / 5.3 against 5.2 / 5.2 (8-bit); at 24 and 32 rows the matrix-core kernel is level or ahead.
 constexpr int kSkinnyAvgRows = 16;
+// Up to this many sorted rows (hence tiles) in a decode step the weight-streaming launch leaves most of the chip's
+// workgroup slots empty (32 workgroups per tile, 512 slots): each tile's reduction is then split over twice the
+// workgroups (GemmArgs::ksplit), on tiles of one row block.
+constexpr int kSplitMaxTiles = 8;
+constexpr int kSplitTileM = 8;
 constexpr int kSharedSkinnyRows = 64;
 
 static bool few_rows(size_t rows, int n_experts) { return rows <= (size_t)kSkinnyAvgRows * (size_t)n_experts; }
@@ -191,6 +196,7 @@ struct FwdLayout {
     size_t h, y, sh_h, sh_y, total;
     int max_tiles, tile_m;
     bool small;
+    bool ksplit; // a handful of tiles of at most 8 rows: the weight-streaming kernel splits each tile's reduction in two
     bool fold; // the shared expert rides in the routed launches: T more sorted rows behind the T*K routed ones
 };
 
@@ -204,6 +210,12 @@ static FwdLayout forward_layout(const Layer *L, int T, bool with_shared = true) 
                        : std::min(qgemm_mfma_tile_m(L->gate.view), qgemm_mfma_tile_m(L->down.view));
     f.fold = with_shared && f.small && L->shared_folded;
     const size_t rows = n + (f.fold ? (size_t)T : 0); // sorted rows of the GEMMs
+    // single-stream decode: at most kSplitMaxTiles tiles even if every row goes to another expert
+    f.ksplit = f.small && rows <= (size_t)kSplitMaxTiles && qgemm_skinny_ksplit_ok(L->gate.view) &&
+               qgemm_skinny_ksplit_ok(L->up.view) && qgemm_skinny_ksplit_ok(L->down.view) &&
+               (!f.fold || (qgemm_skinny_ksplit_ok(L->sgate.view) && qgemm_skinny_ksplit_ok(L->sup.view) &&
+                            qgemm_skinny_ksplit_ok(L->sdown.view)));
+    if (f.ksplit) f.tile_m = kSplitTileM;
     f.max_tiles = pack_max_tiles(n, L->E, f.tile_m) + (f.fold ? ceil_div(T, f.tile_m) : 0);
     f.order = b.take(rows * 4);
     f.inv = b.take(n * 4);
@@ -300,6 +312,7 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     gu.n_tiles = po.n_tiles;
     gu.max_tiles = f.max_tiles;
     gu.tile_m = f.tile_m;
+    gu.ksplit = f.ksplit ? 1 : 0;
     gu.swiglu_limit = L->swiglu_limit;
     gu.swiglu_limit_dense = L->shared_swiglu_limit;
     if (L->score_before_down && d_scores) {
@@ -317,6 +330,7 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     dn.n_tiles = po.n_tiles;
     dn.max_tiles = f.max_tiles;
     dn.tile_m = f.tile_m;
+    dn.ksplit = f.ksplit ? 1 : 0;
 
     // Decode sizes: both GEMMs in one launch; a down workgroup waits for its own tile's gate/up workgroups only, so
     // the down projection fills the chip while the last gate/up workgroups drain (timed as the gate/up stage).

@@ -116,12 +116,20 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
     const int cols = g.b0.cols, n_out = g.b0.rows;
     const int n_steps = cols / KSTEP;
     const size_t e = t.expert;
+    // Few tiles in the launch (a decode step of one or two sequences): the launch cannot fill the chip, every SIMD has
+    // one wavefront, and that wavefront's chain of dependent steps sets the time. The reduction of a tile is then cut
+    // in two: wavefronts 0-3 take the first half of the steps and 4-7 the second half for HALF as many weight rows
+    // per workgroup (twice the workgroups), and the halves meet through LDS before the epilogue. Packed layout and
+    // tiles of one row block only (the launcher builds no larger tiles then).
+    const bool ks = PACKED && !MBLK && RJT == 1 && g.ksplit != 0;
+    const int kh = ks ? wave >> 2 : 0, wq = ks ? wave & 3 : wave; // reduction half, wavefront within the half
+    const int n_loc = ks ? n_steps >> 1 : n_steps, sb0 = kh * n_loc; // this wavefront's steps: sb0 .. sb0 + n_loc - 1
 
     // ---- this lane's weight row ------------------------------------------------------------------------
     // A wavefront past the last block of weight rows repeats that block (and stores nothing): every wavefront
     // of the workgroup then runs the same control flow, which the barriers below rely on.
-    const int proj = gate_up ? (wave & 1) : 0;      // gate/up: even wavefronts take gate rows, odd ones up rows
-    const int col_raw = ((int)blockIdx.x * cg + (gate_up ? wave >> 1 : wave)) * 32;
+    const int proj = gate_up ? (wq & 1) : 0;        // gate/up: even wavefronts take gate rows, odd ones up rows
+    const int col_raw = ((int)blockIdx.x * (ks ? cg >> 1 : cg) + (gate_up ? wq >> 1 : wq)) * 32;
     const QView &qv = proj ? g.b1 : g.b0;           // this wavefront's matrix stack
     const int col_last = ((n_out - 1) >> 5) << 5;
     const int col0 = col_raw < n_out ? col_raw : col_last;
@@ -156,8 +164,8 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
         }
 #pragma unroll
         for (int mi = 0; mi < NM; ++mi) {
-            s.raw[mi] = cs[mi].load_chunk_stream(step);
-            if (!MBLK) cs[mi].load_meta(qv, step, s.sb[mi]);
+            s.raw[mi] = cs[mi].load_chunk_stream(step + sb0);
+            if (!MBLK) cs[mi].load_meta(qv, step + sb0, s.sb[mi]);
         }
     };
     // ---- blocks of scale / bias entries (MBLK) -------------------------------------------------------------
@@ -271,7 +279,7 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
         // wavefront polls, the barrier holds the others), then fetch the rows
 #pragma unroll
         for (int j = 0; j < PRE; ++j)
-            if (j < n_steps) load_stage(j, ring[j], j % LG);
+            if (j < n_loc) load_stage(j, ring[j], j % LG);
         if (wave == 0) {
             uint32_t polls = 0;
             while (__hip_atomic_load(&g.tile_done[slot], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < g.tile_done_target &&
@@ -297,9 +305,9 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
         for (int mi = 0; mi < NM; ++mi) cs[mi].pin(); // keeps the weight loads behind the requests above
 #pragma unroll
         for (int j = 0; j < PRE; ++j)
-            if (j < n_steps) load_stage(j, ring[j], j % LG);
+            if (j < n_loc) load_stage(j, ring[j], j % LG);
         // every ring stage holds at least NM loads younger than the activation requests
-        if (n_steps >= PRE) __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt(PRE * NM));
+        if (n_loc >= PRE) __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt(PRE * NM));
         else __builtin_amdgcn_s_waitcnt(skinny_wait_vmcnt(0));
     }
     __syncthreads();
@@ -329,8 +337,8 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
         // One step: decode every projection's chunk first, then issue the matrix instructions of the projections
         // alternately (independent accumulation chains), then apply the scales. `xs` = step within the span.
         auto consume = [&](int gstep, int p8, int xs, const SkinnyStage<NM> &s) {
-            const uint8_t *xstep = xlane + (size_t)xs * KSTEP * 2;
-            const float *gs_step = gs_lds + xs * rp + 4 * h;
+            const uint8_t *xstep = xlane + (size_t)(xs + sb0) * KSTEP * 2;
+            const float *gs_step = gs_lds + (xs + sb0) * rp + 4 * h;
             Meta meta[NM];
             if (MBLK) {
                 uint32_t sbm[NM][2];
@@ -421,12 +429,12 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
             turn_write(0);
 #pragma unroll
             for (int i = 0; i < LG; ++i) // the stages of group 0 are free again: the group one round on
-                load_stage(STAGES + i < n_steps ? STAGES + i : n_steps - LG + i, ring[i], i);
+                load_stage(STAGES + i < n_loc ? STAGES + i : n_loc - LG + i, ring[i], i);
         }
 
         // whole rounds of the ring run without guards (the look-ahead is clamped onto the last step: a few repeated
         // loads at the very end instead of a branch per step); a partial last round runs the guarded copy
-        const int full = n_steps / ROUND * ROUND;
+        const int full = n_loc / ROUND * ROUND;
         int x0 = 0, next_span = span_steps; // first step of the span in LDS, first step of the next one
 #pragma unroll 1
         for (int s0 = 0; s0 < full; s0 += ROUND) {
@@ -453,33 +461,33 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
                         turn_write((j + LG) % STAGES); // the next group; its stages then take the loads a round later
 #pragma unroll
                         for (int i = 0; i < LG; ++i) // past the end: the last group again (unused)
-                            load_stage(ahead + LG + i < n_steps ? ahead + LG + i : n_steps - LG + i, ring[(j + LG) % STAGES + i], i);
+                            load_stage(ahead + LG + i < n_loc ? ahead + LG + i : n_loc - LG + i, ring[(j + LG) % STAGES + i], i);
                     }
                     turned.raw[0] = turned_raw[j % LG];
                     consume(step, j & 7, step - x0, turned);
                     continue;
                 }
-                load_stage(ahead < n_steps ? ahead : n_steps - 1, ring[(j + PRE) % STAGES]);
+                load_stage(ahead < n_loc ? ahead : n_loc - 1, ring[(j + PRE) % STAGES]);
                 consume(step, j & 7, step - x0, ring[j % STAGES]);
             }
         }
-        if (RJT == 1 && full < n_steps) { // only tiles of one row block get here (larger ones need whole rounds per span)
+        if (RJT == 1 && full < n_loc) { // only tiles of one row block get here (larger ones need whole rounds per span)
 #pragma unroll
             for (int j = 0; j < ROUND; ++j) {
                 const int step = full + j;
                 if (GROUPED) { // the reduction is a whole number of groups, and everything left is already in the ring
-                    if (step < n_steps) {
+                    if (step < n_loc) {
                         if (j % LG == 0) {
                             turn_read();
-                            if (step + LG < n_steps) turn_write((j + LG) % STAGES);
+                            if (step + LG < n_loc) turn_write((j + LG) % STAGES);
                         }
                         turned.raw[0] = turned_raw[j % LG];
                         consume(step, j & 7, step, turned);
                     }
                     continue;
                 }
-                if (step + PRE < n_steps) load_stage(step + PRE, ring[(j + PRE) % STAGES]);
-                if (step < n_steps) consume(step, j & 7, step, ring[j % STAGES]);
+                if (step + PRE < n_loc) load_stage(step + PRE, ring[(j + PRE) % STAGES]);
+                if (step < n_loc) consume(step, j & 7, step, ring[j % STAGES]);
             }
         }
 
@@ -491,12 +499,22 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
 #pragma unroll
             for (int r = 0; r < 4 * RJT; ++r) v[mi][r] = (FACTORED ? facc[mi][r] : acc[mi][r]) * rs;
         }
+        if (ks) { // the second half of the reduction joins the first (RJT == 1 here: four values per lane)
+            float4 *kx = (float4 *)xs_lds + 256 * RJT + wq * 64 + lane; // behind the gate/up exchange area below
+            __syncthreads(); // every wavefront has left the main loop: the activation window is free
+            if (kh == 1) kx[0] = make_float4(v[0][0], v[0][1], v[0][2], v[0][3]);
+            __syncthreads();
+            if (kh == 0) {
+                const float4 u = kx[0];
+                v[0][0] += u.x, v[0][1] += u.y, v[0][2] += u.z, v[0][3] += u.w;
+            }
+        }
         if (gate_up) {
             // the up wavefront hands its values to the gate wavefront of the same weight rows, through the
             // activation window (free once every wavefront has left the main loop)
-            float4 *xch = (float4 *)xs_lds + ((wave >> 1) * 64 + lane) * RJT;
+            float4 *xch = (float4 *)xs_lds + ((wq >> 1) * 64 + lane) * RJT;
             __syncthreads();
-            if (proj == 1) {
+            if (proj == 1 && kh == 0) {
 #pragma unroll
                 for (int j = 0; j < RJT; ++j) xch[j] = make_float4(v[0][4 * j], v[0][4 * j + 1], v[0][4 * j + 2], v[0][4 * j + 3]);
             }
@@ -509,7 +527,7 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
                 }
             }
         }
-        const bool storer = store_on && proj == 0;
+        const bool storer = store_on && proj == 0 && kh == 0;
         const float swiglu_limit = (t.flags & kTileDense) ? g.swiglu_limit_dense : g.swiglu_limit;
 #pragma unroll
         for (int j = 0; j < RJT; ++j) {
@@ -556,7 +574,7 @@ __global__ __launch_bounds__(2 * kSkinnyWaves * 64) void qgemm_skinny_kernel(Gem
     (void)b;
     const uint32_t slot = blockIdx.y - (second ? (uint32_t)a.max_tiles : 0u);
     const int sync = !paired ? kSkinnySyncNone : second ? kSkinnySyncWait : kSkinnySyncSignal;
-    if ((int)blockIdx.x * (g.gate_up ? 1 : 2) * kSkinnyWaves * 32 >= g.b0.rows) return; // the grid is sized for the wider role
+    if ((int)blockIdx.x * (g.gate_up ? 1 : 2) * kSkinnyWaves * 32 >= (g.ksplit ? 2 : 1) * g.b0.rows) return; // the grid is sized for the wider role
     Tile t;
     if (g.tiles) {
         const uint32_t n_tiles = *g.n_tiles; // both loads are issued before either is needed
@@ -599,6 +617,15 @@ bool qgemm_skinny_supports(const QView &b) {
     // unquantized weights: resident (re-ordered) stacks only, whole 32-row blocks
     if (b.mode == DMOE_QUANT_NONE && !(b.packed && b.rows % 32 == 0 && ((uintptr_t)b.w % 16) == 0)) return false;
     return b.cols % (2 * skinny_vals(b)) == 0 && skinny_lds_bytes(b) <= 150 * 1024;
+}
+
+// GemmArgs::ksplit needs the packed layout, two halves of the reduction that are whole ring rounds and start on a
+// group boundary
+bool qgemm_skinny_ksplit_ok(const QView &b) {
+    if (!qgemm_skinny_supports(b) || !b.packed) return false;
+    const int n_steps = b.cols / (2 * skinny_vals(b));
+    if (n_steps % (2 * kSkinnyStages) != 0) return false;
+    return b.group <= 0 || (b.cols / 2) % b.group == 0;
 }
 
 // rows of scales (and biases) that are 16-byte aligned and a whole number of 16-byte blocks long
@@ -651,7 +678,7 @@ struct SkinnyLaunch {
         const size_t lds = skinny_lds_bytes(g.b0) + (MBLK ? kSkinnyTurnBytes : 0);
         DMOE_TRY((skinny_raise_limit<Fmt, FACTORED, PACKED, MBLK>())); // done by dmoe_init for its device; a flag test otherwise
         // 8 wavefronts per workgroup: 128 output columns of gate AND up, or 256 of a single projection
-        auto blocks_x = [](const GemmArgs &a) { return ceil_div(a.b0.rows, (a.gate_up ? 1 : 2) * kSkinnyWaves * 32); };
+        auto blocks_x = [](const GemmArgs &a) { return ceil_div((a.ksplit ? 2 : 1) * a.b0.rows, (a.gate_up ? 1 : 2) * kSkinnyWaves * 32); };
         dim3 block(2 * kSkinnyWaves * 64);
         if (second) {
             GemmArgs a = g, b = *second;
@@ -695,6 +722,9 @@ bool qgemm_skinny_pair_supports(const GemmArgs &gu, const GemmArgs &dn) {
 
 int launch_qgemm_skinny_pair(const GemmArgs &gu, const GemmArgs &dn, hipStream_t st) {
     DMOE_REQUIRE(qgemm_skinny_pair_supports(gu, dn), "skinny GEMM pair: arguments do not form a gate/up + down pair");
+    DMOE_REQUIRE(gu.ksplit == dn.ksplit && (!gu.ksplit || (gu.tile_m <= kSkinnyRowBlock && qgemm_skinny_ksplit_ok(gu.b0) &&
+                                                           qgemm_skinny_ksplit_ok(gu.b1) && qgemm_skinny_ksplit_ok(dn.b0))),
+                 "skinny GEMM pair: a split reduction needs packed weights and tiles of at most %d rows", kSkinnyRowBlock);
     DMOE_REQUIRE(gu.a && gu.out && dn.out && ((uintptr_t)gu.a % 16) == 0 && ((uintptr_t)dn.a % 16) == 0, "skinny GEMM pair: bad pointer");
     DMOE_REQUIRE(gu.b1.rows == gu.b0.rows && gu.b1.cols == gu.b0.cols && gu.b1.mode == gu.b0.mode && gu.b1.bits == gu.b0.bits &&
                      gu.b1.group == gu.b0.group && gu.b1.packed == gu.b0.packed,
@@ -715,6 +745,8 @@ int launch_qgemm_skinny(const GemmArgs &g, hipStream_t st) {
         DMOE_REQUIRE(g.b1.rows == g.b0.rows && g.b1.cols == g.b0.cols && g.b1.mode == g.b0.mode &&
                          g.b1.bits == g.b0.bits && g.b1.group == g.b0.group && g.b1.packed == g.b0.packed,
                      "skinny GEMM: gate and up projections differ in shape or format");
+    DMOE_REQUIRE(!g.ksplit || (g.tile_m <= kSkinnyRowBlock && qgemm_skinny_ksplit_ok(g.b0) && (!g.gate_up || qgemm_skinny_ksplit_ok(g.b1))),
+                 "skinny GEMM: a split reduction needs packed weights and tiles of at most %d rows", kSkinnyRowBlock);
     if (g.max_tiles == 0) return DMOE_OK;
     if (g.b0.mode == DMOE_QUANT_NONE) return SkinnyLaunch{g, st}.template go<FmtBf16, false, true>();
     return dispatch_format(g.b0, SkinnyLaunch{g, st});
