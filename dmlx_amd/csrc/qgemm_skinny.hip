@@ -84,7 +84,7 @@ constexpr size_t kSkinnyTurnBytes = (size_t)2 * kSkinnyWaves * 4 * 1024;
 // MBLK (MLX layout only): the scale / bias entries of a row are not fetched one per step (32 cache lines touched per
 // load for 2 useful bytes each, again at every step: these loads, not the weights, bounded the MLX-layout path) but 16
 // bytes at a time - eight bf16 or sixteen E8M0 entries, the next block requested while the current one is in use.
-template <typename Fmt, bool FACTORED, bool PACKED, int RJT, bool MBLK>
+template <typename Fmt, bool FACTORED, bool PACKED, int RJT, bool MBLK, bool KSPLIT = false>
 __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, uint8_t *skinny_lds, const bool gate_up,
                                             const int sync, const uint32_t slot) {
     using CS = ChunkStream<Fmt, PACKED>;
@@ -121,7 +121,8 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
     // in two: wavefronts 0-3 take the first half of the steps and 4-7 the second half for HALF as many weight rows
     // per workgroup (twice the workgroups), and the halves meet through LDS before the epilogue. Packed layout and
     // tiles of one row block only (the launcher builds no larger tiles then).
-    const bool ks = PACKED && !MBLK && RJT == 1 && g.ksplit != 0;
+    static_assert(!KSPLIT || (PACKED && !MBLK && RJT == 1), "the split reduction exists for packed one-row-block tiles");
+    constexpr bool ks = KSPLIT; // a kernel of its own: the other instantiations carry none of this
     const int kh = ks ? wave >> 2 : 0, wq = ks ? wave & 3 : wave; // reduction half, wavefront within the half
     const int n_loc = ks ? n_steps >> 1 : n_steps, sb0 = kh * n_loc; // this wavefront's steps: sb0 .. sb0 + n_loc - 1
 
@@ -559,7 +560,7 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
 // y < a.max_tiles are the gate/up tiles, the next a.max_tiles the down tiles of the same list. The hardware starts
 // workgroups in index order, so every producer of a tile is running or done by the time a consumer of it starts to
 // wait; the down workgroups that become resident while the last gate/up workgroups drain stream their weights meanwhile.
-template <typename Fmt, bool FACTORED, bool PACKED, bool MBLK = false>
+template <typename Fmt, bool FACTORED, bool PACKED, bool MBLK = false, bool KSPLIT = false>
 __global__ __launch_bounds__(2 * kSkinnyWaves * 64) void qgemm_skinny_kernel(GemmArgs a, GemmArgs b, int paired) {
     extern __shared__ __attribute__((aligned(16))) uint8_t skinny_lds[];
     const bool second = paired && blockIdx.y >= (uint32_t)a.max_tiles; // workgroup-uniform
@@ -574,7 +575,7 @@ __global__ __launch_bounds__(2 * kSkinnyWaves * 64) void qgemm_skinny_kernel(Gem
     (void)b;
     const uint32_t slot = blockIdx.y - (second ? (uint32_t)a.max_tiles : 0u);
     const int sync = !paired ? kSkinnySyncNone : second ? kSkinnySyncWait : kSkinnySyncSignal;
-    if ((int)blockIdx.x * (g.gate_up ? 1 : 2) * kSkinnyWaves * 32 >= (g.ksplit ? 2 : 1) * g.b0.rows) return; // the grid is sized for the wider role
+    if ((int)blockIdx.x * (g.gate_up ? 1 : 2) * kSkinnyWaves * 32 >= (KSPLIT ? 2 : 1) * g.b0.rows) return; // the grid is sized for the wider role
     Tile t;
     if (g.tiles) {
         const uint32_t n_tiles = *g.n_tiles; // both loads are issued before either is needed
@@ -588,6 +589,10 @@ __global__ __launch_bounds__(2 * kSkinnyWaves * 64) void qgemm_skinny_kernel(Gem
         if ((int)t.row0 >= g.dense_rows) return;
         uint32_t left = (uint32_t)g.dense_rows - t.row0;
         t.nrows = left < (uint32_t)g.tile_m ? left : (uint32_t)g.tile_m;
+    }
+    if (KSPLIT) { // the launcher builds no tile above one row block for this kernel
+        skinny_tile<Fmt, FACTORED, PACKED, 1, MBLK, KSPLIT>(g, t, skinny_lds, g.gate_up, sync, slot);
+        return;
     }
     if (__builtin_amdgcn_readfirstlane((int)t.nrows) <= kSkinnyRowBlock)
         skinny_tile<Fmt, FACTORED, PACKED, 1, MBLK>(g, t, skinny_lds, g.gate_up, sync, slot);
@@ -643,10 +648,10 @@ static bool mlx_meta_blocks(const QView &b) {
            (!b.biases || ((uintptr_t)b.biases % 16) == 0);
 }
 
-template <typename Fmt, bool FACTORED, bool PACKED, bool MBLK>
+template <typename Fmt, bool FACTORED, bool PACKED, bool MBLK, bool KSPLIT = false>
 static int skinny_raise_limit() {
     static LdsLimit limit; // per instantiation
-    return raise_lds_limit(limit, (const void *)qgemm_skinny_kernel<Fmt, FACTORED, PACKED, MBLK>, 150 * 1024);
+    return raise_lds_limit(limit, (const void *)qgemm_skinny_kernel<Fmt, FACTORED, PACKED, MBLK, KSPLIT>, 150 * 1024);
 }
 // the instantiations SkinnyLaunch can pick for one format
 template <typename Fmt>
@@ -655,6 +660,8 @@ static int skinny_prepare_format() {
     constexpr bool has_entries = Fmt::kMetaEntryBytes != 0;
     DMOE_TRY((skinny_raise_limit<Fmt, can_factor, true, false>()));
     DMOE_TRY((skinny_raise_limit<Fmt, false, true, false>()));
+    DMOE_TRY((skinny_raise_limit<Fmt, can_factor, true, false, true>()));
+    DMOE_TRY((skinny_raise_limit<Fmt, false, true, false, true>()));
     DMOE_TRY((skinny_raise_limit<Fmt, can_factor, false, has_entries>()));
     DMOE_TRY((skinny_raise_limit<Fmt, false, false, has_entries>()));
     DMOE_TRY((skinny_raise_limit<Fmt, can_factor, false, false>()));
@@ -662,6 +669,7 @@ static int skinny_prepare_format() {
 }
 int qgemm_skinny_prepare() {
     DMOE_TRY((skinny_raise_limit<FmtBf16, false, true, false>()));
+    DMOE_TRY((skinny_raise_limit<FmtBf16, false, true, false, true>()));
     DMOE_TRY(skinny_prepare_format<FmtAffine4>());
     DMOE_TRY(skinny_prepare_format<FmtAffine8>());
     DMOE_TRY(skinny_prepare_format<FmtMxfp4>());
@@ -672,11 +680,14 @@ struct SkinnyLaunch {
     const GemmArgs &g;
     hipStream_t st;
     const GemmArgs *second = nullptr; // paired launch: the down projection behind the gate/up GEMM `g`
-    template <typename Fmt, bool FACTORED, bool PACKED, bool MBLK = false>
+    template <typename Fmt, bool FACTORED, bool PACKED, bool MBLK = false, bool KSPLIT = false>
     int go() {
-        auto kern = qgemm_skinny_kernel<Fmt, FACTORED, PACKED, MBLK>;
+        if constexpr (PACKED && !MBLK && !KSPLIT) {
+            if (g.ksplit) return go<Fmt, FACTORED, PACKED, MBLK, true>(); // validated by the launch functions
+        }
+        auto kern = qgemm_skinny_kernel<Fmt, FACTORED, PACKED, MBLK, KSPLIT>;
         const size_t lds = skinny_lds_bytes(g.b0) + (MBLK ? kSkinnyTurnBytes : 0);
-        DMOE_TRY((skinny_raise_limit<Fmt, FACTORED, PACKED, MBLK>())); // done by dmoe_init for its device; a flag test otherwise
+        DMOE_TRY((skinny_raise_limit<Fmt, FACTORED, PACKED, MBLK, KSPLIT>())); // done by dmoe_init for its device; a flag test otherwise
         // 8 wavefronts per workgroup: 128 output columns of gate AND up, or 256 of a single projection
         auto blocks_x = [](const GemmArgs &a) { return ceil_div((a.ksplit ? 2 : 1) * a.b0.rows, (a.gate_up ? 1 : 2) * kSkinnyWaves * 32); };
         dim3 block(2 * kSkinnyWaves * 64);
