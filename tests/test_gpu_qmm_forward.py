@@ -566,6 +566,37 @@ def test_layer_with_a_hidden_size_that_is_not_a_power_of_two(dmoe, orc, ws, fmt,
     _check_layer(dmoe, orc, ws, wl)
 
 
+@pytest.mark.parametrize("fmt", ["affine4", "affine4g32", "affine4g128", "affine8", "mxfp4", "fp8row", "bf16"])
+def test_single_sequence_decode_step(dmoe, orc, ws, fmt):
+    """Steps of at most 8 sorted rows (one or two sequences): the weight-streaming kernel splits every tile's
+    reduction over two groups of wavefronts that meet in LDS. D = 2048 and F = 1024 are whole ring rounds per half
+    for every format, so the split kernel runs; D = 1536 is not (its steps do not halve into whole rounds for the
+    4-bit formats) and takes the unsplit kernel on the same rows. With a shared expert of the routed format (it rides
+    in the routed launch as one more row per token), of another format (a launch of its own), and none; both
+    positions of the routing weight; SwiGLU limits that clamp a fifth of the values (gate and up values have a
+    standard deviation of 0.9 here; limits far below that would shrink the activations, against which their error is
+    measured, a hundredfold while the 8-bit and the unfactored 4-bit decoders' bf16 weight rounding stays what it is)."""
+    E = 12
+    case = 0
+    for D, F in ((2048, 1024), (1536, 1024)):
+        routed = (_stack(fmt, E, F, D, 9001), _stack(fmt, E, F, D, 9002), _stack(fmt, E, D, F, 9003))
+        for T, K in ((1, 6), (1, 8), (2, 3), (2, 4), (3, 2)):
+            for sfmt in (fmt, None, "fp8row" if fmt != "fp8row" else "affine8"):
+                case += 1
+                if T * K + (T if sfmt == fmt else 0) > 8 and D != 2048:
+                    continue
+                g = torch.Generator(device="cuda").manual_seed(9100 + case)
+                x = torch.randn((T, D), generator=g, device="cuda").to(torch.bfloat16)
+                scores = torch.sigmoid(torch.randn((T, E), generator=g, device="cuda"))
+                shared = None if sfmt is None else (_stack(sfmt, 1, F, D, 9200 + case), _stack(sfmt, 1, F, D, 9300 + case),
+                                                    _stack(sfmt, 1, D, F, 9400 + case))
+                wl = workloads.Workload(f"single sequence {fmt} D={D} T={T} K={K} shared={sfmt}", T, D, F, E, E, K, x,
+                                        scores, None, None, None, True, 1.5, *routed, shared,
+                                        swiglu_limit=1.0 if case % 2 else 0.0, shared_swiglu_limit=0.5 if case % 3 == 0 else 0.0,
+                                        score_before_down=bool(case % 4 < 2))
+                _check_layer(dmoe, orc, ws, wl)
+
+
 def test_forward_edge_cases(dmoe, orc, ws):
     wl = workloads.make(1, scale=0.125)
     layer = dmoe.Layer(wl.D, wl.F, wl.K, wl.gate, wl.up, wl.down, swiglu_limit=wl.swiglu_limit, shared=wl.shared)
