@@ -55,7 +55,7 @@ class SafetensorsOptsC(C.Structure):
                 ("shared_swiglu_limit", C.c_float), ("resident_mask", C.c_void_p), ("n_experts_total", C.c_int)]
 
 
-SCORE_SOFTMAX, SCORE_SIGMOID, SCORE_SQRTSOFTPLUS = 0, 1, 2
+SCORE_SOFTMAX, SCORE_SIGMOID, SCORE_SQRTSOFTPLUS, SCORE_SQRTSOFTPLUS_STABLE = 0, 1, 2, 3
 
 # every symbol include/dmoe.h declares
 EXPORTS = [

@@ -340,6 +340,16 @@ __device__ __forceinline__ float det_logf(float x) {
     return fmaf(fe, 0.693359375f, r);
 }
 
+// softplus(x) = max(x, 0) + log1p(exp(-|x|)): log1p(u) for u in [0, 1] as log(w) * (u / (w - 1)) with w = 1 + u
+// rounded (the quotient undoes the rounding of w to first order), u itself where w rounds to 1. No overflow for large
+// x, no loss of the small results for very negative x.
+__device__ __forceinline__ float det_softplusf(float x) {
+    const float u = det_expf(-fabsf(x));
+    const float w = 1.0f + u;
+    const float l = w == 1.0f ? u : det_logf(w) * (u / (w - 1.0f));
+    return (x > 0.0f ? x : 0.0f) + l;
+}
+
 // One wavefront per token: adds the segment sums left to right, rounds the logit to bf16, applies the scoring
 // function and, with ROUTE, goes straight on to the selection (bias, Smelt mask, top-k, weights from the unbiased
 // scores, renormalisation, route scale: deepseek_v4.zig:589-678) with the scores still in registers, so they make no
@@ -416,7 +426,8 @@ __global__ __launch_bounds__(kGateWaves * 64) void gate_scores_kernel(float *__r
         for (int i = 0; i < EPL; ++i) {
             if (lane + 64 * i >= E) continue;
             if (scoring == DMOE_SCORE_SIGMOID) v[i] = 1.0f / (1.0f + det_expf(-v[i]));
-            else v[i] = sqrtf(det_logf(1.0f + det_expf(v[i]))); // the reference's literal form (:575-583)
+            else if (scoring == DMOE_SCORE_SQRTSOFTPLUS) v[i] = sqrtf(det_logf(1.0f + det_expf(v[i]))); // the reference's literal form (:575-583)
+            else v[i] = sqrtf(det_softplusf(v[i]));
         }
     }
     if (scores) {
@@ -482,7 +493,7 @@ int dmoe_gate_create(dmoe_gate *out, const dmoe_gate_desc *d, dmoe_stream s) {
     DMOE_REQUIRE(d->n_experts >= 1 && d->n_experts <= 1024 && d->top_k >= 1 && d->top_k <= d->n_experts,
                  "gate_create: bad expert count %d / top_k %d", d->n_experts, d->top_k);
     DMOE_REQUIRE(d->dim >= 8 && d->dim % 8 == 0, "gate_create: dim %d must be a positive multiple of 8", d->dim);
-    DMOE_REQUIRE(d->scoring_func >= DMOE_SCORE_SOFTMAX && d->scoring_func <= DMOE_SCORE_SQRTSOFTPLUS,
+    DMOE_REQUIRE(d->scoring_func >= DMOE_SCORE_SOFTMAX && d->scoring_func <= DMOE_SCORE_SQRTSOFTPLUS_STABLE,
                  "gate_create: unknown scoring function %d", d->scoring_func);
     DMOE_REQUIRE(d->weight_source == DMOE_WEIGHTS_COPY_FROM_HOST || d->weight_source == DMOE_WEIGHTS_COPY_FROM_DEVICE,
                  "gate_create: weight_source must be a copying one (the weight is re-ordered)");

@@ -204,7 +204,8 @@ struct SmeltConfig {      // deepseek_v4_loader.zig:250-294
 
 // ---- deepseek_v4.zig: gate epilogue, SwitchGLU, MoE ----------------------------------------------------------
 
-enum class ScoringFunc { softmax, sigmoid, sqrtsoftplus }; // deepseek_v4.zig:82-86
+// deepseek_v4.zig:82-86, plus sqrtsoftplus_stable (DMOE_SCORE_SQRTSOFTPLUS_STABLE: no counterpart in the reference)
+enum class ScoringFunc { softmax, sigmoid, sqrtsoftplus, sqrtsoftplus_stable };
 
 // DSV4Gate (deepseek_v4.zig:521-681). `forward(ctx, scores)` takes the result of the scoring function (the
 // gate epilogue, :589-678); once `load` has uploaded the router weight, `forwardHidden` serves the whole

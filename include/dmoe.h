@@ -373,7 +373,13 @@ int dmoe_moe_layer_forward_static(uint16_t *d_out, uint32_t *d_out_indices, floa
 typedef enum {
     DMOE_SCORE_SOFTMAX = 0,
     DMOE_SCORE_SIGMOID = 1,
-    DMOE_SCORE_SQRTSOFTPLUS = 2 /* sqrt(log(1 + exp(x))), the reference's default (:48) */
+    DMOE_SCORE_SQRTSOFTPLUS = 2, /* sqrt(log(1 + exp(x))), the reference's default (:48), literally as it computes it
+                                  * (:575-583): +inf from x = 88.73 on */
+    /* Not in the reference's enum: the same score through the overflow-free softplus max(x, 0) + log1p(exp(-|x|)) of
+     * the Python model the reference follows (its docs/en/deepseek-v4/remaining-deviations.md:10 lists the literal form
+     * as an open deviation from that). Equal to the literal form to rounding wherever that one is finite and above
+     * 1e-3; a caller opts in, the default stays the reference's arithmetic. */
+    DMOE_SCORE_SQRTSOFTPLUS_STABLE = 3
 } dmoe_scoring_func;
 
 /* DSV4Gate fields (deepseek_v4.zig:521-535). Pointers are host or device memory as `weight_source` says

@@ -129,9 +129,13 @@ void orc_gate_scores(const float *logits, int T, int E, int func, float *out) {
             for (int e = 0; e < E; e++) o[e] /= sum;
         } else if (func == ORC_SCORE_SIGMOID) {
             for (int e = 0; e < E; e++) o[e] = 1.0f / (1.0f + expf(-x[e]));
-        } else {
+        } else if (func == ORC_SCORE_SQRTSOFTPLUS) {
             /* the reference's literal form, overflow for large x included (:575-583) */
             for (int e = 0; e < E; e++) o[e] = sqrtf(logf(1.0f + expf(x[e])));
+        } else {
+            /* the stable softplus of the Python model the reference follows (logaddexp(x, 0) = max + log1p(exp(-|x|));
+             * docs/en/deepseek-v4/remaining-deviations.md:10 lists the literal form above as a deviation from it) */
+            for (int e = 0; e < E; e++) o[e] = sqrtf(fmaxf(x[e], 0.0f) + log1pf(expf(-fabsf(x[e]))));
         }
     }
 }
@@ -220,6 +224,19 @@ float orc_det_logf(float x) {
     return fmaf(fe, 0.693359375f, r);
 }
 
+/* softplus(x) = max(x, 0) + log1p(exp(-|x|)) in f32 from the two routines above. log1p(u) for u in [0, 1] is
+ * log(w) * (u / (w - 1)) with w = 1 + u rounded (the quotient undoes the rounding of w to first order), and u itself
+ * where w rounds to 1. No overflow for large x (the result is x), no loss of the small results for very negative x
+ * (the result is exp(x)). NaN passes through. Not part of the reference's Zig (which has the literal
+ * log(1 + exp(x)), deepseek_v4.zig:575-583); it is the form of the Python model that
+ * docs/en/deepseek-v4/remaining-deviations.md:10 names as the target. */
+float orc_det_softplusf(float x) {
+    float u = orc_det_expf(-fabsf(x));
+    float w = 1.0f + u;
+    float l = w == 1.0f ? u : orc_det_logf(w) * (u / (w - 1.0f));
+    return (x > 0.0f ? x : 0.0f) + l;
+}
+
 /* deepseek_v4.zig:567-585, op by op, with orc_det_expf / orc_det_logf in place of MLX's exp / log.
  * softmax (:569): exp(x - max) / sum, the sum taken as 64 strided partial sums (element e goes to
  * partial e mod 64, in increasing e) that are then folded by halves (p[i] += p[i + 32], 16, .. 1). */
@@ -241,8 +258,10 @@ void orc_gate_scores_det(const float *logits, int T, int E, int func, float *out
             for (int e = 0; e < E; e++) o[e] = o[e] / part[0];
         } else if (func == ORC_SCORE_SIGMOID) {
             for (int e = 0; e < E; e++) o[e] = 1.0f / (1.0f + orc_det_expf(-x[e]));
-        } else {
+        } else if (func == ORC_SCORE_SQRTSOFTPLUS) {
             for (int e = 0; e < E; e++) o[e] = sqrtf(orc_det_logf(1.0f + orc_det_expf(x[e])));
+        } else {
+            for (int e = 0; e < E; e++) o[e] = sqrtf(orc_det_softplusf(x[e]));
         }
     }
 }

@@ -50,7 +50,7 @@ extern "C" {
 #endif
 
 enum { ORC_AFFINE = 0, ORC_MXFP4 = 1, ORC_FP8_ROW = 2, ORC_NONE = 3 };
-enum { ORC_SCORE_SOFTMAX = 0, ORC_SCORE_SIGMOID = 1, ORC_SCORE_SQRTSOFTPLUS = 2 };
+enum { ORC_SCORE_SOFTMAX = 0, ORC_SCORE_SIGMOID = 1, ORC_SCORE_SQRTSOFTPLUS = 2, ORC_SCORE_SQRTSOFTPLUS_STABLE = 3 };
 enum { ORC_SMELT_UNIFORM = 0, ORC_SMELT_FIRST = 1 };
 
 /* One quantized matrix stack [n_mats, rows, cols] in MLX layout.
@@ -81,6 +81,7 @@ void orc_gate_logits(const uint16_t *x, const uint16_t *wg, int T, int D, int E,
 void orc_gate_scores_det(const float *logits, int T, int E, int func, float *scores_out);
 float orc_det_expf(float x);
 float orc_det_logf(float x);
+float orc_det_softplusf(float x);
 /* deepseek_v4.zig:589-678 (selection on biased/masked scores, weights from the
  * unbiased ones, renorm when not softmax, * route_scale) */
 void orc_gate_route(const float *scores, const float *bias, const uint8_t *resident,

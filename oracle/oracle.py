@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "_build", "libdmoe_oracle.so")
 
 AFFINE, MXFP4, FP8_ROW, NONE = 0, 1, 2, 3
-SCORE_SOFTMAX, SCORE_SIGMOID, SCORE_SQRTSOFTPLUS = 0, 1, 2
+SCORE_SOFTMAX, SCORE_SIGMOID, SCORE_SQRTSOFTPLUS, SCORE_SQRTSOFTPLUS_STABLE = 0, 1, 2, 3
 SMELT_UNIFORM, SMELT_FIRST = 0, 1
 
 
@@ -176,6 +176,12 @@ def det_expf(x):
 
 def det_logf(x):
     f = lib().orc_det_logf
+    f.restype = C.c_float
+    return np.array([f(C.c_float(float(v))) for v in np.asarray(x, np.float32).ravel()], np.float32)
+
+
+def det_softplusf(x):
+    f = lib().orc_det_softplusf
     f.restype = C.c_float
     return np.array([f(C.c_float(float(v))) for v in np.asarray(x, np.float32).ravel()], np.float32)
 

@@ -22,7 +22,7 @@ def _case(seed, T, D, E, with_bias, with_mask, spread):
     return x, wg, bias, mask
 
 
-@pytest.mark.parametrize("func", [0, 1, 2])
+@pytest.mark.parametrize("func", [0, 1, 2, 3])
 @pytest.mark.parametrize("T,D,E,K,with_bias,with_mask", [
     (64, 4096, 256, 6, True, False),     # decode shape of configuration 1: one reduction segment per wavefront
     (5, 200, 72, 3, True, True),         # short last segment, experts not a multiple of 64, Smelt mask
@@ -68,7 +68,8 @@ def test_gate_prefill_full_size_bit_exact(dmoe, orc, ws):
 
 
 def test_gate_extreme_logits(dmoe, orc, ws):
-    """Saturating inputs: sigmoid -> 0 / 1, softplus overflow of the reference's literal form (exp -> inf)."""
+    """Saturating inputs: sigmoid -> 0 / 1, softplus overflow of the reference's literal form (exp -> inf), and the
+    overflow-free variant on the same logits."""
     T, D, E = 4, 64, 64
     x = torch.full((T, D), 8.0, device="cuda").to(torch.bfloat16)
     wg = torch.zeros((E, D), device="cuda")
@@ -76,11 +77,15 @@ def test_gate_extreme_logits(dmoe, orc, ws):
     wg[1] = -0.25     # logit -128
     wg[2] = 0.0
     wg = wg.to(torch.bfloat16)
-    for func in (1, 2):
+    for func in (1, 2, 3):
         gate = dmoe.Gate(wg, 2, func)
         _, _, scores = gate.forward(x, ws, want_scores=True)
         want = orc.gate_scores_det(orc.gate_logits(bf16_bits(x), bf16_bits(wg)), func)
         np.testing.assert_array_equal(scores.cpu().numpy().view(np.uint32), want.view(np.uint32))
+        if func == 2:
+            assert bool(torch.isinf(scores[:, 0]).all())
+        if func == 3:   # the overflow-free softplus: sqrt(128) where the literal form gives infinity
+            assert bool((scores[:, 0] == 128.0 ** 0.5).all()) and bool(torch.isfinite(scores).all())
         gate.close()
 
 
@@ -139,7 +144,7 @@ def test_gate_logits_tiny_and_huge_magnitudes(dmoe, orc, ws, T):
     x, wg = x.to(torch.bfloat16), wg.to(torch.bfloat16)
     logits = orc.gate_logits(bf16_bits(x), bf16_bits(wg))
     assert np.isinf(logits).any() and (np.abs(logits[np.isfinite(logits)]) < 2.0 ** -126).any(), "the case must reach both ends"
-    for func in (1, 2):
+    for func in (1, 2, 3):
         gate = dmoe.Gate(wg, 4, func)
         _, _, scores = gate.forward(x, ws, want_scores=True)
         want = orc.gate_scores_det(logits, func)

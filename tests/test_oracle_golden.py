@@ -117,6 +117,7 @@ def test_gate_scores_closed_forms(orc):
     np.testing.assert_allclose(orc.gate_scores(x, orc.SCORE_SOFTMAX), sm / sm.sum(1, keepdims=True), rtol=1e-5)
     np.testing.assert_allclose(orc.gate_scores(x, orc.SCORE_SIGMOID), 1 / (1 + np.exp(-xd)), rtol=1e-5)
     np.testing.assert_allclose(orc.gate_scores(x, orc.SCORE_SQRTSOFTPLUS), np.sqrt(np.log1p(np.exp(xd))), rtol=1e-4)
+    np.testing.assert_allclose(orc.gate_scores(x, orc.SCORE_SQRTSOFTPLUS_STABLE), np.sqrt(np.logaddexp(xd, 0.0)), rtol=1e-6)
 
 
 # ---------------------------------------------------------------- remap / dedup / smelt ----------------
@@ -462,6 +463,31 @@ def test_det_exp_log_within_one_ulp_of_the_exact_value(orc):
     assert np.isnan(orc.det_expf([np.nan])[0])
 
 
+def test_det_softplus_against_the_exact_function(orc):
+    """The overflow-free softplus behind DMOE_SCORE_SQRTSOFTPLUS_STABLE, against float64 logaddexp(x, 0): within
+    two units in the last place from -85 to 200 (a dropped log1p correction, a wrong sign of |x| or a missing max(x, 0)
+    each miss that by orders of magnitude somewhere on the range), equal to x where exp(-x) no longer registers, and
+    finite where the reference's literal log(1 + exp(x)) overflows. Where the literal form is accurate the two agree to
+    rounding; below x = -15 the literal form has lost the value (1 + exp(x) rounds to 1) and the stable one has not."""
+    x = np.concatenate([np.linspace(-85.0, 200.0, 5701), [0.0, -0.0, 1e-6, -1e-6, 16.6, 17.4, 88.7, 88.8]]).astype(np.float32)
+    got = orc.det_softplusf(x).astype(np.float64)
+    ref = np.logaddexp(x.astype(np.float64), 0.0)
+    ulp = np.spacing(ref.astype(np.float32)).astype(np.float64)
+    assert (np.abs(got - ref) / ulp).max() < 2.0, (np.abs(got - ref) / ulp).max()
+    big = np.array([30.0, 88.8, 128.0, 3e38], np.float32)
+    np.testing.assert_array_equal(orc.det_softplusf(big), big)
+    assert orc.det_softplusf([0.0])[0] == np.float32(np.log(2.0)) and orc.det_softplusf([-100.0])[0] == 0.0
+    assert np.isnan(orc.det_softplusf([np.nan])[0]) and np.isinf(orc.det_softplusf([np.inf])[0])
+    # the scoring function built on it, next to the literal one
+    xs = np.linspace(-20.0, 100.0, 9 * 40).astype(np.float32).reshape(9, 40)
+    stable, literal = orc.gate_scores_det(xs, orc.SCORE_SQRTSOFTPLUS_STABLE), orc.gate_scores_det(xs, orc.SCORE_SQRTSOFTPLUS)
+    np.testing.assert_allclose(stable, np.sqrt(np.logaddexp(xs.astype(np.float64), 0.0)), rtol=3e-7)
+    ok = np.isfinite(literal) & (xs > -6.0)
+    assert not ok.all() and np.isinf(literal[xs > 88.8]).all() and np.isfinite(stable).all()
+    np.testing.assert_allclose(stable[ok], literal[ok], rtol=2e-5)   # 1 + exp(x) rounded: up to 2^-24 / exp(-6) on the log
+    assert (literal[xs < -17.0] == 0.0).all() and (stable[xs < -17.0] > 0.0).all()
+
+
 def test_gate_logits_match_a_float64_matmul(orc):
     rng = np.random.default_rng(5)
     T, D, E = 7, 392, 24      # a short last segment (392 = 3 * 128 + 8)
@@ -481,7 +507,7 @@ def test_gate_logits_match_a_float64_matmul(orc):
 def test_gate_scores_det_agree_with_libm(orc):
     rng = np.random.default_rng(6)
     logits = orc.bf16_to_f32(orc.f32_to_bf16((rng.standard_normal((9, 70)) * 4).astype(np.float32)))
-    for func in (0, 1, 2):
+    for func in (0, 1, 2, 3):
         a, b = orc.gate_scores_det(logits, func), orc.gate_scores(logits, func)
         np.testing.assert_allclose(a, b, rtol=2e-6, atol=1e-12)
     sm = orc.gate_scores_det(logits, 0)
