@@ -59,7 +59,7 @@ SCORE_SOFTMAX, SCORE_SIGMOID, SCORE_SQRTSOFTPLUS, SCORE_SQRTSOFTPLUS_STABLE = 0,
 
 # every symbol include/dmoe.h declares
 EXPORTS = [
-    "dmoe_quant_mode_from_string", "dmoe_version", "dmoe_last_error", "dmoe_init",
+    "dmoe_quant_mode_from_string", "dmoe_version", "dmoe_dequant_fp8_block", "dmoe_last_error", "dmoe_init",
     "dmoe_stream_create", "dmoe_stream_destroy", "dmoe_stream_synchronize",
     "dmoe_malloc", "dmoe_free", "dmoe_copy_to_device", "dmoe_copy_to_host",
     "dmoe_workspace_create", "dmoe_workspace_destroy", "dmoe_workspace_reserved",
@@ -289,6 +289,18 @@ def dequantize(qw, mat_index=0, fused=False):
     c = qw.c()
     fn = lib().dmoe_debug_dequantize_fused if fused else lib().dmoe_dequantize
     check(fn(_ptr(out), C.byref(c), mat_index, _stream()))
+    return out
+
+
+def dequant_fp8_block(w, scale, block_size):
+    """dmoe_dequant_fp8_block: w uint8 [rows, cols] (E4M3FN), scale float32 or uint8 (E8M0)
+    [ceil(rows / block), ceil(cols / block)] -> bf16 [rows, cols]."""
+    rows, cols = w.shape
+    assert w.dtype == torch.uint8 and w.is_contiguous() and scale.is_contiguous()
+    assert scale.dtype in (torch.float32, torch.uint8) and tuple(scale.shape) == (-(-rows // block_size), -(-cols // block_size))
+    out = torch.empty((rows, cols), dtype=torch.bfloat16, device=w.device)
+    check(lib().dmoe_dequant_fp8_block(_ptr(out), _ptr(w), _ptr(scale), int(scale.dtype == torch.uint8), rows, cols,
+                                       block_size, _stream()))
     return out
 
 

@@ -144,9 +144,66 @@ struct DequantLaunch {
     }
 };
 
+// FP8 E4M3 bytes [rows, cols] with one scale per block x block tile -> bf16. One thread per 16 bytes of a row (the
+// launcher takes this kernel when a 16-byte piece never straddles two tiles), two 16-byte stores each.
+template <bool E8M0>
+__global__ void dequant_fp8_block_kernel(uint16_t *__restrict__ out, const uint8_t *__restrict__ w, const void *__restrict__ scale,
+                                         int rows, int cols, int block, int scale_cols) {
+    const int chunks_per_row = cols / 16;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)rows * chunks_per_row) return;
+    const int row = (int)(i / chunks_per_row), c = (int)(i - (size_t)row * chunks_per_row);
+    const size_t si = (size_t)(row / block) * scale_cols + (size_t)(c * 16 / block);
+    const float sc = E8M0 ? e8m0_to_f32(((const uint8_t *)scale)[si]) : ((const float *)scale)[si];
+    const uint4 raw = *(const uint4 *)(w + (size_t)row * cols + (size_t)c * 16);
+    uint32_t pairs[8];
+    FmtFp8Row::decode(raw, Meta{1.0f, 0.0f}, pairs);
+#pragma unroll
+    for (int p = 0; p < 8; ++p)
+        pairs[p] = pack_bf16x2(bf16_bits_to_f32(pairs[p] & 0xffffu) * sc, bf16_bits_to_f32(pairs[p] >> 16) * sc);
+    uint4 *o = (uint4 *)(out + (size_t)row * cols + (size_t)c * 16);
+    o[0] = make_uint4(pairs[0], pairs[1], pairs[2], pairs[3]);
+    o[1] = make_uint4(pairs[4], pairs[5], pairs[6], pairs[7]);
+}
+
+// any shape, block size and alignment: one thread per value
+template <bool E8M0>
+__global__ void dequant_fp8_block_scalar_kernel(uint16_t *__restrict__ out, const uint8_t *__restrict__ w,
+                                                const void *__restrict__ scale, int rows, int cols, int block, int scale_cols) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)rows * cols) return;
+    const int row = (int)(i / cols), col = (int)(i - (size_t)row * cols);
+    const size_t si = (size_t)(row / block) * scale_cols + (size_t)(col / block);
+    const float sc = E8M0 ? e8m0_to_f32(((const uint8_t *)scale)[si]) : ((const float *)scale)[si];
+    out[i] = f32_to_bf16_bits(e4m3_to_f32(w[i]) * sc);
+}
+
 } // namespace dmoe
 
 using namespace dmoe;
+
+extern "C" int dmoe_dequant_fp8_block(uint16_t *d_out, const uint8_t *d_weight, const void *d_scale, int scale_is_e8m0,
+                                      int rows, int cols, int block_size, dmoe_stream s) {
+    DMOE_REQUIRE(d_out && d_weight && d_scale, "dequant_fp8_block: null pointer");
+    DMOE_REQUIRE(rows >= 0 && cols >= 0 && block_size >= 1, "dequant_fp8_block: bad shape [%d,%d] / block %d", rows, cols, block_size);
+    if (rows == 0 || cols == 0) return DMOE_OK;
+    const int scale_cols = ceil_div(cols, block_size);
+    const size_t n = (size_t)rows * (size_t)cols;
+    const bool wide = cols % 16 == 0 && block_size % 16 == 0 && ((uintptr_t)d_weight % 16) == 0 && ((uintptr_t)d_out % 16) == 0;
+    const size_t threads = wide ? n / 16 : n;
+    DMOE_REQUIRE((threads + 255) / 256 <= 0x7fffffffull, "dequant_fp8_block: [%d,%d] is too large for one call", rows, cols);
+    const dim3 grid((unsigned)((threads + 255) / 256)), blk(256);
+    hipStream_t st = to_hip(s);
+    if (wide) {
+        if (scale_is_e8m0) hipLaunchKernelGGL(dequant_fp8_block_kernel<true>, grid, blk, 0, st, d_out, d_weight, d_scale, rows, cols, block_size, scale_cols);
+        else hipLaunchKernelGGL(dequant_fp8_block_kernel<false>, grid, blk, 0, st, d_out, d_weight, d_scale, rows, cols, block_size, scale_cols);
+    } else {
+        if (scale_is_e8m0) hipLaunchKernelGGL(dequant_fp8_block_scalar_kernel<true>, grid, blk, 0, st, d_out, d_weight, d_scale, rows, cols, block_size, scale_cols);
+        else hipLaunchKernelGGL(dequant_fp8_block_scalar_kernel<false>, grid, blk, 0, st, d_out, d_weight, d_scale, rows, cols, block_size, scale_cols);
+    }
+    DMOE_LAUNCH_CHECK();
+    return DMOE_OK;
+}
 
 static int dequantize_common(uint16_t *d_out, const dmoe_qweight *qw, int mat_index, bool fused, dmoe_stream s) {
     QView q;

@@ -613,6 +613,16 @@ inline Array dequantize(const Context &ctx, const QuantizedWeight &w, int mat_in
     check(dmoe_dequantize((uint16_t *)out.data(), &q, mat_index, ctx.stream()));
     return out;
 }
+// dequantFp8(ctx, weight, scale, block_size) (deepseek_v4_loader.zig:922-990): weight uint8 [rows, cols] (E4M3FN), scale
+// f32 or uint8 (E8M0) [ceil(rows / block), ceil(cols / block)] -> bf16 [rows, cols]
+inline Array dequantFp8(const Context &ctx, const Array &weight, const Array &scale, int block_size) {
+    if (weight.shape().size() != 2) throw Error(DMOE_ERR_INVALID, "dequantFp8: weight must be [rows, cols]");
+    const int rows = weight.shape()[0], cols = weight.shape()[1];
+    Array out(ctx, DType::bfloat16, {rows, cols});
+    check(dmoe_dequant_fp8_block((uint16_t *)out.data(), (const uint8_t *)weight.data(), scale.data(),
+                                 scale.dtype() == DType::uint8 ? 1 : 0, rows, cols, block_size, ctx.stream()));
+    return out;
+}
 } // namespace quantize_mod
 namespace ops {
 // gatherMm(ctx, a, b, lhs?, rhs, sorted) with unquantized experts (deepseek_v4.zig:978). The reference hands over

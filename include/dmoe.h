@@ -212,6 +212,15 @@ typedef struct {
  * E2M1 * 2^(s-127) (mxfp4, exact), e4m3 * row_scale rounded to bf16 (fp8row). Device pointers in `qw`. */
 int dmoe_dequantize(uint16_t *d_out, const dmoe_qweight *qw, int mat_index, dmoe_stream s);
 
+/* dequantFp8 (deepseek_v4_loader.zig:922-990) with scaleToFloat (:839-856): FP8 E4M3FN bytes [rows, cols] with one
+ * scale per block_size x block_size tile, d_scale [ceil(rows / block_size), ceil(cols / block_size)] as f32, or as
+ * E8M0 bytes (scale_is_e8m0 != 0: 2^(s-127), the value the reference's exp((s-127) ln 2) stands for; 255 is NaN)
+ * -> d_out bf16 [rows, cols] = bf16(f32(fp8) * scale), one rounding. rows and cols need not be multiples of the block
+ * (the reference pads and truncates; the values are the same). The FP4 counterpart, dequantFp4 (:859-920), is
+ * dmoe_dequantize on a DMOE_QUANT_MXFP4 matrix (low nibble first, one E8M0 byte per 32 values). */
+int dmoe_dequant_fp8_block(uint16_t *d_out, const uint8_t *d_weight, const void *d_scale, int scale_is_e8m0,
+                           int rows, int cols, int block_size, dmoe_stream s);
+
 /* quantize_mod.gatherQmm(x, w, scales, biases, lhs_indices, rhs_indices, transpose = true, cfg, sorted)
  * (call shape deepseek_v4.zig:976, expert_preload.zig:265; mlx.core.gather_qmm):
  *   out[r, :] = x[lhs ? lhs[r] : r, :] . dequant(W[rhs[r]])^T     r < R

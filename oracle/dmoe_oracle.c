@@ -545,6 +545,21 @@ void orc_dequantize(const orc_qmat *m, int mi, uint16_t *out) {
             out[(size_t)r * m->cols + c] = orc_f32_to_bf16(orc_dequant_value(m, mi, r, c));
 }
 
+/* dequantFp8, deepseek_v4_loader.zig:922-990: w u8 [rows, cols] (E4M3FN, fromFp8 -> bf16 is exact), scale
+ * [ceil(rows/block), ceil(cols/block)] through scaleToFloat (:839-856: f32 as it is, u8 as E8M0), weight viewed as
+ * [m/bs, bs, n/bs, bs] times scale[:, None, :, None] in f32 (:957-970), then astype(bf16) (:981-984). The padding to
+ * whole blocks (:936-955) and the truncation (:979-982) do not change any value. */
+void orc_dequant_fp8_block(const uint8_t *w, const void *scale, int scale_is_e8m0, int rows, int cols, int block,
+                           uint16_t *out) {
+    int scale_cols = (cols + block - 1) / block;
+    for (int r = 0; r < rows; r++)
+        for (int c = 0; c < cols; c++) {
+            size_t si = (size_t)(r / block) * scale_cols + (size_t)(c / block);
+            float sc = scale_is_e8m0 ? e8m0_to_f32(((const uint8_t *)scale)[si]) : ((const float *)scale)[si];
+            out[(size_t)r * cols + c] = orc_f32_to_bf16(e4m3_to_f32(w[(size_t)r * cols + c]) * sc);
+        }
+}
+
 /* the same values in f32, before the rounding to bf16 */
 void orc_dequantize_f32(const orc_qmat *m, int mi, float *out) {
     for (int r = 0; r < m->rows; r++) dequant_row_f32(m, mi, r, out + (size_t)r * m->cols);

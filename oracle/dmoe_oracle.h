@@ -121,6 +121,8 @@ void orc_reduce_experts(const float *expert_outs, const float *w, int T, int K, 
 
 /* dequantize -> bf16 [rows, cols] of matrix `mat_index` of the stack */
 void orc_dequantize(const orc_qmat *m, int mat_index, uint16_t *out_bf16);
+void orc_dequant_fp8_block(const uint8_t *w, const void *scale, int scale_is_e8m0, int rows, int cols, int block,
+                           uint16_t *out);
 /* whole matrix / single value in f32, before the bf16 rounding */
 void orc_dequantize_f32(const orc_qmat *m, int mat_index, float *out_f32);
 float orc_dequant_value(const orc_qmat *m, int mat_index, int row, int col);

@@ -299,6 +299,18 @@ def dequantize(qm, mat_index=0):
     return out
 
 
+def dequant_fp8_block(w, scale, block):
+    """w uint8 [rows, cols]; scale float32 or uint8 (E8M0) [ceil(rows/block), ceil(cols/block)] -> uint16 (bf16) [rows, cols]"""
+    w = _c(w, np.uint8)
+    e8m0 = scale.dtype == np.uint8
+    scale = _c(scale, np.uint8 if e8m0 else np.float32)
+    rows, cols = w.shape
+    assert scale.shape == (-(-rows // block), -(-cols // block)), scale.shape
+    out = np.empty((rows, cols), np.uint16)
+    lib().orc_dequant_fp8_block(_p(w), _p(scale), int(e8m0), rows, cols, block, _p(out))
+    return out
+
+
 def dequantize_f32(qm, mat_index=0):
     out = np.empty((qm.rows, qm.cols), np.float32)
     c = qm.c()

@@ -331,6 +331,27 @@ static void test_gather_mm(Context &ctx) {
     for (int i = 0; i < rows * cols; ++i) EXPECT(back[i] == w[(size_t)rows * cols + i]);
 }
 
+// quantize_mod::dequantFp8 with values exact in bf16: byte 0x38 is 1.0, 0x40 is 2.0, 0xB8 is -1.0 (E4M3FN); a 3 x 5 weight
+// with 2 x 2 blocks (neither dimension a whole number of blocks) and scales that are powers of two, once as f32 and
+// once as E8M0 bytes
+static void test_dequant_fp8(Context &ctx) {
+    const int rows = 3, cols = 5, bs = 2;
+    const uint8_t w[rows * cols] = {0x38, 0x40, 0xB8, 0x38, 0x40, 0x40, 0x40, 0x38, 0xB8, 0x00, 0x38, 0xB8, 0x40, 0x40, 0x38};
+    const float val[rows * cols] = {1, 2, -1, 1, 2, 2, 2, 1, -1, 0, 1, -1, 2, 2, 1};
+    const float sf[2 * 3] = {1.0f, 0.5f, 4.0f, 2.0f, 0.25f, 8.0f};
+    const uint8_t se[2 * 3] = {127, 126, 129, 128, 125, 130};
+    Array wa = Array::fromData(ctx, w, {rows, cols}, DType::uint8);
+    Array fa = Array::fromData(ctx, sf, {2, 3}, DType::float32), ea = Array::fromData(ctx, se, {2, 3}, DType::uint8);
+    auto a = quantize_mod::dequantFp8(ctx, wa, fa, bs).dataSlice<uint16_t>();
+    auto b = quantize_mod::dequantFp8(ctx, wa, ea, bs).dataSlice<uint16_t>();
+    for (int r = 0; r < rows; ++r)
+        for (int c = 0; c < cols; ++c) {
+            const float want = val[r * cols + c] * sf[(r / bs) * 3 + c / bs];
+            EXPECT(from_bf16(a[(size_t)r * cols + c]) == want);
+            EXPECT(from_bf16(b[(size_t)r * cols + c]) == want);
+        }
+}
+
 int main() {
     try {
         Context ctx(0);
@@ -342,6 +363,7 @@ int main() {
         test_gate_from_hidden(ctx);
         test_block_post(ctx);
         test_gather_mm(ctx);
+        test_dequant_fp8(ctx);
         ctx.synchronize();
     } catch (const Error &e) {
         std::printf("dmoe::Error %d: %s\n", e.code, e.what());

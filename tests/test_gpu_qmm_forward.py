@@ -64,6 +64,29 @@ def test_dequantize_bit_exact(dmoe, orc, fmt):
             assert ((got[nan] & 0x7FFF) > 0x7F80).all()
 
 
+@pytest.mark.parametrize("rows,cols,block", [(512, 768, 128), (200, 336, 128), (37, 50, 16), (64, 48, 24), (33, 64, 1),
+                                             (4096, 2048, 128)])
+def test_dequant_fp8_block_bit_exact(dmoe, orc, rows, cols, block):
+    """dmoe_dequant_fp8_block (dequantFp8, deepseek_v4_loader.zig:922-990) against the oracle: every E4M3 byte, shapes
+    that are not whole blocks, block sizes that send the call to the one-value-per-thread kernel (columns or blocks not
+    multiples of 16), f32 and E8M0 scales with the extreme exponents, and one weight matrix of a real expert's size."""
+    g = torch.Generator(device="cuda").manual_seed(rows + cols)
+    w = torch.randint(0, 256, (rows, cols), generator=g, device="cuda", dtype=torch.uint8)
+    w[0, :min(cols, 256)] = torch.arange(min(cols, 256), dtype=torch.uint8, device="cuda")
+    sr, sc = -(-rows // block), -(-cols // block)
+    scale_f = (torch.rand((sr, sc), generator=g, device="cuda") * 0.01 + 1e-4).float()
+    scale_e = torch.randint(90, 150, (sr, sc), generator=g, device="cuda", dtype=torch.uint8)
+    scale_e.view(-1)[:3] = torch.tensor([0, 254, 255], dtype=torch.uint8, device="cuda")[:scale_e.numel()][:3]
+    for scale in (scale_f, scale_e):
+        got = bf16_bits(dmoe.dequant_fp8_block(w, scale, block))
+        want = orc.dequant_fp8_block(w.cpu().numpy(), scale.cpu().numpy(), block)
+        nan = (want & 0x7FFF) > 0x7F80
+        np.testing.assert_array_equal(got[~nan], want[~nan])
+        assert ((got[nan] & 0x7FFF) > 0x7F80).all()
+    with pytest.raises(dmoe.DmoeError):
+        dmoe.check(dmoe.lib().dmoe_dequant_fp8_block(None, None, None, 0, 4, 4, 2, None))
+
+
 @pytest.mark.parametrize("fmt", FORMATS)
 @pytest.mark.parametrize("R,n_mats,rows,cols", [(24, 8, 256, 1024),     # small-M path (<= 4 rows per expert on average)
                                                 (700, 4, 256, 512),     # MFMA path, ragged segments

@@ -229,6 +229,37 @@ def test_fp8_e4m3_all_codes_match_torch(orc):
     np.testing.assert_array_equal(deq[ok], ref[ok])
 
 
+@pytest.mark.parametrize("rows,cols,block", [(256, 384, 128), (200, 330, 128), (7, 50, 16), (33, 64, 1)])
+def test_fp8_block_dequant_matches_the_reference_op_sequence_in_torch(orc, rows, cols, block):
+    """dequantFp8 (deepseek_v4_loader.zig:922-990) evaluated with torch on the CPU exactly as the reference writes it -
+    fromFp8 to bf16, zero-pad to whole blocks, view as [m/bs, bs, n/bs, bs], times scale[:, None, :, None] in f32, back,
+    truncate, astype(bf16) - against the oracle's per-element restatement. Shapes that need the padding, a block of one,
+    f32 scales and E8M0 scales (the reference's exp((s - 127) ln 2) taken as the exact power of two)."""
+    g = torch.Generator().manual_seed(rows * 1000 + cols)
+    w = torch.randint(0, 256, (rows, cols), generator=g, dtype=torch.uint8)
+    w[0, :min(cols, 256)] = torch.arange(min(cols, 256), dtype=torch.uint8)
+    sr, sc = -(-rows // block), -(-cols // block)
+    for e8m0 in (False, True):
+        if e8m0:
+            scale = torch.randint(100, 140, (sr, sc), generator=g, dtype=torch.uint8)
+            scale_f32 = torch.exp2(scale.float() - 127.0)
+        else:
+            scale = (torch.rand((sr, sc), generator=g) * 0.01 + 1e-4).float()
+            scale_f32 = scale
+        w_bf16 = w.view(torch.float8_e4m3fn).to(torch.bfloat16)
+        pm, pn = sr * block, sc * block
+        padded = torch.zeros((pm, pn), dtype=torch.bfloat16)
+        padded[:rows, :cols] = w_bf16
+        scaled = padded.reshape(sr, block, sc, block).float() * scale_f32[:, None, :, None]
+        want = scaled.reshape(pm, pn)[:rows, :cols].to(torch.bfloat16)
+        got = orc.dequant_fp8_block(w.numpy(), scale.numpy(), block)
+        want_bits = want.view(torch.int16).numpy().view(np.uint16)
+        nan = np.isnan(want.float().numpy())
+        assert nan.any() == bool(((w & 0x7F) == 0x7F).any())
+        np.testing.assert_array_equal(got[~nan], want_bits[~nan])
+        assert ((got[nan] & 0x7FFF) > 0x7F80).all()
+
+
 def test_mxfp4_codes_and_scales(orc, golden):
     """E2M1 table of deepseek_v4_loader.zig:861-863 times 2^(s-127), low nibble first; exact in bf16."""
     table = np.array(golden["e2m1_table"]["values"], np.float64)
