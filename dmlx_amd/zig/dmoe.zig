@@ -214,6 +214,15 @@ pub fn gatherQmm(ctx: Context, x: DeviceArray(u16), q: *const c.dmoe_qweight, lh
     return out;
 }
 
+/// dequantFp8(ctx, weight, scale, block_size) (src/models/deepseek_v4_loader.zig:922-990): FP8 E4M3 bytes [rows, cols]
+/// with one scale per block_size x block_size tile (f32, or E8M0 bytes with `scale_is_e8m0`) -> bf16 [rows, cols].
+pub fn dequantFp8(ctx: Context, weight: DeviceArray(u8), scale_ptr: *const anyopaque, scale_is_e8m0: bool, rows: usize, cols: usize, block_size: usize) Error!DeviceArray(u16) {
+    const out = try DeviceArray(u16).alloc(rows * cols);
+    errdefer out.deinit();
+    try check(c.dmoe_dequant_fp8_block(@ptrCast(@alignCast(out.ptr)), @ptrCast(weight.ptr), scale_ptr, @intFromBool(scale_is_e8m0), @intCast(rows), @intCast(cols), @intCast(block_size), ctx.stream));
+    return out;
+}
+
 /// A weight stack made resident once in the layout the kernels stream (the long-lived weight Arrays of the
 /// reference's layer structs); `gatherQmm` on it gives the same bits as on the MLX layout, faster.
 pub const ResidentWeight = struct {
