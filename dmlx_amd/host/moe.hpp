@@ -402,6 +402,19 @@ class DSV4SwitchGLU {
                                                 (const uint32_t *)slot_indices.data(), T, ctx.workspace(), ctx.stream()));
         return out;
     }
+    // DSV4MoE.forward from the gate's scores on (deepseek_v4.zig:1021-1052) in one call: selection (bias, Smelt mask,
+    // renormalisation, route_scale as in DSV4Gate.forward :589-678), then forward(). scores f32 [N, n_experts_total];
+    // bias f32 [n_experts_total] / resident_mask u8 [n_experts_total] or null.
+    Array forwardFromScores(const Context &ctx, const Array &x, const Array &scores, const Array *bias, const Array *resident_mask,
+                            bool renorm, float route_scale) const {
+        const int T = x.shape().at(0), E = scores.shape().at(1);
+        Array out(ctx, DType::bfloat16, {T, hidden_});
+        check(dmoe_moe_layer_forward((uint16_t *)out.data(), nullptr, nullptr, layer_, (const uint16_t *)x.data(),
+                                     (const float *)scores.data(), bias ? (const float *)bias->data() : nullptr,
+                                     resident_mask ? (const uint8_t *)resident_mask->data() : nullptr, T, E, renorm ? 1 : 0,
+                                     route_scale, ctx.workspace(), ctx.stream()));
+        return out;
+    }
     dmoe_layer handle() const { return layer_; }
     int hidden() const { return hidden_; }
     int top_k() const { return top_k_; }
@@ -410,6 +423,29 @@ class DSV4SwitchGLU {
     dmoe_layer layer_{};
     int hidden_, ffn_, top_k_;
 };
+
+// The sort block of DSV4SwitchGLU.forward (deepseek_v4.zig:749-784) on its own: rows (t * K + k) grouped by expert, ties
+// in ascending flat index. order = argsort(flat indices) (:753), inv_order = argsort(order) (:758), token = order / K
+// (:765-772), plus rows per expert and their exclusive scan (offsets has n_experts + 1 entries).
+struct SortedRows {
+    Array order, inv_order, token, counts, offsets;
+};
+inline SortedRows sortByExpert(const Context &ctx, const Array &indices, int n_experts) {
+    const int T = indices.shape().at(0), K = indices.shape().at(1);
+    SortedRows r{Array(ctx, DType::uint32, {T * K}), Array(ctx, DType::uint32, {T * K}), Array(ctx, DType::uint32, {T * K}),
+                 Array(ctx, DType::uint32, {n_experts}), Array(ctx, DType::uint32, {n_experts + 1})};
+    check(dmoe_pack((uint32_t *)r.order.data(), (uint32_t *)r.inv_order.data(), (uint32_t *)r.token.data(), nullptr,
+                    (uint32_t *)r.counts.data(), (uint32_t *)r.offsets.data(), nullptr, nullptr, (const uint32_t *)indices.data(), T,
+                    K, n_experts, ctx.workspace(), ctx.stream()));
+    return r;
+}
+// mlx_take(expert_remap, indices).astype(u32) (deepseek_v4.zig:1035-1039, expert_preload.zig:200-206); remap i32 on the device
+inline Array remapIndices(const Context &ctx, const Array &remap, const Array &indices) {
+    Array out(ctx, DType::uint32, indices.shape());
+    check(dmoe_remap_indices((uint32_t *)out.data(), (const int32_t *)remap.data(), (const uint32_t *)indices.data(), indices.size(),
+                             (int)remap.size(), ctx.stream()));
+    return out;
+}
 
 // ---- expert_provider.zig --------------------------------------------------------------------------------------
 

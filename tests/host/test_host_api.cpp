@@ -228,6 +228,12 @@ static void test_layer_closed_form(const Context &ctx) {
         const double want = 1.5 * bdr * F * h; // renormalised weights sum to 1, times route_scale
         for (int d = 0; d < D; d += 37) NEAR(from_bf16(y[(size_t)t * D + d]), want, std::fabs(want) * 2e-2 + 1e-6);
     }
+    // the same step as one call from the scores on (a second handle on the same weights): the same bytes
+    DSV4SwitchGLU direct(ctx, D, F, K, gate, up, down, opt);
+    Array y2 = direct.forwardFromScores(ctx, hidden.reshaped({T, D}), Array::fromData(ctx, scores.data(), {T, E}, DType::float32),
+                                        nullptr, nullptr, true, 1.5f);
+    auto y2v = y2.dataSlice<uint16_t>();
+    for (size_t i = 0; i < y.size(); ++i) EXPECT(y2v[i] == y[i]);
     // error path: an unknown layer index is reported, not ignored
     bool threw = false;
     try {
@@ -331,6 +337,25 @@ static void test_gather_mm(Context &ctx) {
     for (int i = 0; i < rows * cols; ++i) EXPECT(back[i] == w[(size_t)rows * cols + i]);
 }
 
+// the sort block of DSV4SwitchGLU.forward and the expert_remap take, on a case small enough to sort by hand:
+// flat indices [2,0, 1,2, 0,2] -> rows grouped by expert with ties in flat order
+static void test_sort_and_remap(Context &ctx) {
+    const uint32_t idx[6] = {2, 0, 1, 2, 0, 2};
+    Array ia = Array::fromData(ctx, idx, {3, 2}, DType::uint32);
+    SortedRows r = sortByExpert(ctx, ia, 3);
+    const uint32_t order[6] = {1, 4, 2, 0, 3, 5}, inv[6] = {3, 0, 2, 4, 1, 5}, token[6] = {0, 2, 1, 0, 1, 2};
+    const uint32_t counts[3] = {2, 1, 3}, offsets[4] = {0, 2, 3, 6};
+    auto o = r.order.dataSlice<uint32_t>(), iv = r.inv_order.dataSlice<uint32_t>(), tk = r.token.dataSlice<uint32_t>();
+    auto cn = r.counts.dataSlice<uint32_t>(), of = r.offsets.dataSlice<uint32_t>();
+    for (int i = 0; i < 6; ++i) EXPECT(o[i] == order[i] && iv[i] == inv[i] && tk[i] == token[i]);
+    for (int e = 0; e < 3; ++e) EXPECT(cn[e] == counts[e]);
+    for (int e = 0; e < 4; ++e) EXPECT(of[e] == offsets[e]);
+    const int32_t remap[3] = {5, 0, 7};
+    auto m = remapIndices(ctx, Array::fromData(ctx, remap, {3}, DType::int32), ia).dataSlice<uint32_t>();
+    const uint32_t want[6] = {7, 5, 0, 7, 5, 7};
+    for (int i = 0; i < 6; ++i) EXPECT(m[i] == want[i]);
+}
+
 // quantize_mod::dequantFp8 with values exact in bf16: byte 0x38 is 1.0, 0x40 is 2.0, 0xB8 is -1.0 (E4M3FN); a 3 x 5 weight
 // with 2 x 2 blocks (neither dimension a whole number of blocks) and scales that are powers of two, once as f32 and
 // once as E8M0 bytes
@@ -364,6 +389,7 @@ int main() {
         test_block_post(ctx);
         test_gather_mm(ctx);
         test_dequant_fp8(ctx);
+        test_sort_and_remap(ctx);
         ctx.synchronize();
     } catch (const Error &e) {
         std::printf("dmoe::Error %d: %s\n", e.code, e.what());
