@@ -10,18 +10,21 @@ from dmlx_amd import workloads
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("config,scale", [(1, 0.5), (2, 0.5), (4, 0.125)])
-def test_layer_step_replays_bit_identically(dmoe, ws, config, scale):
+@pytest.mark.parametrize("config,scale,tokens", [(1, 0.5, None), (2, 0.5, None), (4, 0.125, None), (1, 1.0, 1), (2, 1.0, 1)])
+def test_layer_step_replays_bit_identically(dmoe, ws, config, scale, tokens):
+    """tokens = 1: a single sequence at full size, whose launch splits every tile's reduction over two groups of
+    wavefronts (twice the workgroups per tile, the halves meeting in LDS)."""
     wl = workloads.make(config, scale=scale)
     layer = dmoe.Layer(wl.D, wl.F, wl.K, wl.gate, wl.up, wl.down, swiglu_limit=wl.swiglu_limit,
                        score_before_down=wl.score_before_down, shared=wl.shared,
-                       shared_swiglu_limit=wl.shared_swiglu_limit, remap=wl.remap)
+                       shared_swiglu_limit=wl.shared_swiglu_limit, remap=wl.remap, borrow=tokens is not None)
+    scores = wl.scores if tokens is None else wl.scores[:tokens].contiguous()
 
     def step(x):
-        return layer.layer_forward(x, wl.scores, wl.bias, wl.resident_mask, wl.renorm, wl.route_scale, ws)
+        return layer.layer_forward(x, scores, wl.bias, wl.resident_mask, wl.renorm, wl.route_scale, ws)
 
-    x_a = wl.x
-    x_b = torch.roll(wl.x, 1, dims=0).contiguous()
+    x_a = wl.x if tokens is None else wl.x[:tokens].contiguous()
+    x_b = torch.roll(wl.x, 1, dims=0).contiguous() if tokens is None else wl.x[tokens:2 * tokens].contiguous()
     want_a, want_b = step(x_a).clone(), step(x_b).clone()   # also sizes the workspace before the capture
     torch.cuda.synchronize()
 
