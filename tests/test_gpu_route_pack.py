@@ -75,6 +75,24 @@ def test_topk_route_bit_exact(dmoe, orc, T, E, K, normalize):
     np.testing.assert_array_equal(_f32_bits(w.cpu().numpy()), _f32_bits(want_w))
 
 
+@pytest.mark.parametrize("T,E,K", [(50, 24, 5), (7, 256, 6), (300, 100, 64), (3, 1024, 8)])
+def test_topk_route_special_values_bit_exact(dmoe, orc, T, E, K):
+    """Negative scores, both zeros, denormals, both infinities and NaNs of both signs: the selection follows the same
+    total order as the oracle (ascending, -0 equal to +0, NaN last, ties to the higher index); the weights are the
+    selected scores' bits (no normalisation, so that NaN and infinity stay where they are)."""
+    from tests.test_oracle_golden import _special_scores
+    scores = _special_scores(T, E, T + E)
+    idx, w = dmoe.topk_route(_dev(scores), K, False)
+    want_idx, want_w = orc.topk_route(scores, K, False)
+    np.testing.assert_array_equal(to_np_u32(idx), want_idx)
+    np.testing.assert_array_equal(_f32_bits(w.cpu().numpy()), _f32_bits(want_w))
+    # the gate's selection on the same values (bias zero, no mask, no renormalisation, scale 1)
+    idx2, w2 = dmoe.gate_route(_dev(scores), None, None, K, False, 1.0)
+    g_idx, g_w = orc.gate_route(scores, None, None, K, False, 1.0)
+    np.testing.assert_array_equal(to_np_u32(idx2), g_idx)
+    np.testing.assert_array_equal(_f32_bits(w2.cpu().numpy()), _f32_bits(g_w))
+
+
 def test_property_18_on_gpu(dmoe):
     """moe_router.zig:455-628 through the GPU path."""
     rng = np.random.default_rng(18)

@@ -86,6 +86,27 @@ def test_topk_matches_stable_argsort_and_tie_rule(orc):
     assert (np.diff(w, axis=1) >= 0).all()
 
 
+def _special_scores(T, E, seed):
+    """Scores with negative values, both zeros, denormals, both infinities and NaNs, several of each per row."""
+    rng = np.random.default_rng(seed)
+    s = rng.standard_normal((T, E)).astype(np.float32)
+    special = np.array([0.0, -0.0, 1e-40, -1e-40, np.inf, -np.inf, np.nan, -np.nan, 3e38, -3e38], np.float32)
+    pick = rng.random((T, E)) < 0.4
+    s[pick] = special[rng.integers(0, len(special), int(pick.sum()))]
+    return s
+
+
+def test_topk_order_of_special_values_matches_numpy(orc):
+    """The order the oracle sorts by (ascending, -0 equal to +0, NaN of either sign after +inf, ties by index) is the one
+    numpy's stable argsort uses; selection on rows full of such values against that library routine."""
+    scores = _special_scores(50, 24, 11)
+    for K in (1, 5, 24):
+        idx, w = orc.topk_route(scores, K, False)
+        want = np.argsort(scores, axis=1, kind="stable")[:, -K:]
+        np.testing.assert_array_equal(idx, want.astype(np.uint32))
+        np.testing.assert_array_equal(w.view(np.uint32), np.take_along_axis(scores, want, 1).view(np.uint32))
+
+
 def test_gate_route_bias_mask_renorm_scale(orc):
     """deepseek_v4.zig:589-678 by brute force: selection on biased+masked scores, weights from the raw
     scores, renormalised and scaled; -1e9, -1000 and -inf masks select the same experts."""
