@@ -185,6 +185,10 @@ constexpr int kSkinnyAvgRows = 16;
 // workgroups (GemmArgs::ksplit), on tiles of one row block.
 constexpr int kSplitMaxTiles = 8;
 constexpr int kSplitTileM = 8;
+#ifndef DMOE_PAIR_MIN_ROWS
+#define DMOE_PAIR_MIN_ROWS 64
+#endif
+constexpr int kPairMinRows = DMOE_PAIR_MIN_ROWS; // decode steps above this many sorted rows run gate/up and down in one launch
 constexpr int kSharedSkinnyRows = 64;
 
 static bool few_rows(size_t rows, int n_experts) { return rows <= (size_t)kSkinnyAvgRows * (size_t)n_experts; }
@@ -337,7 +341,10 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
     gu.tile_done = po.tile_done;
     dn.spin_limit = w->spin_limit;
     dn.wait_expired = w->flags;
-    if (f.small && w->paired && qgemm_skinny_pair_supports(gu, dn)) {
+    // (Up to kPairMinRows sorted rows the two projections run as two launches: with so few tiles nearly every gate/up
+    // workgroup is resident from the start, no down workgroup can begin before they end, and what the single launch
+    // adds is the hand-over through memory - stores acknowledged, counter, poll - of 6-8 us per step.)
+    if (f.small && w->paired && n + (f.fold ? (size_t)T : 0) > (size_t)kPairMinRows && qgemm_skinny_pair_supports(gu, dn)) {
         DMOE_TRY(stage_begin(w, DMOE_STAGE_GATE_UP, st));
         DMOE_TRY(launch_qgemm_skinny_pair(gu, dn, st));
         DMOE_TRY(stage_end(w, DMOE_STAGE_GATE_UP, st));

@@ -733,9 +733,7 @@ bool qgemm_skinny_pair_supports(const GemmArgs &gu, const GemmArgs &dn) {
 
 int launch_qgemm_skinny_pair(const GemmArgs &gu, const GemmArgs &dn, hipStream_t st) {
     DMOE_REQUIRE(qgemm_skinny_pair_supports(gu, dn), "skinny GEMM pair: arguments do not form a gate/up + down pair");
-    DMOE_REQUIRE(gu.ksplit == dn.ksplit && (!gu.ksplit || (gu.tile_m <= kSkinnyRowBlock && qgemm_skinny_ksplit_ok(gu.b0) &&
-                                                           qgemm_skinny_ksplit_ok(gu.b1) && qgemm_skinny_ksplit_ok(dn.b0))),
-                 "skinny GEMM pair: a split reduction needs packed weights and tiles of at most %d rows", kSkinnyRowBlock);
+    DMOE_REQUIRE(!gu.ksplit && !dn.ksplit, "skinny GEMM pair: the split reduction is for single launches (steps of a few rows run as two)");
     DMOE_REQUIRE(gu.a && gu.out && dn.out && ((uintptr_t)gu.a % 16) == 0 && ((uintptr_t)dn.a % 16) == 0, "skinny GEMM pair: bad pointer");
     DMOE_REQUIRE(gu.b1.rows == gu.b0.rows && gu.b1.cols == gu.b0.cols && gu.b1.mode == gu.b0.mode && gu.b1.bits == gu.b0.bits &&
                      gu.b1.group == gu.b0.group && gu.b1.packed == gu.b0.packed,

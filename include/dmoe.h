@@ -101,9 +101,10 @@ int dmoe_workspace_reserved(size_t *out_bytes, dmoe_workspace ws);
 int dmoe_workspace_check(dmoe_workspace ws, dmoe_stream s);
 /* polls (~0.25 us each) a waiting workgroup makes before it gives up; default 65536. For tests of the give-up path. */
 int dmoe_workspace_set_wait_limit(dmoe_workspace ws, unsigned polls);
-/* 1 (default): decode-sized calls run gate/up and down in one launch, as described at dmoe_workspace_check;
- * 0: always two launches in a row (same results, a few per cent slower, no waits inside kernels). No counterpart in
- * the reference. */
+/* 1 (default): decode-sized calls of more than 64 expert rows (T * K, plus T when the shared expert rides along) run
+ * gate/up and down in one launch, as described at dmoe_workspace_check; smaller ones take two launches, which is faster
+ * there. 0: always two launches in a row (same results, a few per cent slower at 64 tokens, no waits inside kernels).
+ * No counterpart in the reference. */
 int dmoe_workspace_set_paired_launch(dmoe_workspace ws, int enabled);
 
 /* Per-stage device timing of the layer forward calls made with this workspace (HIP events recorded on the
