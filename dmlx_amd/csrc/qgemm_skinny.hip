@@ -501,7 +501,7 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
             for (int r = 0; r < 4 * RJT; ++r) v[mi][r] = (FACTORED ? facc[mi][r] : acc[mi][r]) * rs;
         }
         if (ks) { // the second half of the reduction joins the first (RJT == 1 here: four values per lane)
-            float4 *kx = (float4 *)xs_lds + 256 * RJT + wq * 64 + lane; // behind the gate/up exchange area below
+            float4 *kx = (float4 *)xs_lds + 256 * RJT + wq * 64 + lane; // bytes 4096 .. 8191, behind the gate/up exchange area below
             __syncthreads(); // every wavefront has left the main loop: the activation window is free
             if (kh == 1) kx[0] = make_float4(v[0][0], v[0][1], v[0][2], v[0][3]);
             __syncthreads();
@@ -605,8 +605,11 @@ static int skinny_vals(const QView &b) {
     return (b.mode == DMOE_QUANT_AFFINE && b.bits == 4) || b.mode == DMOE_QUANT_MXFP4 ? 32 : 16;
 }
 static size_t skinny_lds_bytes(const QView &b) {
-    // a two-row-block tile reads (and ignores) up to 24 floats past its last step's sums: the 128 bytes in the offset
-    return skinny_turn_offset(b.cols, 2 * skinny_vals(b));
+    // a two-row-block tile reads (and ignores) up to 24 floats past its last step's sums: the 128 bytes in the offset.
+    // At least 16 KiB: once the main loop is done the wavefronts exchange their sums through the start of the window
+    // (gate/up pairs: 4 KiB per row block of the tile, up to 16 KiB; split reduction: bytes 4096 .. 8191), which a
+    // short reduction dimension would not cover.
+    return std::max(skinny_turn_offset(b.cols, 2 * skinny_vals(b)), (size_t)16384);
 }
 
 // Rows per tile to build tile lists with for this weight shape: a tile of 2 (4) row blocks splits the reduction

@@ -620,6 +620,30 @@ def test_single_sequence_decode_step(dmoe, orc, ws, fmt):
                 _check_layer(dmoe, orc, ws, wl)
 
 
+@pytest.mark.parametrize("fmt,D,F,E,K,T", [("bf16", 512, 512, 4, 2, 64),      # 32-row tiles over an 8 KiB activation window
+                                           ("bf16", 256, 256, 4, 2, 1),       # one sequence: split reduction, 4 KiB window
+                                           ("affine4", 128, 256, 8, 2, 8),    # a 2 KiB window
+                                           ("affine4", 192, 128, 8, 2, 3),
+                                           ("affine8", 64, 64, 4, 2, 5),      # 1 KiB
+                                           ("mxfp4", 1024, 64, 4, 2, 40)])    # down projection: a reduction of one step
+def test_short_reduction_dimensions(dmoe, orc, ws, fmt, D, F, E, K, T):
+    """Hidden / FFN sizes so small that the activations of a tile take less LDS than the sums the wavefronts exchange
+    once the reduction is done (up to 16 KiB for a 32-row gate/up tile): the exchange must still have its room. With
+    and without a shared expert riding in the routed launch."""
+    g = torch.Generator(device="cuda").manual_seed(D + F + T)
+    x = torch.randn((T, D), generator=g, device="cuda").to(torch.bfloat16)
+    scores = torch.sigmoid(torch.randn((T, E), generator=g, device="cuda"))
+    for with_shared in (False, True):
+        shared = (_stack(fmt, 1, F, D, 61), _stack(fmt, 1, F, D, 62), _stack(fmt, 1, D, F, 63)) if with_shared else None
+        wl = workloads.Workload(f"short reduction {fmt} D={D} F={F} T={T} shared={with_shared}", T, D, F, E, E, K, x, scores,
+                                None, None, None, True, 1.5, _stack(fmt, E, F, D, 51), _stack(fmt, E, F, D, 52),
+                                _stack(fmt, E, D, F, 53), shared)
+        for q in (wl.gate, wl.up, wl.down):
+            if fmt == "bf16":
+                q.w *= 4.0   # outputs well above the bf16 rounding of the short sums
+        _check_layer(dmoe, orc, ws, wl)
+
+
 def test_forward_edge_cases(dmoe, orc, ws):
     wl = workloads.make(1, scale=0.125)
     layer = dmoe.Layer(wl.D, wl.F, wl.K, wl.gate, wl.up, wl.down, swiglu_limit=wl.swiglu_limit, shared=wl.shared)
