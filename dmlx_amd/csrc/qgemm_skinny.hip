@@ -31,6 +31,7 @@ namespace dmoe {
 
 constexpr int kSkinnyWaves = 4;          // 32-row blocks of weight rows per workgroup
 constexpr int kSkinnyStages = 8;
+constexpr int kSkinnySmallStages = 6;    // packed layout, tiles of one row block (see STAGES in skinny_tile)
 constexpr int kSkinnyGroupedStages = 16; // ring depth when the loads are issued four steps at a time
 constexpr int kSkinnyRowBlock = 8;       // tile rows per row block: the LDS window holds 8 whole rows of activations
 
@@ -104,7 +105,13 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
     // no barrier is involved).
     constexpr bool GROUPED = MBLK && RJT == 1;
     constexpr int LG = 4; // steps per 128-byte line = loads per group
-    constexpr int STAGES = GROUPED ? kSkinnyGroupedStages : (RJT == 1 || !FACTORED) ? kSkinnyStages : kSkinnyStages / 2;
+    // The bulk of a decode step - packed weights, tiles of one row block - measured best with SIX stages (ring of 4 / 5 /
+    // 6 / 8 / 10 stages, same box: 64-token step 0.2549 / 0.2525 / 0.2527 / 0.2553 / 0.2652 ms, MXFP4 step 0.1351 / 0.1340
+    // / 0.1335 / 0.1343 / 0.1349 ms; smaller batches alike): what a deeper ring adds in flight it costs before the first step.
+    constexpr int STAGES = GROUPED                           ? kSkinnyGroupedStages
+                           : (PACKED && RJT == 1 && !MBLK)   ? kSkinnySmallStages
+                           : (RJT == 1 || !FACTORED)         ? kSkinnyStages
+                                                             : kSkinnyStages / 2;
     constexpr int PRE = GROUPED ? STAGES : STAGES - 1; // stages requested before the first step is consumed
     constexpr int ROUND = MBLK && STAGES < 8 ? 8 : STAGES;  // steps per unrolled round (MBLK: whole blocks of entries)
     static_assert(ROUND % STAGES == 0 && (!MBLK || ROUND % 8 == 0), "rounds are whole turns of the ring");
