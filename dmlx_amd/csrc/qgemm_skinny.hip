@@ -440,9 +440,12 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
                 load_stage(STAGES + i < n_loc ? STAGES + i : n_loc - LG + i, ring[i], i);
         }
 
-        // whole rounds of the ring run without guards (the look-ahead is clamped onto the last step: a few repeated
-        // loads at the very end instead of a branch per step); a partial last round runs the guarded copy
-        const int full = n_loc / ROUND * ROUND;
+        // Whole rounds of the ring run without guards, the rest in a guarded copy. Tiles of one row block end their
+        // unguarded rounds where the look-ahead would pass the last step (LEAN_TAIL: no chunk is requested twice - the
+        // repeated requests of a look-ahead clamped onto the last step, one per ring stage and wavefront, were a tenth
+        // of a 64-step wavefront's loads); larger tiles need whole rounds per span and clamp instead.
+        constexpr bool LEAN_TAIL = RJT == 1 && !GROUPED;
+        const int full = LEAN_TAIL ? (n_loc > PRE ? (n_loc - PRE) / ROUND * ROUND : 0) : n_loc / ROUND * ROUND;
         int x0 = 0, next_span = span_steps; // first step of the span in LDS, first step of the next one
 #pragma unroll 1
         for (int s0 = 0; s0 < full; s0 += ROUND) {
@@ -475,14 +478,15 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
                     consume(step, j & 7, step - x0, turned);
                     continue;
                 }
-                load_stage(ahead < n_loc ? ahead : n_loc - 1, ring[(j + PRE) % STAGES]);
+                load_stage(LEAN_TAIL || ahead < n_loc ? ahead : n_loc - 1, ring[(j + PRE) % STAGES]);
                 consume(step, j & 7, step - x0, ring[j % STAGES]);
             }
         }
-        if (RJT == 1 && full < n_loc) { // only tiles of one row block get here (larger ones need whole rounds per span)
+#pragma unroll 1
+        for (int t0 = full; RJT == 1 && t0 < n_loc; t0 += ROUND) { // only tiles of one row block get here
 #pragma unroll
             for (int j = 0; j < ROUND; ++j) {
-                const int step = full + j;
+                const int step = t0 + j;
                 if (GROUPED) { // the reduction is a whole number of groups, and everything left is already in the ring
                     if (step < n_loc) {
                         if (j % LG == 0) {
