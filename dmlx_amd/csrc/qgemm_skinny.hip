@@ -81,6 +81,8 @@ __host__ __device__ constexpr size_t skinny_turn_offset(int cols, int kstep) {
            (size_t)(cols / kstep) * kSkinnyRowBlock * sizeof(float) + 128;
 }
 constexpr size_t kSkinnyTurnBytes = (size_t)2 * kSkinnyWaves * 4 * 1024;
+// where a tile's outputs are gathered before they are stored: behind the exchange areas of the epilogue (16 KiB)
+constexpr size_t kSkinnyStageOffset = 16384, kSkinnyStageBytes = (size_t)kSkinnyTileM * 256 * 2;
 
 // MBLK (MLX layout only): the scale / bias entries of a row are not fetched one per step (32 cache lines touched per
 // load for 2 useful bytes each, again at every step: these loads, not the weights, bounded the MLX-layout path) but 16
@@ -541,15 +543,27 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
         }
         const bool storer = store_on && proj == 0 && kh == 0;
         const float swiglu_limit = (t.flags & kTileDense) ? g.swiglu_limit_dense : g.swiglu_limit;
+        // A lane holds ONE column of up to 16 rows: stored from here that is a 2-byte store per row and lane, and a
+        // tile of 32 rows spent 6-7 us of its workgroup's life on them. Instead the values go to LDS (behind the
+        // exchange areas) and leave as 8-byte pieces of a row, one or two per thread. Output rows that cannot be cut
+        // into such pieces keep the direct stores.
+        const bool wide_out = (n_out & 3) == 0 && (g.ldo & 3) == 0 && ((uintptr_t)g.out & 7) == 0;
+        const int cw_shift = (gate_up ? 7 : 8) - (ks ? 1 : 0); // log2 of the workgroup's output columns
+        uint16_t *const stage = (uint16_t *)(skinny_lds + kSkinnyStageOffset); // [tile rows][columns of the workgroup]
+        if (wide_out && !gate_up && !ks) __syncthreads(); // (the other roles have met at a barrier since the main loop)
 #pragma unroll
         for (int j = 0; j < RJT; ++j) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int i = 8 * j + 4 * h + r;
-                if (!storer || i >= nrows) continue;
+                if (proj != 0 || kh != 0 || i >= nrows || (!wide_out && !storer)) continue;
                 const uint32_t p = t.row0 + (uint32_t)i;
                 float val = gate_up ? limited_swiglu(v[0][4 * j + r], v[1][4 * j + r], swiglu_limit) : v[0][4 * j + r];
                 if (g.row_scale && p < g.row_scale_rows) val *= g.row_scale[g.row_scale_idx ? g.row_scale_idx[p] : p];
+                if (wide_out) {
+                    stage[(i << cw_shift) + (gate_up ? wq >> 1 : wq) * 32 + ln] = f32_to_bf16_bits(val);
+                    continue;
+                }
                 const size_t dst = g.out_rows ? g.out_rows[p] : p;
                 // a producer's rows are read by workgroups on other XCDs within the same launch: device-scope
                 // stores (written through this XCD's L2), so no cache-wide write-back is needed before the signal
@@ -557,6 +571,21 @@ __device__ __forceinline__ void skinny_tile(const GemmArgs &g, const Tile &t, ui
                     __hip_atomic_store(&g.out[dst * (size_t)g.ldo + n], f32_to_bf16_bits(val), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 else
                     g.out[dst * (size_t)g.ldo + n] = f32_to_bf16_bits(val);
+            }
+        }
+        if (wide_out) {
+            __syncthreads();
+            const int pp_shift = cw_shift - 2;                     // 4-column pieces per row
+            const int strip0 = (int)blockIdx.x << cw_shift;        // the workgroup's first output column
+            for (int idx = tid; idx < (nrows << pp_shift); idx += WAVES * 64) {
+                const int r = idx >> pp_shift, c = (idx - (r << pp_shift)) * 4;
+                if (strip0 + c >= n_out) continue;                 // a strip that ends past the matrix
+                const uint32_t p = t.row0 + (uint32_t)r;
+                const size_t dst = g.out_rows ? g.out_rows[p] : p;
+                const uint64_t d = *(const uint64_t *)(stage + (r << cw_shift) + c);
+                uint64_t *o = (uint64_t *)(g.out + dst * (size_t)g.ldo + strip0 + c);
+                if (sync == kSkinnySyncSignal) __hip_atomic_store(o, d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                else *o = d;
             }
         }
         if (sync == kSkinnySyncSignal) {
@@ -617,10 +646,10 @@ static int skinny_vals(const QView &b) {
 }
 static size_t skinny_lds_bytes(const QView &b) {
     // a two-row-block tile reads (and ignores) up to 24 floats past its last step's sums: the 128 bytes in the offset.
-    // At least 16 KiB: once the main loop is done the wavefronts exchange their sums through the start of the window
-    // (gate/up pairs: 4 KiB per row block of the tile, up to 16 KiB; split reduction: bytes 4096 .. 8191), which a
-    // short reduction dimension would not cover.
-    return std::max(skinny_turn_offset(b.cols, 2 * skinny_vals(b)), (size_t)16384);
+    // At least 32 KiB: once the main loop is done the wavefronts exchange their sums through the start of the window
+    // (gate/up pairs: 4 KiB per row block of the tile, up to 16 KiB; split reduction: bytes 4096 .. 8191) and gather
+    // the tile's outputs behind that (up to 32 rows of 256 columns), which a short reduction dimension would not cover.
+    return std::max(skinny_turn_offset(b.cols, 2 * skinny_vals(b)), kSkinnyStageOffset + kSkinnyStageBytes);
 }
 
 // Rows per tile to build tile lists with for this weight shape: a tile of 2 (4) row blocks splits the reduction
