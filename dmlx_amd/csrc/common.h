@@ -166,6 +166,21 @@ size_t pack_scratch_bytes(size_t n, int E);
 // stable counting sort of n = T*K expert ids (< E) + tile list with `tile_m` rows per tile (0 = none)
 int launch_pack(const PackOut &o, const uint32_t *d_idx, size_t n, int K, int E, int tile_m,
                 void *d_scratch, hipStream_t st);
+// The gate's selection (dmoe_gate_route) as one argument, for the launch that does selection and packing together
+struct RouteArgs {
+    uint32_t *out_idx = nullptr; // [T, K] router expert ids
+    float *out_w = nullptr;      // [T, K]
+    const float *scores = nullptr, *bias = nullptr;
+    const uint8_t *resident = nullptr;
+    int T = 0, E = 0, K = 0, normalize = 0, apply_scale = 1;
+    float route_scale = 1.0f;
+};
+int launch_route(const RouteArgs &r, hipStream_t st);
+// One or two sequences (T * K <= 16 rows, at most 256 router experts): selection and packing in ONE launch of T
+// wavefronts, one token each; wavefront 0 then packs the rows by itself. Same results as launch_route + launch_pack;
+// `E` = resident expert slots (what the ids are packed by, after o.remap).
+bool route_pack_tiny_supports(const RouteArgs &r);
+int launch_route_pack_tiny(const PackOut &o, const RouteArgs &r, int E, int tile_m, hipStream_t st);
 
 // ---- grouped quantized GEMM ----------------------------------------------------------------------------
 struct QView { // device view of one dmoe_qweight stack

@@ -276,7 +276,7 @@ static int run_gemm(const GemmArgs &g, bool small, hipStream_t st, int small_row
 // routed experts on slot ids: fills ws->y ([T*K, D] bf16 in flat (t,k) order) or `y_out` when given
 static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, const uint16_t *d_x,
                           const uint32_t *d_ids, bool remap, const float *d_scores, int T, uint16_t *y_out,
-                          hipStream_t st) {
+                          hipStream_t st, const RouteArgs *route = nullptr) {
     size_t n = (size_t)T * L->K;
     PackOut po;
     po.order = at<uint32_t>(w, f.order);
@@ -301,7 +301,8 @@ static int routed_forward(const Layer *L, Workspace *w, const FwdLayout &f, cons
         po.remap = L->remap;
         po.n_remap = (uint32_t)L->n_total;
     }
-    DMOE_TRY(launch_pack(po, d_ids, n, L->K, L->E, f.tile_m, at<void>(w, f.scratch), st));
+    if (route) DMOE_TRY(launch_route_pack_tiny(po, *route, L->E, f.tile_m, st)); // the selection has not run yet: one launch for both
+    else DMOE_TRY(launch_pack(po, d_ids, n, L->K, L->E, f.tile_m, at<void>(w, f.scratch), st));
     DMOE_TRY(stage_end(w, DMOE_STAGE_PACK, st));
 
     GemmArgs gu;
@@ -645,9 +646,11 @@ int dmoe_layer_destroy(dmoe_layer layer) {
     return DMOE_OK;
 }
 
+// `route` (optional): the gate's selection has not run yet and is to share a launch with the packing; it fills
+// d_indices and d_scores (= route->out_idx, route->out_w) on the way.
 static int forward_common(uint16_t *d_out, uint16_t *y_out, Layer *L, const uint16_t *d_x, const uint32_t *d_indices,
                           const float *d_scores, int T, bool apply_remap, bool with_shared, dmoe_workspace ws,
-                          dmoe_stream s) {
+                          dmoe_stream s, const RouteArgs *route = nullptr) {
     DMOE_REQUIRE(T >= 0, "forward: T=%d", T);
     if (T == 0) return DMOE_OK;
     DMOE_REQUIRE(d_x && d_indices, "forward: null pointer");
@@ -671,7 +674,7 @@ static int forward_common(uint16_t *d_out, uint16_t *y_out, Layer *L, const uint
         DMOE_TRY(side_stream_ready(w));
         DMOE_HIP(hipEventRecord(w->fork, st));
     }
-    DMOE_TRY(routed_forward(L, w, f, d_x, d_indices, remap, d_scores, T, y_out, st));
+    DMOE_TRY(routed_forward(L, w, f, d_x, d_indices, remap, d_scores, T, y_out, st, route));
     if (side_shared) {
         DMOE_HIP(hipStreamWaitEvent(w->side, w->fork, 0));
         DMOE_TRY(stage_begin(w, DMOE_STAGE_SHARED, w->side));
@@ -728,8 +731,14 @@ int dmoe_moe_layer_forward(uint16_t *d_out, uint32_t *d_out_indices, float *d_ou
     DMOE_TRY(workspace_reserve(ws, b.off, &w));
     uint32_t *idx = d_out_indices ? d_out_indices : at<uint32_t>(w, o_idx);
     float *wts = d_out_weights ? d_out_weights : at<float>(w, o_w);
+    RouteArgs r;
+    r.out_idx = idx, r.out_w = wts, r.scores = d_scores, r.bias = d_bias, r.resident = d_resident_mask;
+    r.T = T, r.E = E_total, r.K = L->K, r.normalize = renorm, r.apply_scale = 1, r.route_scale = route_scale;
+    DMOE_REQUIRE(d_scores != nullptr, "moe_layer_forward: scores is null");
+    // one or two sequences: the selection shares a launch with the packing (and is timed as the packing stage)
+    if (route_pack_tiny_supports(r)) return forward_common(d_out, nullptr, L, d_x, idx, wts, T, true, true, ws, s, &r);
     DMOE_TRY(stage_begin(w, DMOE_STAGE_ROUTE, to_hip(s)));
-    DMOE_TRY(dmoe_gate_route(idx, wts, d_scores, d_bias, d_resident_mask, T, E_total, L->K, renorm, route_scale, s));
+    DMOE_TRY(launch_route(r, to_hip(s)));
     DMOE_TRY(stage_end(w, DMOE_STAGE_ROUTE, to_hip(s)));
     return forward_common(d_out, nullptr, L, d_x, idx, wts, T, true, true, ws, s);
 }

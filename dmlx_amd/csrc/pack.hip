@@ -9,6 +9,7 @@
 //
 // Up to 1024 rows everything runs in ONE launch (16 wavefronts x 64 rows); above that in three.
 #include "common.h"
+#include "route_device.h"
 
 namespace dmoe {
 
@@ -195,6 +196,137 @@ __global__ __launch_bounds__(kPackThreads) void pack_fused_kernel(PackOut o, con
     pack_fused_body(o, e, active, n, K, E, tile_m, pack_sm, scan_sm);
 }
 
+// ---- one wavefront, n <= 64 ---------------------------------------------------------------------------------
+// A decode step of a few sequences: lane i = row i, every other row's id comes over with v_readlane, and nothing needs
+// LDS, a barrier or a histogram. Same outputs. The loops over the other rows are serial, so this only pays for one or
+// two sequences (6 rows: 6.7 us against 7.2 us for the 1024-thread kernel, 48 rows: 16.9 against 7.5 us).
+constexpr uint32_t kPackWaveRows = 16;
+__device__ __forceinline__ uint32_t lane_value(uint32_t v, uint32_t j) { return (uint32_t)__builtin_amdgcn_readlane((int)v, (int)j); }
+
+__device__ __forceinline__ void pack_wave_body(const PackOut &o, uint32_t e, bool active, uint32_t n, int K, int E,
+                                               int tile_m, int lane) {
+    if (active && e >= (uint32_t)E) { // a corrupt id: stay in bounds, and tell the host
+        if (o.bad_ids) atomicAdd(o.bad_ids, 1u);
+        e = (uint32_t)E - 1;
+    }
+    const uint32_t key = active ? e : 0xffffffffu;
+    // rows of smaller experts, earlier rows of this expert, rows of this expert
+    uint32_t below = 0, before = 0, same = 0;
+    for (uint32_t j = 0; j < n; ++j) {
+        const uint32_t ej = lane_value(key, j);
+        below += ej < key ? 1u : 0u;
+        same += ej == key ? 1u : 0u;
+        before += (ej == key && j < (uint32_t)lane) ? 1u : 0u;
+    }
+    if (active) place_row(o, below + before, (uint32_t)lane, e, K);
+    // the first row of an expert speaks for it: its tiles, its place among the live experts
+    const bool first = active && before == 0;
+    const uint32_t tm = tile_m > 0 ? (uint32_t)tile_m : 1u;
+    const uint32_t nt = (tile_m > 0 && first) ? (same + tm - 1) / tm : 0u;
+    const uint32_t last_rows = same - (nt ? (nt - 1) * tm : 0);
+    const uint32_t n_big = nt == 0 ? 0 : (nt - 1) + (last_rows > kPackSmallTileRows ? 1u : 0u);
+    const uint32_t n_small = nt - n_big;
+    const uint64_t firsts = __ballot(first);
+    uint32_t live_rank = 0, live_tot = 0, big_ex = 0, small_ex = 0, big_tot = 0, small_tot = 0;
+    for (uint32_t j = 0; j < n; ++j) {
+        if (!((firsts >> j) & 1ull)) continue; // uniform
+        const uint32_t ej = lane_value(key, j), bj = lane_value(n_big, j), sj = lane_value(n_small, j);
+        const bool lt = ej < key;
+        live_rank += lt ? 1u : 0u;
+        big_ex += lt ? bj : 0u;
+        small_ex += lt ? sj : 0u;
+        live_tot += 1u, big_tot += bj, small_tot += sj;
+    }
+    // rows per expert and where they start, for every expert of the layer
+    for (uint32_t x = (uint32_t)lane; x < (uint32_t)E; x += 64) {
+        uint32_t c = 0, lo = 0;
+        for (uint32_t j = 0; j < n; ++j) {
+            const uint32_t ej = lane_value(key, j);
+            c += ej == x ? 1u : 0u;
+            lo += ej < x ? 1u : 0u;
+        }
+        if (o.counts) o.counts[x] = c;
+        if (o.offsets) o.offsets[x] = lo;
+    }
+    if (lane == 0 && o.offsets) o.offsets[E] = n;
+    if (first && o.live) o.live[live_rank] = e;
+    if (lane == 0 && o.n_live) *o.n_live = live_tot;
+    for (uint32_t i = (uint32_t)lane; i < o.n_done; i += 64) o.tile_done[i] = 0;
+    // the folded always-on expert: identity rows behind the routed ones, its tiles ahead of the routed tiles
+    const uint32_t nt_dense = (o.dense_rows + tm - 1) / tm;
+    for (uint32_t i = (uint32_t)lane; i < o.dense_rows; i += 64) {
+        o.order[n + i] = n + i;
+        if (o.token) o.token[n + i] = i;
+        if (o.sorted_e) o.sorted_e[n + i] = o.dense_expert;
+    }
+    if (tile_m > 0 && o.tiles) {
+        for (uint32_t j = (uint32_t)lane; j < nt_dense; j += 64) {
+            Tile t;
+            t.expert = o.dense_expert;
+            t.row0 = n + j * tm;
+            const uint32_t left = o.dense_rows - j * tm;
+            t.nrows = left < tm ? left : tm;
+            t.flags = kTileDense;
+            o.tiles[j] = t;
+        }
+        for (uint32_t j = 0; j < nt; ++j) { // nt = 0 on every lane but an expert's first
+            Tile t;
+            t.expert = e;
+            t.row0 = below + j * tm;
+            const uint32_t left = same - j * tm;
+            t.nrows = left < tm ? left : tm;
+            t.flags = 0;
+            o.tiles[nt_dense + (j < n_big ? big_ex + j : big_tot + small_ex)] = t;
+        }
+        if (lane == 0 && o.n_tiles) *o.n_tiles = nt_dense + big_tot + small_tot;
+    }
+}
+
+__global__ __launch_bounds__(64) void pack_wave_kernel(PackOut o, const uint32_t *__restrict__ idx, uint32_t n, int K,
+                                                       int E, int tile_m) {
+    const int lane = lane_id();
+    const bool active = (uint32_t)lane < n;
+    const uint32_t e = active ? packed_id(o, idx[lane]) : 0u;
+    pack_wave_body(o, e, active, n, K, E, tile_m, lane);
+}
+
+// selection and packing of one or two sequences in one launch: wavefront t routes token t, wavefront 0 packs
+__global__ __launch_bounds__(kPackWaveRows * 64) void route_pack_tiny_kernel(PackOut o, RouteArgs r, int E, int tile_m) {
+    __shared__ uint32_t ids[kPackWaveRows];
+    const int lane = lane_id(), t = (int)(threadIdx.x >> 6);
+    {
+        const float *const rows[1] = {r.scores + (size_t)t * r.E};
+        uint32_t my_idx[1];
+        float w[1];
+        route_tokens<1, 4>(rows, r.bias, r.resident, r.E, r.K, r.normalize, r.apply_scale, r.route_scale, lane, my_idx, w);
+        if (lane < r.K) {
+            const size_t at = (size_t)t * r.K + lane;
+            r.out_idx[at] = my_idx[0];
+            r.out_w[at] = w[0];
+            ids[at] = my_idx[0];
+        }
+    }
+    __syncthreads();
+    if (t != 0) return;
+    const uint32_t n = (uint32_t)(r.T * r.K);
+    const bool active = (uint32_t)lane < n;
+    const uint32_t e = active ? packed_id(o, ids[lane]) : 0u;
+    pack_wave_body(o, e, active, n, r.K, E, tile_m, lane);
+}
+
+bool route_pack_tiny_supports(const RouteArgs &r) {
+    return r.T >= 1 && r.K >= 1 && (size_t)r.T * (size_t)r.K <= (size_t)kPackWaveRows && r.E >= r.K && r.E <= 256;
+}
+
+int launch_route_pack_tiny(const PackOut &o, const RouteArgs &r, int E, int tile_m, hipStream_t st) {
+    DMOE_REQUIRE(route_pack_tiny_supports(r), "route + pack: T=%d K=%d E=%d is not a batch of one or two sequences", r.T, r.K, r.E);
+    DMOE_REQUIRE(E >= 1 && E <= kPackThreads, "pack: E=%d out of range [1,%d]", E, kPackThreads);
+    DMOE_REQUIRE(r.out_idx && r.out_w && r.scores && o.order, "route + pack: null pointer");
+    hipLaunchKernelGGL(route_pack_tiny_kernel, dim3(1), dim3((unsigned)r.T * 64), 0, st, o, r, E, tile_m);
+    DMOE_LAUNCH_CHECK();
+    return DMOE_OK;
+}
+
 // ---- three launches, any n --------------------------------------------------------------------------------
 __global__ __launch_bounds__(kScatterWaves * 64) void pack_hist_kernel(PackOut o, uint32_t *__restrict__ cnt,
                                                                        const uint32_t *__restrict__ idx,
@@ -290,8 +422,12 @@ int launch_pack(const PackOut &o, const uint32_t *d_idx, size_t n, int K, int E,
     DMOE_REQUIRE(K >= 1, "pack: K=%d", K);
     DMOE_REQUIRE(n < (1ull << 31), "pack: too many rows");
     DMOE_REQUIRE(n == 0 || (o.order != nullptr && d_idx != nullptr), "pack: null pointer");
+    if (n <= (size_t)kPackWaveRows) { // also covers n == 0: counts / offsets / n_tiles / n_live are still written (all zero)
+        hipLaunchKernelGGL(pack_wave_kernel, dim3(1), dim3(64), 0, st, o, d_idx, (uint32_t)n, K, E, tile_m);
+        DMOE_LAUNCH_CHECK();
+        return DMOE_OK;
+    }
     if (n <= (size_t)kPackThreads) {
-        // also covers n == 0: counts/offsets/n_tiles/n_live are still written (all zero)
         size_t lds = sizeof(uint32_t) * (size_t)kPackWaves * E;
         hipLaunchKernelGGL(pack_fused_kernel, dim3(1), dim3(kPackThreads), lds, st, o, d_idx, (uint32_t)n, K, E,
                            tile_m);

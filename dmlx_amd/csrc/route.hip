@@ -47,6 +47,11 @@ static int launch_route(uint32_t *out_idx, float *out_w, const float *scores, co
     return DMOE_OK;
 }
 
+int launch_route(const RouteArgs &r, hipStream_t st) {
+    return launch_route(r.out_idx, r.out_w, r.scores, r.bias, r.resident, r.T, r.E, r.K, r.normalize, r.apply_scale,
+                        r.route_scale, st);
+}
+
 __global__ void remap_kernel(uint32_t *__restrict__ out, const int32_t *__restrict__ remap,
                              const uint32_t *__restrict__ idx, size_t n, uint32_t n_total) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;

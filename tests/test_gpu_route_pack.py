@@ -140,6 +140,10 @@ def test_gate_route_bit_exact(dmoe, orc, T, E, K, masked):
 
 
 @pytest.mark.parametrize("T,K,E", [(0, 6, 8), (1, 1, 4), (16, 2, 8), (64, 6, 256), (64, 6, 51), (170, 6, 256),
+                                   # up to 16 rows: the single-wavefront kernel (one sequence, 16 rows exactly, 1024
+                                   # experts, nearly every row on the same few experts); and sizes just above it
+                                   (1, 6, 256), (2, 8, 1024), (16, 1, 16), (5, 3, 3), (3, 5, 40), (2, 6, 256),
+                                   (10, 6, 256), (64, 1, 16), (8, 8, 1024), (9, 7, 3), (17, 1, 40),
                                    (171, 6, 256), (2080, 6, 256), (8192, 6, 256), (5000, 3, 1000), (300, 1, 1)])
 def test_pack_bit_exact(dmoe, orc, ws, T, K, E):
     rng = np.random.default_rng(T * 7 + K + E)
