@@ -502,6 +502,17 @@ struct DSV4MoE {
         Array y = stream_provider->forward(ctx, layer_idx, flat, routed.second, routed.first);
         return y.reshaped({B, S, D});
     }
+    // DSV4MoE.forward(hidden_states, input_ids, stream) as the reference declares it (deepseek_v4.zig:1010-1056): the
+    // gate runs from the hidden states (router weight uploaded with gate.load), input_ids only matter on hash layers
+    Array forward(const Context &ctx, const Array &hidden_states, const Array *input_ids = nullptr) const {
+        const auto &sh = hidden_states.shape();
+        const int B = sh.at(0), S = sh.at(1), D = sh.at(2);
+        Array flat = hidden_states.reshaped({B * S, D});
+        auto routed = gate.forwardHidden(ctx, flat, input_ids);
+        if (!stream_provider) throw Error(DMOE_ERR_INVALID, "PreloadProviderNotInitialized");
+        Array y = stream_provider->forward(ctx, layer_idx, flat, routed.second, routed.first);
+        return y.reshaped({B, S, D});
+    }
 };
 
 // ---- batch_builder.zig ----------------------------------------------------------------------------------------

@@ -228,6 +228,21 @@ static void test_layer_closed_form(const Context &ctx) {
         const double want = 1.5 * bdr * F * h; // renormalised weights sum to 1, times route_scale
         for (int d = 0; d < D; d += 37) NEAR(from_bf16(y[(size_t)t * D + d]), want, std::fabs(want) * 2e-2 + 1e-6);
     }
+    // DSV4MoE.forward(hidden_states) as the reference declares it: the gate runs from the hidden states. Both experts
+    // are selected whatever the logits are (K = E), the renormalised weights sum to one, every expert gives the same
+    // output: the closed form above again
+    {
+        std::vector<uint16_t> wg((size_t)E * D);
+        for (int e = 0; e < E; ++e)
+            for (int d = 0; d < D; ++d) wg[(size_t)e * D + d] = bf16(0.01f * (float)((e * 5 + d) % 7 - 3));
+        moe.gate.load(ctx, wg.data(), D);
+        auto yh = moe.forward(ctx, hidden).dataSlice<uint16_t>();
+        for (int t = 0; t < T; ++t) {
+            const double g = bgr * sumx[t], h = g / (1.0 + std::exp(-g)) * g;
+            const double want = 1.5 * bdr * F * h;
+            for (int d = 0; d < D; d += 37) NEAR(from_bf16(yh[(size_t)t * D + d]), want, std::fabs(want) * 2e-2 + 1e-6);
+        }
+    }
     // the same step as one call from the scores on (a second handle on the same weights): the same bytes
     DSV4SwitchGLU direct(ctx, D, F, K, gate, up, down, opt);
     Array y2 = direct.forwardFromScores(ctx, hidden.reshaped({T, D}), Array::fromData(ctx, scores.data(), {T, E}, DType::float32),
